@@ -1,0 +1,190 @@
+// extern "C" entry points: argument validation (no HIP call before it passes) and dispatch to
+// the launchers in the kernel translation units.
+#include "common.h"
+
+int launch_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, hipStream_t st);
+int launch_gptq_permute_rows(const int32_t* qweight, const int32_t* perm, int K, int N, int32_t* out, hipStream_t st);
+int launch_permute_cols(const void* in, int64_t ld_in, const int32_t* perm, int M, int C, int gather, void* out,
+                        int64_t ld_out, hipStream_t st);
+int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out,
+                     hipStream_t st);
+int lora_grad_splits(int M, int C);
+int launch_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
+                     int act_dtype, int out_dtype, void* out, void* workspace, hipStream_t st);
+int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,
+                         int64_t ldh, int act_dtype, hipStream_t st);
+int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx, void* e,
+                            void* g, void* h_out, int64_t ldeg, int act_dtype, hipStream_t st);
+
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool is_act(int d) { return d == FMSA_BF16 || d == FMSA_F16; }
+
+int check_weight(const fmsa_gptq_weight* w, int group_multiple) {
+  if (!w->qweight || !w->scales || !w->qzeros) return FMSA_ERR_NULL;
+  if (w->K <= 0 || w->N <= 0 || w->group_size <= 0) return FMSA_ERR_SHAPE;
+  if (w->K % 32 != 0 || w->N % 32 != 0) return FMSA_ERR_SHAPE;  // qlinear_tritonv2.py:57-60
+  if (w->zero_offset != 0 && w->zero_offset != 1) return FMSA_ERR_SHAPE;
+  if (!aligned16(w->qweight) || !aligned16(w->scales) || !aligned16(w->qzeros)) return FMSA_ERR_ALIGN;
+  if (group_multiple > 0) {
+    // The fused kernels assume the group of row k is k / group_size: act-order weights must be
+    // repacked with fmsa_gptq_permute_rows first.  The forward reads scale/zero once per 64-wide
+    // K stage (group_size % 64 == 0); the input-gradient kernel needs one group per packed
+    // qweight row (group_size % 8 == 0).
+    if (w->g_idx) return FMSA_ERR_UNSUPPORTED;
+    if (w->group_size % group_multiple != 0) return FMSA_ERR_UNSUPPORTED;
+  }
+  return FMSA_OK;
+}
+
+int check_rank(int r) {
+  if (r < 0) return FMSA_ERR_SHAPE;
+  if (r % 8 != 0 || r > 128) return FMSA_ERR_UNSUPPORTED;
+  return FMSA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* fmsa_strerror(int code) {
+  switch (code) {
+    case FMSA_OK: return "ok";
+    case FMSA_ERR_NULL: return "a required pointer is NULL";
+    case FMSA_ERR_SHAPE: return "invalid dimension";
+    case FMSA_ERR_ALIGN: return "pointer or leading dimension is not 16-byte aligned";
+    case FMSA_ERR_DTYPE: return "unknown dtype";
+    case FMSA_ERR_UNSUPPORTED: return "configuration not covered by the gfx950 kernels";
+    case FMSA_ERR_WORKSPACE: return "workspace missing or too small";
+    case FMSA_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown error";
+  }
+}
+
+int fmsa_abi_version(void) { return 1; }
+
+int fmsa_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, void* stream) {
+  if (!w || !out) return FMSA_ERR_NULL;
+  if (int rc = check_weight(w, 0)) return rc;
+  if (out_dtype != FMSA_F16 && out_dtype != FMSA_BF16 && out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
+  if (!aligned16(out)) return FMSA_ERR_ALIGN;
+  return launch_gptq_dequant(w, out_dtype, out, (hipStream_t)stream);
+}
+
+int fmsa_gptq_permute_rows(const int32_t* qweight, const int32_t* perm, int K, int N, int32_t* qweight_out,
+                           void* stream) {
+  if (!qweight || !perm || !qweight_out) return FMSA_ERR_NULL;
+  if (K <= 0 || N <= 0 || K % 8 != 0) return FMSA_ERR_SHAPE;
+  if (qweight == qweight_out) return FMSA_ERR_UNSUPPORTED;  // not an in-place operation
+  return launch_gptq_permute_rows(qweight, perm, K, N, qweight_out, (hipStream_t)stream);
+}
+
+int fmsa_permute_cols(const void* in, int64_t ld_in, const int32_t* perm, int M, int C, int gather, int act_dtype,
+                      void* out, int64_t ld_out, void* stream) {
+  if (!in || !perm || !out) return FMSA_ERR_NULL;
+  if (M <= 0 || C <= 0 || ld_in < C || ld_out < C) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  if (in == out) return FMSA_ERR_UNSUPPORTED;
+  return launch_permute_cols(in, ld_in, perm, M, C, gather, out, ld_out, (hipStream_t)stream);
+}
+
+int fmsa_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out,
+                   void* stream) {
+  if (!X || !Wd || !out) return FMSA_ERR_NULL;
+  if (M <= 0 || C <= 0 || r <= 0 || ldx < C) return FMSA_ERR_SHAPE;
+  if (int rc = check_rank(r)) return rc;
+  if (C % 8 != 0) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  if (!aligned16(X) || !aligned16(Wd) || ldx % 8 != 0) return FMSA_ERR_ALIGN;
+  return launch_lora_down(X, ldx, Wd, M, C, r, act_dtype, out, (hipStream_t)stream);
+}
+
+size_t fmsa_lora_grad_workspace(int M, int C, int r) {
+  if (M <= 0 || C <= 0 || r <= 0) return 0;
+  return (size_t)lora_grad_splits(M, C) * (size_t)r * (size_t)C * sizeof(float);
+}
+
+int fmsa_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
+                   int act_dtype, int out_dtype, void* out, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!L || !R || !out) return FMSA_ERR_NULL;
+  if (M <= 0 || C <= 0 || r <= 0 || ldr < C) return FMSA_ERR_SHAPE;
+  if (C % 2 != 0 || ldr % 2 != 0) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  if (out_dtype != FMSA_F16 && out_dtype != FMSA_BF16 && out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
+  if (!workspace || workspace_bytes < fmsa_lora_grad_workspace(M, C, r)) return FMSA_ERR_WORKSPACE;
+  if ((reinterpret_cast<uintptr_t>(R) & 3u) || (reinterpret_cast<uintptr_t>(workspace) & 7u)) return FMSA_ERR_ALIGN;
+  return launch_lora_grad(L, R, ldr, M, C, r, scale, transpose_out, act_dtype, out_dtype, out, workspace,
+                          (hipStream_t)stream);
+}
+
+int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,
+                       int64_t ldh, int act_dtype, void* stream) {
+  if (!projs || !X) return FMSA_ERR_NULL;
+  if (n_proj < 1 || n_proj > 3 || M <= 0) return FMSA_ERR_SHAPE;
+  if (mode != FMSA_FWD_LINEAR && mode != FMSA_FWD_SWIGLU) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  const int K = projs[0].w.K;
+  if (ldx < K) return FMSA_ERR_SHAPE;
+  if (!aligned16(X) || ldx % 8 != 0) return FMSA_ERR_ALIGN;
+  for (int p = 0; p < n_proj; ++p) {
+    const fmsa_fwd_proj& s = projs[p];
+    if (int rc = check_weight(&s.w, 64)) return rc;
+    if (s.w.K != K) return FMSA_ERR_SHAPE;
+    if (!s.Y) return FMSA_ERR_NULL;
+    if (s.ldy < s.w.N) return FMSA_ERR_SHAPE;
+    if (!aligned16(s.Y) || s.ldy % 8 != 0) return FMSA_ERR_ALIGN;
+    if (int rc = check_rank(s.r)) return rc;
+    if (s.r > 0) {
+      if (!s.U || !s.B) return FMSA_ERR_NULL;
+      if (!aligned16(s.U) || !aligned16(s.B)) return FMSA_ERR_ALIGN;
+    }
+    if (s.bias && !aligned16(s.bias)) return FMSA_ERR_ALIGN;
+  }
+  if (mode == FMSA_FWD_SWIGLU) {
+    if (n_proj != 2 || projs[0].w.N != projs[1].w.N) return FMSA_ERR_SHAPE;
+    if (!H) return FMSA_ERR_NULL;
+    if (ldh < projs[0].w.N) return FMSA_ERR_SHAPE;
+    if (!aligned16(H) || ldh % 8 != 0) return FMSA_ERR_ALIGN;
+  }
+  return launch_gptq_lora_fwd(projs, n_proj, X, ldx, M, mode, H, ldh, act_dtype, (hipStream_t)stream);
+}
+
+int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx, void* e,
+                          void* g, void* h_out, int64_t ldeg, int act_dtype, void* stream) {
+  if (!projs) return FMSA_ERR_NULL;
+  if (n_proj < 1 || n_proj > 3 || M <= 0) return FMSA_ERR_SHAPE;
+  if (mode != FMSA_BWD_LINEAR && mode != FMSA_BWD_SWIGLU) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  const int K = projs[0].w.K;
+  for (int p = 0; p < n_proj; ++p) {
+    const fmsa_bwd_proj& s = projs[p];
+    if (int rc = check_weight(&s.w, 8)) return rc;
+    if (s.w.K != K) return FMSA_ERR_SHAPE;
+    if (!s.dY) return FMSA_ERR_NULL;
+    if (s.lddy < s.w.N) return FMSA_ERR_SHAPE;
+    if (!aligned16(s.dY) || s.lddy % 8 != 0) return FMSA_ERR_ALIGN;
+    if (int rc = check_rank(s.r)) return rc;
+    if (s.r > 0) {
+      if (!s.T || !s.At) return FMSA_ERR_NULL;
+      if (!aligned16(s.T) || !aligned16(s.At)) return FMSA_ERR_ALIGN;
+    }
+    if (s.mask_src) {
+      if (s.ldmask < K) return FMSA_ERR_SHAPE;
+      if ((reinterpret_cast<uintptr_t>(s.mask_src) & 3u) || s.ldmask % 2 != 0) return FMSA_ERR_ALIGN;
+    }
+  }
+  if (mode == FMSA_BWD_SWIGLU) {
+    if (n_proj != 1) return FMSA_ERR_SHAPE;
+    if (!e || !g || !h_out) return FMSA_ERR_NULL;
+    if (ldeg < K) return FMSA_ERR_SHAPE;
+    if (!aligned16(e) || !aligned16(g) || !aligned16(h_out) || ldeg % 8 != 0) return FMSA_ERR_ALIGN;
+  } else {
+    if (!dX) return FMSA_ERR_NULL;
+    if (lddx < K) return FMSA_ERR_SHAPE;
+    if (!aligned16(dX) || lddx % 8 != 0) return FMSA_ERR_ALIGN;
+  }
+  return launch_gptq_lora_bwd_dx(projs, n_proj, M, mode, dX, lddx, e, g, h_out, ldeg, act_dtype, (hipStream_t)stream);
+}
+
+}  // extern "C"

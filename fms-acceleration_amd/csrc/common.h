@@ -1,0 +1,120 @@
+// Shared device helpers for the gfx950 kernels: vector types, MFMA wrappers, the GPTQ nibble
+// unpack and the storage-type conversions.  Everything here is wave64 / CDNA4 specific.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "../../include/fmsa.h"
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define FMSA_DEVI __device__ __forceinline__
+
+// Compile-time loop: the body receives std::integral_constant<int, I>, so register arrays indexed
+// by the loop variable can never fall back to dynamic (scratch-memory) indexing.
+template <int I, int N, typename F> FMSA_DEVI void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+// ---- scalar conversions with a single round-to-nearest-even --------------------------------
+FMSA_DEVI float fp16_bits_to_f32(uint16_t h) {
+  union { uint16_t u; f16_t f; } c;
+  c.u = h;
+  return (float)c.f;
+}
+FMSA_DEVI float bf16_bits_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+
+// Two fp32 -> packed storage type, RNE, low half = a.
+template <typename T> FMSA_DEVI uint32_t pack2(float a, float b);
+template <> FMSA_DEVI uint32_t pack2<bf16_t>(float a, float b) {
+  uint32_t r;
+  asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+template <> FMSA_DEVI uint32_t pack2<f16_t>(float a, float b) {
+  union { f16_t h[2]; uint32_t u; } c;
+  c.h[0] = (f16_t)a;  // v_cvt_f16_f32 is RNE under the default mode
+  c.h[1] = (f16_t)b;
+  return c.u;
+}
+template <typename T> FMSA_DEVI uint16_t pack1(float a) { return (uint16_t)(pack2<T>(a, 0.f) & 0xffffu); }
+
+template <typename T> FMSA_DEVI float unpack_lo(uint32_t v);
+template <typename T> FMSA_DEVI float unpack_hi(uint32_t v);
+template <> FMSA_DEVI float unpack_lo<bf16_t>(uint32_t v) { return __uint_as_float(v << 16); }
+template <> FMSA_DEVI float unpack_hi<bf16_t>(uint32_t v) { return __uint_as_float(v & 0xffff0000u); }
+template <> FMSA_DEVI float unpack_lo<f16_t>(uint32_t v) { return fp16_bits_to_f32((uint16_t)(v & 0xffffu)); }
+template <> FMSA_DEVI float unpack_hi<f16_t>(uint32_t v) { return fp16_bits_to_f32((uint16_t)(v >> 16)); }
+template <typename T> FMSA_DEVI float unpack1(uint16_t v) { return unpack_lo<T>((uint32_t)v); }
+
+// byte j of x as fp32 (one VALU op each)
+FMSA_DEVI float ubyte0(uint32_t x) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(x)); return r; }
+FMSA_DEVI float ubyte1(uint32_t x) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(x)); return r; }
+FMSA_DEVI float ubyte2(uint32_t x) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(x)); return r; }
+FMSA_DEVI float ubyte3(uint32_t x) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(x)); return r; }
+
+// ---- GPTQ: eight nibbles of one int32 -> eight storage-type values --------------------------
+// value_j = RNE( sf * nib_j + nsz ) with nsz = -sf * (z + zero_offset).  sf is an fp16 scale
+// widened to fp32 (11 significant bits) and nib, z are < 32, so sf*nib, nsz and their sum are
+// all exact in fp32: the only rounding is the final conversion, as in
+// UL/gptq/triton/kernels.py:118-122.
+template <typename T> FMSA_DEVI u32x4 dequant8(uint32_t w, float sf, float nsz) {
+  const uint32_t lo = w & 0x0F0F0F0Fu;         // nibbles 0,2,4,6 in bytes 0..3
+  const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;  // nibbles 1,3,5,7
+  u32x4 r;
+  r[0] = pack2<T>(__builtin_fmaf(sf, ubyte0(lo), nsz), __builtin_fmaf(sf, ubyte0(hi), nsz));
+  r[1] = pack2<T>(__builtin_fmaf(sf, ubyte1(lo), nsz), __builtin_fmaf(sf, ubyte1(hi), nsz));
+  r[2] = pack2<T>(__builtin_fmaf(sf, ubyte2(lo), nsz), __builtin_fmaf(sf, ubyte2(hi), nsz));
+  r[3] = pack2<T>(__builtin_fmaf(sf, ubyte3(lo), nsz), __builtin_fmaf(sf, ubyte3(hi), nsz));
+  return r;
+}
+
+// ---- MFMA 32x32x16: D[i][j] += sum_k A[i][k] * B[k][j] ---------------------------------------
+// Operand fragments are 8 consecutive contraction elements per lane: lane l supplies row
+// (l & 31) of A / column (l & 31) of B at k = 8*(l >> 5) .. +7.  The accumulator register
+// 4*i0 + i1 of lane l is D[8*i0 + 4*(l >> 5) + i1][l & 31].
+template <typename T> FMSA_DEVI f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c);
+template <> FMSA_DEVI f32x16 mfma32<bf16_t>(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+template <> FMSA_DEVI f32x16 mfma32<f16_t>(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+// MFMA 16x16x32: lane l supplies row/column (l & 15) at k = 8*(l >> 4) .. +7; accumulator
+// register i of lane l is D[4*(l >> 4) + i][l & 15].
+template <typename T> FMSA_DEVI f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c);
+template <> FMSA_DEVI f32x4 mfma16<bf16_t>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+template <> FMSA_DEVI f32x4 mfma16<f16_t>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// ---- workgroup-id remap: consecutive ids land on different XCDs (id % 8), each with its own
+// L2.  Give every XCD a contiguous range of logical tiles so neighbours share operands in L2.
+FMSA_DEVI int xcd_remap(int pid, int total) {
+  const int NXCD = 8;
+  if (total % NXCD != 0) return pid;
+  return (pid % NXCD) * (total / NXCD) + pid / NXCD;
+}
+
+// SiLU pieces with the reference's rounding points (UL/swiglu.py:26-33, 65-83).
+FMSA_DEVI float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+// Host-side launch helpers (api.hip)
+#define FMSA_CHECK_LAUNCH()                                   \
+  do {                                                        \
+    if (hipGetLastError() != hipSuccess) return FMSA_ERR_LAUNCH; \
+  } while (0)

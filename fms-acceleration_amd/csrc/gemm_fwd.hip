@@ -1,0 +1,326 @@
+// Fused forward:  Y = X * deq(W) + s * U * B^T (+ bias), optional SwiGLU over a gate/up pair.
+//
+// Tiling (one workgroup = 4 waves = 256 lanes, one workgroup per CU):
+//   workgroup tile  256 tokens x 256 output columns, K walked in stages of 64
+//   wave tile       256 tokens x 64 columns = 8 x 2 MFMA 32x32x16 tiles, 256 fp32 accumulators
+//   X operand       global -> registers -> LDS (row stride 72 elements = 144 B, conflict-free for
+//                   16-byte fragment reads), double buffered, one barrier per stage
+//   W operand       never touches LDS: one packed int32 (8 nibbles along K at one column) is
+//                   exactly the 8-element MFMA fragment of the lane that owns that column, so each
+//                   lane loads its own words (a wave reads 2 x 128 B contiguous per load), unpacks
+//                   them in registers and feeds the MFMA directly.  Each wave owns distinct
+//                   columns, so no weight is unpacked twice inside a workgroup.
+// The MFMA is issued as D^T = W^T-fragment x X-fragment: a lane then holds 4 consecutive output
+// columns per accumulator quad, which turns the epilogue stores into 8-byte vectors.
+// The rank-r LoRA term is one extra MFMA step per 16 ranks in the epilogue, scaled by s in fp32
+// before the single rounding of the output.
+#include "common.h"
+
+namespace {
+
+constexpr int BM = 256;
+constexpr int BK = 64;
+constexpr int LDS_STRIDE = BK + 8;  // elements
+constexpr int MT = 8;
+constexpr int NT = 2;
+
+struct FwdProjDev {
+  const int32_t* qweight;
+  const uint16_t* scales;
+  const int32_t* qzeros;
+  const uint16_t* U;
+  const uint16_t* B;
+  const uint16_t* bias;
+  uint16_t* Y;
+  int64_t ldy;
+  int N, group_size, zero_offset, r;
+  float s;
+};
+
+struct FwdArgs {
+  FwdProjDev p[3];
+  int nblk_start[4];
+  const uint16_t* X;
+  int64_t ldx;
+  int M, K, mode, nbm, nbn;
+  uint16_t* H;
+  int64_t ldh;
+};
+
+// a.p[p] for a runtime (wave-uniform) p without dynamic indexing of the kernel-argument struct,
+// which would force a copy of it into scratch memory.
+FMSA_DEVI FwdProjDev select_proj(const FwdArgs& a, int p) { return p == 0 ? a.p[0] : (p == 1 ? a.p[1] : a.p[2]); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t lds[2][BM * LDS_STRIDE];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int l32 = lane & 31;
+  const int half = lane >> 5;
+
+  // ---- tile assignment: XCD-contiguous ranges, then grouped-M order inside the range --------
+  int pid = xcd_remap(blockIdx.x, a.nbm * a.nbn);
+  constexpr int GROUP_M = 8;
+  const int width = GROUP_M * a.nbn;
+  const int first_m = (pid / width) * GROUP_M;
+  const int gsz = min(a.nbm - first_m, GROUP_M);
+  const int bm = first_m + (pid % width) % gsz;
+  const int bn = (pid % width) / gsz;
+  const int m0 = bm * BM;
+
+  int pj[NT], col0[NT];
+  bool active[NT];
+  if (a.mode == FMSA_FWD_SWIGLU) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      pj[j] = j;
+      col0[j] = bn * 128 + wave * 32;
+    }
+  } else {
+    int p = 0;
+    if (bn >= a.nblk_start[1]) p = 1;
+    if (bn >= a.nblk_start[2]) p = 2;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      pj[j] = p;
+      col0[j] = (bn - a.nblk_start[p]) * 256 + wave * 64 + j * 32;
+    }
+  }
+  const int32_t* qwp[NT];
+  const uint16_t* scp[NT];
+  const int32_t* zp[NT];
+  int Np[NT], zshift[NT], gs[NT];
+  float zoff[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const FwdProjDev P = select_proj(a, pj[j]);
+    active[j] = col0[j] < P.N;
+    if (!active[j]) col0[j] = 0;
+    const int col = col0[j] + l32;
+    Np[j] = P.N;
+    gs[j] = P.group_size;
+    qwp[j] = P.qweight + col;
+    scp[j] = P.scales + col;
+    zp[j] = P.qzeros + (col >> 3);
+    zshift[j] = 4 * (col & 7);
+    zoff[j] = (float)P.zero_offset;
+  }
+
+  const int K = a.K;
+  const int n_stages = (K + BK - 1) / BK;
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
+
+  u32x4 a_st[8];        // X staging: 8 x 16 B per lane per stage
+  uint32_t q_cur[NT][4], q_nxt[NT][4];
+  float sf[NT], nsz[NT];
+  int g_cur[NT];
+  uint16_t sc_nxt[NT];
+  uint32_t zw_nxt[NT];
+  bool g_changed[NT];
+
+  auto load_stage = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c >> 3, oct = c & 7;
+      const int gm = m0 + row, gk = k0 + 8 * oct;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (gm < a.M && gk < K) v = *reinterpret_cast<const u32x4*>(a.X + (size_t)gm * a.ldx + gk);
+      a_st[i] = v;
+    }
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int k8 = (k0 >> 3) + 2 * t + half;
+        q_nxt[j][t] = (8 * k8 < K) ? (uint32_t)qwp[j][(size_t)k8 * Np[j]] : 0u;
+      }
+      const int g = k0 / gs[j];
+      g_changed[j] = (g != g_cur[j]);
+      if (g_changed[j]) {
+        sc_nxt[j] = scp[j][(size_t)g * Np[j]];
+        zw_nxt[j] = (uint32_t)zp[j][(size_t)g * (Np[j] >> 3)];
+        g_cur[j] = g;
+      }
+    }
+  };
+  auto commit_stage = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c >> 3, oct = c & 7;
+      *reinterpret_cast<u32x4*>(&lds[buf][row * LDS_STRIDE + oct * 8]) = a_st[i];
+    }
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) q_cur[j][t] = q_nxt[j][t];
+      if (g_changed[j]) {
+        sf[j] = fp16_bits_to_f32(sc_nxt[j]);
+        const float z = (float)((zw_nxt[j] >> zshift[j]) & 0xFu) + zoff[j];
+        nsz[j] = -sf[j] * z;  // exact: 11-bit x 5-bit
+      }
+    }
+  };
+
+#pragma unroll
+  for (int j = 0; j < NT; ++j) g_cur[j] = -1;
+  load_stage(0);
+  commit_stage(0);
+  __syncthreads();
+
+  for (int s = 0; s < n_stages; ++s) {
+    const int buf = s & 1;
+    if (s + 1 < n_stages) load_stage((s + 1) * BK);
+    const uint16_t* lb = lds[buf];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      u32x4 wf[NT];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) wf[j] = dequant8<T>(q_cur[j][t], sf[j], nsz[j]);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const u32x4 xf =
+            *reinterpret_cast<const u32x4*>(&lb[(32 * mt + l32) * LDS_STRIDE + 16 * t + 8 * half]);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[j], xf, acc[mt][j]);
+      }
+    }
+    if (s + 1 < n_stages) commit_stage(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------
+  // accumulator register 4*i0+i1 of acc[mt][j] is Y[m0 + 32*mt + l32][col0[j] + 8*i0 + 4*half + i1]
+  static_for<0, MT>([&](auto mt_c) {
+    constexpr int mt = decltype(mt_c)::value;
+    const int m = m0 + 32 * mt + l32;
+    const bool m_ok = m < a.M;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const FwdProjDev P = select_proj(a, pj[j]);
+      if (P.r > 0) {
+        f32x16 tmp;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) tmp[i] = 0.f;
+        for (int j0 = 0; j0 < P.r; j0 += 16) {
+          const int ko = j0 + 8 * half;
+          u32x4 uf = {0u, 0u, 0u, 0u}, bf = {0u, 0u, 0u, 0u};
+          if (ko < P.r) {
+            if (m_ok) uf = *reinterpret_cast<const u32x4*>(P.U + (size_t)m * P.r + ko);
+            bf = *reinterpret_cast<const u32x4*>(P.B + (size_t)(col0[j] + l32) * P.r + ko);
+          }
+          tmp = mfma32<T>(bf, uf, tmp);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][j][i] += P.s * tmp[i];
+      }
+      if (P.bias) {
+#pragma unroll
+        for (int i0 = 0; i0 < 4; ++i0) {
+          const u32x2 bv = *reinterpret_cast<const u32x2*>(P.bias + col0[j] + 8 * i0 + 4 * half);
+          acc[mt][j][4 * i0 + 0] += unpack_lo<T>(bv[0]);
+          acc[mt][j][4 * i0 + 1] += unpack_hi<T>(bv[0]);
+          acc[mt][j][4 * i0 + 2] += unpack_lo<T>(bv[1]);
+          acc[mt][j][4 * i0 + 3] += unpack_hi<T>(bv[1]);
+        }
+      }
+    }
+    if (!m_ok) return;
+    if (a.mode == FMSA_FWD_SWIGLU) {
+      if (!active[0]) return;
+      const FwdProjDev& Pe = a.p[0];
+      const FwdProjDev& Pg = a.p[1];
+#pragma unroll
+      for (int i0 = 0; i0 < 4; ++i0) {
+        const int n = col0[0] + 8 * i0 + 4 * half;
+        u32x2 ev, gv, hv;
+        float hf[4];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          ev[q] = pack2<T>(acc[mt][0][4 * i0 + 2 * q], acc[mt][0][4 * i0 + 2 * q + 1]);
+          gv[q] = pack2<T>(acc[mt][1][4 * i0 + 2 * q], acc[mt][1][4 * i0 + 2 * q + 1]);
+          // f = RNE(e32 * sigmoid(e32)) on the rounded e; h = RNE(f * g) on the rounded g
+          const float e0 = unpack_lo<T>(ev[q]), e1 = unpack_hi<T>(ev[q]);
+          const uint32_t fv = pack2<T>(e0 * sigmoidf_(e0), e1 * sigmoidf_(e1));
+          hf[2 * q] = unpack_lo<T>(fv) * unpack_lo<T>(gv[q]);
+          hf[2 * q + 1] = unpack_hi<T>(fv) * unpack_hi<T>(gv[q]);
+        }
+        hv[0] = pack2<T>(hf[0], hf[1]);
+        hv[1] = pack2<T>(hf[2], hf[3]);
+        *reinterpret_cast<u32x2*>(Pe.Y + (size_t)m * Pe.ldy + n) = ev;
+        *reinterpret_cast<u32x2*>(Pg.Y + (size_t)m * Pg.ldy + n) = gv;
+        *reinterpret_cast<u32x2*>(a.H + (size_t)m * a.ldh + n) = hv;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        if (!active[j]) continue;
+        const FwdProjDev P = select_proj(a, pj[j]);
+#pragma unroll
+        for (int i0 = 0; i0 < 4; ++i0) {
+          u32x2 yv;
+          yv[0] = pack2<T>(acc[mt][j][4 * i0 + 0], acc[mt][j][4 * i0 + 1]);
+          yv[1] = pack2<T>(acc[mt][j][4 * i0 + 2], acc[mt][j][4 * i0 + 3]);
+          *reinterpret_cast<u32x2*>(P.Y + (size_t)m * P.ldy + col0[j] + 8 * i0 + 4 * half) = yv;
+        }
+      }
+    }
+  });
+}
+
+}  // namespace
+
+int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode,
+                         void* H, int64_t ldh, int act_dtype, hipStream_t st) {
+  FwdArgs a{};
+  a.X = (const uint16_t*)X;
+  a.ldx = ldx;
+  a.M = M;
+  a.K = projs[0].w.K;
+  a.mode = mode;
+  a.H = (uint16_t*)H;
+  a.ldh = ldh;
+  int nb = 0;
+  for (int p = 0; p < 3; ++p) {
+    a.nblk_start[p] = (p < n_proj) ? nb : 0x7fffffff;
+    if (p >= n_proj) continue;
+    const fmsa_fwd_proj& s = projs[p];
+    FwdProjDev& d = a.p[p];
+    d.qweight = s.w.qweight;
+    d.scales = s.w.scales;
+    d.qzeros = s.w.qzeros;
+    d.U = (const uint16_t*)s.U;
+    d.B = (const uint16_t*)s.B;
+    d.bias = (const uint16_t*)s.bias;
+    d.Y = (uint16_t*)s.Y;
+    d.ldy = s.ldy;
+    d.N = s.w.N;
+    d.group_size = s.w.group_size;
+    d.zero_offset = s.w.zero_offset;
+    d.r = s.r;
+    d.s = s.s;
+    nb += (s.w.N + 255) / 256;
+  }
+  a.nblk_start[3] = 0x7fffffff;
+  if (mode == FMSA_FWD_SWIGLU) nb = (projs[0].w.N + 127) / 128;
+  a.nbn = nb;
+  a.nbm = (M + BM - 1) / BM;
+  dim3 grid(a.nbm * a.nbn), block(256);
+  if (act_dtype == FMSA_BF16)
+    hipLaunchKernelGGL(gptq_lora_fwd_kernel<bf16_t>, grid, block, 0, st, a);
+  else
+    hipLaunchKernelGGL(gptq_lora_fwd_kernel<f16_t>, grid, block, 0, st, a);
+  FMSA_CHECK_LAUNCH();
+  return FMSA_OK;
+}

@@ -1,0 +1,262 @@
+"""ctypes binding of libfmsa_hip.so (C ABI declared in include/fmsa.h).
+
+The library is built in-tree by ``build_hip.py`` and loaded from ``../lib``.  Nothing here falls
+back to another implementation: if the library is missing, or a call returns an error code, a
+RuntimeError is raised.  torch is used only for device memory (tensors) and the current stream.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
+from typing import Optional, Sequence
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libfmsa_hip.so")
+
+F16, BF16, F32 = 0, 1, 2
+FWD_LINEAR, FWD_SWIGLU = 0, 1
+BWD_LINEAR, BWD_SWIGLU = 0, 1
+
+_DTYPE_ENUM = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
+
+EXPORTED_SYMBOLS = (
+    "fmsa_strerror",
+    "fmsa_abi_version",
+    "fmsa_gptq_dequant",
+    "fmsa_gptq_permute_rows",
+    "fmsa_permute_cols",
+    "fmsa_lora_down",
+    "fmsa_lora_grad_workspace",
+    "fmsa_lora_grad",
+    "fmsa_gptq_lora_fwd",
+    "fmsa_gptq_lora_bwd_dx",
+)
+
+
+class GptqWeight(Structure):
+    _fields_ = [
+        ("qweight", c_void_p),
+        ("scales", c_void_p),
+        ("qzeros", c_void_p),
+        ("g_idx", c_void_p),
+        ("K", c_int32),
+        ("N", c_int32),
+        ("group_size", c_int32),
+        ("zero_offset", c_int32),
+    ]
+
+
+class FwdProj(Structure):
+    _fields_ = [
+        ("w", GptqWeight),
+        ("U", c_void_p),
+        ("B", c_void_p),
+        ("bias", c_void_p),
+        ("Y", c_void_p),
+        ("ldy", c_int64),
+        ("r", c_int32),
+        ("s", c_float),
+    ]
+
+
+class BwdProj(Structure):
+    _fields_ = [
+        ("w", GptqWeight),
+        ("dY", c_void_p),
+        ("lddy", c_int64),
+        ("T", c_void_p),
+        ("At", c_void_p),
+        ("mask_src", c_void_p),
+        ("ldmask", c_int64),
+        ("r", c_int32),
+        ("s", c_float),
+    ]
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python fms-acceleration_amd/build_hip.py` "
+            "(there is no fallback path for the fused quantised-LoRA kernels)"
+        )
+    L = ctypes.CDLL(LIB_PATH)
+    L.fmsa_strerror.restype = ctypes.c_char_p
+    L.fmsa_strerror.argtypes = [c_int]
+    L.fmsa_abi_version.restype = c_int
+    L.fmsa_gptq_dequant.argtypes = [POINTER(GptqWeight), c_int, c_void_p, c_void_p]
+    L.fmsa_gptq_permute_rows.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]
+    L.fmsa_permute_cols.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int64, c_void_p]
+    L.fmsa_lora_down.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]
+    L.fmsa_lora_grad_workspace.restype = c_size_t
+    L.fmsa_lora_grad_workspace.argtypes = [c_int, c_int, c_int]
+    L.fmsa_lora_grad.argtypes = [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                                 c_void_p, c_void_p, c_size_t, c_void_p]
+    L.fmsa_gptq_lora_fwd.argtypes = [POINTER(FwdProj), c_int, c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
+                                     c_int, c_void_p]
+    L.fmsa_gptq_lora_bwd_dx.argtypes = [POINTER(BwdProj), c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p,
+                                        c_void_p, c_int64, c_int, c_void_p]
+    for name in EXPORTED_SYMBOLS:
+        getattr(L, name)  # AttributeError here means the library is stale: rebuild it
+    _lib = L
+    return L
+
+
+class FmsaError(RuntimeError):
+    def __init__(self, fn: str, code: int):
+        msg = lib().fmsa_strerror(code).decode()
+        super().__init__(f"{fn} failed with code {code}: {msg}")
+        self.code = code
+
+
+def _check(fn: str, code: int):
+    if code != 0:
+        raise FmsaError(fn, code)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def _stream(t: torch.Tensor):
+    if not t.is_cuda:
+        raise RuntimeError("libfmsa_hip kernels need tensors on the GPU (there is no CPU implementation)")
+    return c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def act_enum(dtype: torch.dtype) -> int:
+    if dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError(f"activations must be float16 or bfloat16, got {dtype}")
+    return _DTYPE_ENUM[dtype]
+
+
+def make_weight(qweight, scales, qzeros, g_idx, group_size: int, zero_offset: int = 0) -> GptqWeight:
+    """GptqWeight from QuantLinear buffers.  g_idx=None declares the identity assignment."""
+    K = qweight.shape[0] * 8
+    N = qweight.shape[1]
+    assert qweight.dtype == torch.int32 and qzeros.dtype == torch.int32 and scales.dtype == torch.float16
+    assert qweight.is_contiguous() and qzeros.is_contiguous() and scales.is_contiguous()
+    return GptqWeight(
+        qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
+        None if g_idx is None else g_idx.data_ptr(), K, N, int(group_size), int(zero_offset),
+    )
+
+
+# ---- thin tensor-level wrappers ------------------------------------------------------------------
+def gptq_dequant(qweight, scales, qzeros, g_idx, group_size, zero_offset=0, out_dtype=torch.float16):
+    """W [K, N] = scales[g] * (q - z - zero_offset), one RNE rounding to out_dtype."""
+    w = make_weight(qweight, scales, qzeros, g_idx, group_size, zero_offset)
+    out = torch.empty((w.K, w.N), dtype=out_dtype, device=qweight.device)
+    _check("fmsa_gptq_dequant", lib().fmsa_gptq_dequant(ctypes.byref(w), _DTYPE_ENUM[out_dtype], _ptr(out), _stream(out)))
+    return out
+
+
+def gptq_permute_rows(qweight, perm):
+    K, N = qweight.shape[0] * 8, qweight.shape[1]
+    out = torch.empty_like(qweight)
+    _check("fmsa_gptq_permute_rows",
+           lib().fmsa_gptq_permute_rows(_ptr(qweight), _ptr(perm), K, N, _ptr(out), _stream(out)))
+    return out
+
+
+def permute_cols(x2d, perm, gather: bool):
+    M, C = x2d.shape
+    out = torch.empty((M, C), dtype=x2d.dtype, device=x2d.device)
+    _check("fmsa_permute_cols",
+           lib().fmsa_permute_cols(_ptr(x2d), x2d.stride(0), _ptr(perm), M, C, int(gather), act_enum(x2d.dtype),
+                                   _ptr(out), out.stride(0), _stream(out)))
+    return out
+
+
+def lora_down(x2d, wd):
+    """out [M, r] = x2d [M, C] @ wd [r, C]^T."""
+    M, C = x2d.shape
+    r = wd.shape[0]
+    assert wd.shape[1] == C and wd.is_contiguous() and wd.dtype == x2d.dtype and x2d.stride(1) == 1
+    out = torch.empty((M, r), dtype=x2d.dtype, device=x2d.device)
+    _check("fmsa_lora_down",
+           lib().fmsa_lora_down(_ptr(x2d), x2d.stride(0), _ptr(wd), M, C, r, act_enum(x2d.dtype), _ptr(out), _stream(out)))
+    return out
+
+
+_ws_cache = {}
+
+
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    key = (device.type, device.index)
+    ws = _ws_cache.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _ws_cache[key] = ws
+    return ws
+
+
+def lora_grad(L, R, scale: float, transpose_out: bool, out_dtype=torch.float32):
+    """scale * L[M, r]^T @ R[M, C] -> [r, C] (or [C, r] when transpose_out)."""
+    M, r = L.shape
+    C = R.shape[1]
+    assert R.shape[0] == M and L.is_contiguous() and R.stride(1) == 1 and L.dtype == R.dtype
+    out = torch.empty((C, r) if transpose_out else (r, C), dtype=out_dtype, device=R.device)
+    nbytes = lib().fmsa_lora_grad_workspace(M, C, r)
+    ws = _workspace(nbytes, R.device)
+    _check("fmsa_lora_grad",
+           lib().fmsa_lora_grad(_ptr(L), _ptr(R), R.stride(0), M, C, r, float(scale), int(transpose_out),
+                                act_enum(R.dtype), _DTYPE_ENUM[out_dtype], _ptr(out), _ptr(ws), ws.numel(), _stream(out)))
+    return out
+
+
+def gptq_lora_fwd(x2d, projs: Sequence[dict], mode: int = FWD_LINEAR):
+    """projs: dicts with keys w (GptqWeight), U, B, bias (tensors or None), r, s.
+    Returns the list of outputs Y_p [M, N_p]; in SWIGLU mode returns (e, g, h)."""
+    M = x2d.shape[0]
+    arr = (FwdProj * len(projs))()
+    outs = []
+    for i, p in enumerate(projs):
+        w = p["w"]
+        y = torch.empty((M, w.N), dtype=x2d.dtype, device=x2d.device)
+        outs.append(y)
+        arr[i] = FwdProj(w, _ptr(p.get("U")) if p["r"] else None, _ptr(p.get("B")) if p["r"] else None,
+                         _ptr(p.get("bias")), _ptr(y), y.stride(0), int(p["r"]), float(p["s"] or 0.0))
+    h = None
+    if mode == FWD_SWIGLU:
+        h = torch.empty_like(outs[0])
+    _check("fmsa_gptq_lora_fwd",
+           lib().fmsa_gptq_lora_fwd(arr, len(projs), _ptr(x2d), x2d.stride(0), M, mode, _ptr(h),
+                                    0 if h is None else h.stride(0), act_enum(x2d.dtype), _stream(x2d)))
+    if mode == FWD_SWIGLU:
+        return outs[0], outs[1], h
+    return outs
+
+
+def gptq_lora_bwd_dx(projs: Sequence[dict], M: int, K: int, mode: int = BWD_LINEAR, e=None, g=None):
+    """projs: dicts with keys w, dY, T, At, mask_src, r, s.  LINEAR mode returns dX [M, K];
+    SWIGLU mode overwrites e <- d_g, g <- d_e and returns h."""
+    arr = (BwdProj * len(projs))()
+    ref = projs[0]["dY"]
+    for i, p in enumerate(projs):
+        dy = p["dY"]
+        assert dy.stride(1) == 1
+        ms = p.get("mask_src")
+        arr[i] = BwdProj(p["w"], _ptr(dy), dy.stride(0), _ptr(p.get("T")) if p["r"] else None,
+                         _ptr(p.get("At")) if p["r"] else None, _ptr(ms), 0 if ms is None else ms.stride(0),
+                         int(p["r"]), float(p["s"] or 0.0))
+    if mode == BWD_SWIGLU:
+        h = torch.empty_like(e)
+        _check("fmsa_gptq_lora_bwd_dx",
+               lib().fmsa_gptq_lora_bwd_dx(arr, len(projs), M, mode, None, 0, _ptr(e), _ptr(g), _ptr(h), e.stride(0),
+                                           act_enum(ref.dtype), _stream(ref)))
+        return h
+    dx = torch.empty((M, K), dtype=ref.dtype, device=ref.device)
+    _check("fmsa_gptq_lora_bwd_dx",
+           lib().fmsa_gptq_lora_bwd_dx(arr, len(projs), M, mode, _ptr(dx), dx.stride(0), None, None, None, 0,
+                                       act_enum(ref.dtype), _stream(ref)))
+    return dx

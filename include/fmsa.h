@@ -1,0 +1,162 @@
+/*
+ * fmsa.h -- C ABI of libfmsa_hip.so: hand-written gfx950 (MI355X) kernels for the fused
+ * quantised-LoRA hot path of fms-acceleration (GPTQ 4-bit / bitsandbytes NF4 base weight,
+ * LoRA adapters, SwiGLU MLP), forward and backward.
+ *
+ * Conventions
+ *   - Every pointer that is not marked "host" is a DEVICE pointer (tensor.data_ptr()).
+ *   - Every function returns FMSA_OK (0) or a negative FMSA_ERR_* code.  Nothing throws,
+ *     nothing allocates, nothing synchronises: work is enqueued on `stream` (a hipStream_t
+ *     passed as void*, e.g. torch.cuda.current_stream().cuda_stream; NULL = default stream).
+ *   - Arguments are validated before any HIP call, so the error paths can be exercised on a
+ *     machine without a GPU.
+ *   - Activations / gradients are row-major 2-D with an explicit leading dimension in ELEMENTS.
+ *     `act_dtype` is FMSA_BF16 or FMSA_F16 and selects both the storage type and the MFMA type.
+ *
+ * Each entry point cites the reference interface it replaces, relative to
+ *   FOAK = plugins/fused-ops-and-kernels/src/fms_acceleration_foak
+ *   UL   = FOAK/fused_ops/unsloth_lora
+ *   GQ   = plugins/accelerated-peft/src/fms_acceleration_peft/gptqmodel
+ */
+#ifndef FMSA_H
+#define FMSA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FMSA_OK 0
+#define FMSA_ERR_NULL (-1)        /* a required pointer is NULL                      */
+#define FMSA_ERR_SHAPE (-2)       /* a dimension is non-positive or violates a rule  */
+#define FMSA_ERR_ALIGN (-3)       /* pointer / leading dimension not 16-byte aligned */
+#define FMSA_ERR_DTYPE (-4)       /* unknown dtype enum                              */
+#define FMSA_ERR_UNSUPPORTED (-5) /* valid input the kernels do not cover            */
+#define FMSA_ERR_WORKSPACE (-6)   /* workspace missing or too small                  */
+#define FMSA_ERR_LAUNCH (-7)      /* hipGetLastError() after the launch was not success */
+
+enum fmsa_dtype { FMSA_F16 = 0, FMSA_BF16 = 1, FMSA_F32 = 2 };
+
+/* Human-readable text for an error code (host pointer to a static string). */
+const char* fmsa_strerror(int code);
+
+/* ABI version; bumped on any signature change. */
+int fmsa_abi_version(void);
+
+/* ------------------------------------------------------------------------------------------
+ * GPTQ 4-bit weight, laid out exactly as QuantLinear's buffers
+ * (GQ/nn_modules/qlinear/qlinear_tritonv2.py:67-99; pack() :104-165):
+ *   qweight int32 [K/8, N]  nibble j of word [k8, n]  = q[8*k8 + j, n]
+ *   qzeros  int32 [G, N/8]  nibble j of word [g, n8]  = z[g, 8*n8 + j]
+ *   scales  fp16  [G, N]
+ *   g_idx   int32 [K]       group of row k; NULL means k / group_size
+ * W[k, n] = fp32(scales[g, n]) * (q[k, n] - (z[g, n] + zero_offset)),  g = g_idx[k]
+ * zero_offset is 1 for checkpoints in the AutoGPTQ v1 zero-point format and 0 otherwise
+ * (UL/gptq/fast_lora.py:100-101, UL/gptq/triton/kernels.py:113-116).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct fmsa_gptq_weight {
+  const int32_t* qweight;
+  const uint16_t* scales;
+  const int32_t* qzeros;
+  const int32_t* g_idx;
+  int32_t K;          /* in-features,  K % 32 == 0  (qlinear_tritonv2.py:57-60) */
+  int32_t N;          /* out-features, N % 32 == 0                               */
+  int32_t group_size; /* > 0; G = ceil(K / group_size)                           */
+  int32_t zero_offset;
+} fmsa_gptq_weight;
+
+/* Replaces dequant248 (UL/gptq/triton/kernels.py:125-153): materialises W[K, N] row-major in
+ * `out_dtype` (FMSA_F16 = the reference's output type, FMSA_BF16, FMSA_F32) with one
+ * round-to-nearest-even of the exact fp32 product.  Handles any g_idx (act-order). */
+int fmsa_gptq_dequant(const fmsa_gptq_weight* w /*host*/, int out_dtype, void* out, void* stream);
+
+/* One-time repack for act-order checkpoints: rows of q are gathered so that
+ * q_sorted[k', :] = q[perm[k'], :], giving a weight whose group index is k' / group_size.
+ * perm int32 [K] (device) is argsort(g_idx, stable).  qweight_out int32 [K/8, N]. */
+int fmsa_gptq_permute_rows(const int32_t* qweight, const int32_t* perm, int K, int N,
+                           int32_t* qweight_out, void* stream);
+
+/* out[m, j] = in[m, perm[j]] (gather == 1) or out[m, perm[j]] = in[m, j] (gather == 0);
+ * used to carry activations into / out of the row order of a repacked act-order weight. */
+int fmsa_permute_cols(const void* in, int64_t ld_in, const int32_t* perm, int M, int C, int gather,
+                      int act_dtype, void* out, int64_t ld_out, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Skinny LoRA GEMMs.
+ * ------------------------------------------------------------------------------------------ */
+
+/* out[M, r] = X[M, C] * Wd[r, C]^T, fp32 accumulate, one rounding to act_dtype.
+ * Covers `X @ A.t()` of matmul_lora (UL/gptq/fast_lora.py:166-167) with Wd = lora_A.weight
+ * [r, K], and `dY @ B` of the backward (:822) with Wd = lora_B.weight^T [r, N].
+ * r % 8 == 0, r <= 128, C % 8 == 0. */
+int fmsa_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype,
+                   void* out, void* stream);
+
+/* out = scale * L[M, r]^T * R[M, C]   (a reduction over the M tokens), written as
+ *   [r, C] when transpose_out == 0   (dA = s * (dY B)^T Xd,  UL/gptq/fast_lora.py:822,824,842)
+ *   [C, r] when transpose_out == 1   (dB = s * dY^T (Xd A^T), :823,825,843)
+ * Deterministic two-pass reduction: partial sums over fixed M-chunks go to `workspace`
+ * (fp32, fmsa_lora_grad_workspace() bytes) and are summed in a fixed order.
+ * out_dtype: FMSA_F32, FMSA_BF16 or FMSA_F16. */
+size_t fmsa_lora_grad_workspace(int M, int C, int r);
+int fmsa_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, int r, float scale,
+                   int transpose_out, int act_dtype, int out_dtype, void* out, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Fused forward:  Y_p = X * deq(W_p) + s_p * U_p * B_p^T (+ bias_p)   for 1..3 projections
+ * sharing X (LoRA_W / LoRA_QKV forward, UL/gptq/fast_lora.py:770-805, 497-589), or the
+ * gate/up pair of LoRA_MLP with the SwiGLU of UL/swiglu.py:20-37 fused into the epilogue
+ * (UL/gptq/fast_lora.py:252-262): mode FMSA_FWD_SWIGLU writes e = Y_0, g = Y_1 and
+ * h = silu(e) * g.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct fmsa_fwd_proj {
+  fmsa_gptq_weight w;
+  const void* U;    /* [M, r] act_dtype = Xd * A^T (fmsa_lora_down); NULL when r == 0 */
+  const void* B;    /* [N, r] act_dtype = lora_B.weight                               */
+  const void* bias; /* [N] act_dtype or NULL                                           */
+  void* Y;          /* [M, N] act_dtype                                                */
+  int64_t ldy;
+  int32_t r;        /* 0 = adapters disabled (base only); else r % 8 == 0, r <= 128    */
+  float s;          /* lora_alpha / r                                                  */
+} fmsa_fwd_proj;
+
+enum fmsa_fwd_mode { FMSA_FWD_LINEAR = 0, FMSA_FWD_SWIGLU = 1 };
+
+int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs /*host*/, int n_proj, const void* X, int64_t ldx,
+                       int M, int mode, void* H, int64_t ldh, int act_dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Fused input-gradient:
+ *   dX = sum_p [ dY_p * deq(W_p)^T + mask_p (.) ( T_p * (s_p A_p) ) ],  T_p = dY_p * B_p
+ * for 1..3 projections sharing the input (LoRA_W / LoRA_QKV / the gate+up half of LoRA_MLP
+ * backward, UL/gptq/fast_lora.py:828-831, 657-674, 388-398).  mask_p = (mask_src_p != 0)
+ * element-wise over [M, K] (the post-dropout input; NULL = no mask).
+ * Mode FMSA_BWD_SWIGLU is the down-projection half of LoRA_MLP backward (:351-366): the result
+ * is dh, and the epilogue applies UL/swiglu.py:50-89 in place: reads e, g; writes h -> `h_out`,
+ * d_g = dh*f -> `e`, d_e -> `g`.  dX is not written in that mode.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct fmsa_bwd_proj {
+  fmsa_gptq_weight w;
+  const void* dY;   /* [M, N] act_dtype */
+  int64_t lddy;
+  const void* T;    /* [M, r] act_dtype = dY * B; NULL when r == 0 */
+  const void* At;   /* [K, r] act_dtype = lora_A.weight^T (contiguous) */
+  const void* mask_src; /* [M, K] act_dtype or NULL */
+  int64_t ldmask;
+  int32_t r;
+  float s;
+} fmsa_bwd_proj;
+
+enum fmsa_bwd_mode { FMSA_BWD_LINEAR = 0, FMSA_BWD_SWIGLU = 1 };
+
+int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs /*host*/, int n_proj, int M, int mode,
+                          void* dX, int64_t lddx, void* e, void* g, void* h_out, int64_t ldeg,
+                          int act_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FMSA_H */

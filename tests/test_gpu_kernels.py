@@ -1,0 +1,232 @@
+"""GPU parity tests of the C-ABI kernels against the CPU oracle (run on the MI355X box)."""
+import pytest
+import torch
+
+from oracle import gptq as ogptq
+from oracle import lora as olora
+from tests.helpers import make_gptq, randn
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2  # max |out - ref| / max |ref| against the fp32 oracle, per tensor
+
+
+def dev(t):
+    return t.cuda()
+
+
+def gweight(w, identity=True):
+    import fmsa_hip
+
+    t = {k: dev(v) for k, v in w["t"].items()}
+    w["dev"] = t
+    return fmsa_hip.make_weight(t["qweight"], t["scales"], t["qzeros"], None if identity else t["g_idx"],
+                                w["group_size"], w["zero_offset"])
+
+
+@pytest.mark.parametrize("K,N,gs", [(256, 256, 128), (2048, 2048, 128), (96, 160, 32), (512, 1024, 64)])
+@pytest.mark.parametrize("act_order", [False, True])
+@pytest.mark.parametrize("v1", [False, True])
+def test_dequant_bit_exact(K, N, gs, act_order, v1):
+    import fmsa_hip
+
+    w = make_gptq(K, N, gs, seed=K + N, act_order=act_order, v1=v1)
+    t = {k: dev(v) for k, v in w["t"].items()}
+    for name, dt in (("fp16", torch.float16), ("bf16", torch.bfloat16), ("fp32", torch.float32)):
+        ref = ogptq.dequant(w["np"]["qweight"], w["np"]["scales"], w["np"]["qzeros"], w["np"]["g_idx"],
+                            zero_offset=w["zero_offset"], out=name)
+        out = fmsa_hip.gptq_dequant(t["qweight"], t["scales"], t["qzeros"], t["g_idx"], w["group_size"],
+                                    w["zero_offset"], dt).cpu()
+        assert torch.equal(out.view(torch.int16 if dt != torch.float32 else torch.int32),
+                           ref.view(torch.int16 if dt != torch.float32 else torch.int32)), name
+        if not act_order:  # NULL g_idx means k // group_size
+            out2 = fmsa_hip.gptq_dequant(t["qweight"], t["scales"], t["qzeros"], None, w["group_size"],
+                                         w["zero_offset"], dt).cpu()
+            assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,C,r", [(512, 2048, 16), (200, 4096, 8), (64, 1056, 64), (33, 96, 24)])
+def test_lora_down(M, C, r, dtype):
+    import fmsa_hip
+
+    x = randn((M, C), 2, dtype)
+    wd = randn((r, C), 1, dtype, 0.05)
+    ref = x.float() @ wd.float().t()
+    out = fmsa_hip.lora_down(dev(x), dev(wd)).cpu()
+    assert olora.max_rel_err(out, ref) < 5e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,C,r,tr", [(512, 2048, 16, False), (200, 1056, 8, True), (4096, 4096, 16, True), (96, 130, 24, False)])
+def test_lora_grad(M, C, r, tr, dtype):
+    import fmsa_hip
+
+    L = randn((M, r), 5, dtype)
+    R = randn((M, C), 6, dtype)
+    ref = 0.5 * (L.float().t() @ R.float())
+    if tr:
+        ref = ref.t()
+    out = fmsa_hip.lora_grad(dev(L), dev(R), 0.5, tr, torch.float32).cpu()
+    assert out.shape == ref.shape
+    assert olora.max_rel_err(out, ref) < 1e-4
+    out2 = fmsa_hip.lora_grad(dev(L), dev(R), 0.5, tr, torch.float32).cpu()
+    assert torch.equal(out, out2), "two-pass reduction must be run-to-run bit-stable"
+    outb = fmsa_hip.lora_grad(dev(L), dev(R), 0.5, tr, dtype).cpu()
+    assert olora.max_rel_err(outb, ref) < 5e-3
+
+
+def _fwd_case(M, K, N, gs, r, dtype, s=2.0, bias=False, seed=0):
+    w = make_gptq(K, N, gs, seed=seed)
+    x = randn((M, K), 2 + seed, dtype)
+    A, B = olora.make_lora(K, N, r, 1 + seed) if r else (None, None)
+    b = randn((N,), 9, dtype, 0.1) if bias else None
+    return w, x, A, B, b, s
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,N,gs,r,bias", [
+    (512, 2048, 2048, 128, 16, False),
+    (256, 256, 256, 128, 16, True),
+    (200, 1024, 1056, 64, 8, False),   # ragged M, N not a multiple of the 256-wide tile
+    (128, 2048, 2048, 128, 0, False),  # adapters disabled: base only
+    (300, 96, 64, 32 * 2, 32, True),   # K not a multiple of the 64-wide stage
+    (64, 512, 512, 512, 64, False),    # one group (group_size == K), rank 64
+])
+def test_fwd_linear(M, K, N, gs, r, bias, dtype):
+    import fmsa_hip
+
+    w, x, A, B, b, s = _fwd_case(M, K, N, gs, r, dtype, bias=bias)
+    ref = olora.lora_linear(x.float(), w["dense"], None if A is None else A.to(dtype).float(),
+                            None if B is None else B.to(dtype).float(), s, None if b is None else b.float())
+    gw = gweight(w)
+    xd = dev(x)
+    p = {"w": gw, "r": r, "s": s, "bias": None if b is None else dev(b)}
+    if r:
+        Ad, Bd = dev(A.to(dtype)), dev(B.to(dtype))
+        p["U"] = fmsa_hip.lora_down(xd, Ad)
+        p["B"] = Bd
+    (y,) = fmsa_hip.gptq_lora_fwd(xd, [p])
+    err = olora.max_rel_err(y.cpu(), ref)
+    assert err < TOL, err
+
+
+def _proj_fwd(w, x_dev, A, B, s, dtype):
+    import fmsa_hip
+
+    p = {"w": gweight(w), "r": A.shape[0], "s": s, "bias": None}
+    p["U"] = fmsa_hip.lora_down(x_dev, dev(A.to(dtype)))
+    p["B"] = dev(B.to(dtype))
+    return p
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fwd_qkv_shared_input(dtype):
+    """q 1024->1024, k/v 1024->256 (GQA-like), one launch over the concatenated N."""
+    import fmsa_hip
+
+    M, K, r, s = 384, 1024, 16, 2.0
+    Ns = [1024, 256, 288]
+    x = randn((M, K), 2, dtype)
+    xd = dev(x)
+    ws = [make_gptq(K, N, 128, seed=10 + i) for i, N in enumerate(Ns)]
+    ABs = [olora.make_lora(K, N, r, 20 + i) for i, N in enumerate(Ns)]
+    projs = [_proj_fwd(w, xd, A, B, s, dtype) for w, (A, B) in zip(ws, ABs)]
+    outs = fmsa_hip.gptq_lora_fwd(xd, projs)
+    for w, (A, B), y in zip(ws, ABs, outs):
+        ref = olora.lora_linear(x.float(), w["dense"], A.to(dtype).float(), B.to(dtype).float(), s)
+        assert olora.max_rel_err(y.cpu(), ref) < TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,H,I", [(256, 512, 1024), (200, 256, 352)])
+def test_fwd_swiglu(M, H, I, dtype):
+    import fmsa_hip
+
+    r, s = 16, 1.0
+    x = randn((M, H), 2, dtype)
+    xd = dev(x)
+    wg, wu = make_gptq(H, I, 128, seed=1), make_gptq(H, I, 128, seed=2)
+    (Ag, Bg), (Au, Bu) = olora.make_lora(H, I, r, 3), olora.make_lora(H, I, r, 4)
+    e, g, h = fmsa_hip.gptq_lora_fwd(xd, [_proj_fwd(wg, xd, Ag, Bg, s, dtype), _proj_fwd(wu, xd, Au, Bu, s, dtype)],
+                                     fmsa_hip.FWD_SWIGLU)
+    e_ref = olora.lora_linear(x.float(), wg["dense"], Ag.to(dtype).float(), Bg.to(dtype).float(), s)
+    g_ref = olora.lora_linear(x.float(), wu["dense"], Au.to(dtype).float(), Bu.to(dtype).float(), s)
+    assert olora.max_rel_err(e.cpu(), e_ref) < TOL
+    assert olora.max_rel_err(g.cpu(), g_ref) < TOL
+    # h must be the reference's SwiGLU of the STORED e, g (same rounding points)
+    h_ref = olora.swiglu_fwd(e.cpu(), g.cpu())
+    assert olora.max_rel_err(h.cpu(), h_ref.float()) < 4e-3
+    assert olora.max_rel_err(h.cpu(), torch.nn.functional.silu(e_ref) * g_ref) < TOL
+
+
+def _proj_bwd(w, dy_dev, A, B, s, dtype, mask_src=None):
+    import fmsa_hip
+
+    p = {"w": gweight(w), "r": A.shape[0], "s": s, "dY": dy_dev, "mask_src": mask_src}
+    p["T"] = fmsa_hip.lora_down(dy_dev, dev(B.to(dtype).t().contiguous()))
+    p["At"] = dev(A.to(dtype).t().contiguous())
+    return p
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,N,gs,r", [
+    (512, 2048, 2048, 128, 16),
+    (200, 1056, 1024, 64, 8),   # ragged M; K not a multiple of the 256-wide output tile
+    (256, 256, 96, 128, 64),    # N not a multiple of the 64-wide stage
+])
+def test_bwd_dx_linear(M, K, N, gs, r, dtype):
+    import fmsa_hip
+
+    s = 2.0
+    w = make_gptq(K, N, gs, seed=3)
+    A, B = olora.make_lora(K, N, r, 4)
+    x = randn((M, K), 2, dtype)
+    x[::7, ::5] = 0  # exact zeros: the LoRA part of dX is masked there
+    dy = randn((M, N), 3, dtype)
+    dyd = dev(dy)
+    dx = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(w, dyd, A, B, s, dtype, mask_src=dev(x))], M, K)
+    ref, _, _ = olora.lora_w_manual(x.float(), w["dense"], A.to(dtype).float(), B.to(dtype).float(), s, dy.float())
+    assert olora.max_rel_err(dx.cpu(), ref) < TOL
+    # without the mask source the LoRA term is applied everywhere
+    dx2 = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(w, dyd, A, B, s, dtype)], M, K)
+    ref2 = dy.float() @ w["dense"].t() + (dy.float() @ B.to(dtype).float()) @ (s * A.to(dtype).float())
+    assert olora.max_rel_err(dx2.cpu(), ref2) < TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16])
+def test_bwd_dx_three_projections(dtype):
+    import fmsa_hip
+
+    M, K, r, s = 320, 1024, 16, 2.0
+    Ns = [1024, 256, 288]
+    x = randn((M, K), 2, dtype)
+    ws = [make_gptq(K, N, 128, seed=10 + i) for i, N in enumerate(Ns)]
+    ABs = [olora.make_lora(K, N, r, 20 + i) for i, N in enumerate(Ns)]
+    dys = [randn((M, N), 30 + i, dtype) for i, N in enumerate(Ns)]
+    projs = [_proj_bwd(w, dev(dy), A, B, s, dtype, mask_src=dev(x)) for w, (A, B), dy in zip(ws, ABs, dys)]
+    dx = fmsa_hip.gptq_lora_bwd_dx(projs, M, K)
+    ref, _ = olora.lora_qkv_manual(x.float(), [(w["dense"], A.to(dtype).float(), B.to(dtype).float(), s)
+                                                 for w, (A, B) in zip(ws, ABs)], [d.float() for d in dys])
+    assert olora.max_rel_err(dx.cpu(), ref) < TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,H,I", [(256, 512, 1024), (200, 256, 352)])
+def test_bwd_swiglu(M, H, I, dtype):
+    """Down-projection backward: dh = dY Wd^T + LoRA, then the in-place SwiGLU backward."""
+    import fmsa_hip
+
+    r, s = 16, 1.0
+    wd = make_gptq(I, H, 128 if I % 128 == 0 else 32 * 11, seed=5)  # down: I -> H, so K = I, N = H
+    Ad, Bd = olora.make_lora(I, H, r, 6)
+    e = randn((M, I), 7, dtype)
+    g = randn((M, I), 8, dtype)
+    dy = randn((M, H), 9, dtype)
+    e_d, g_d = dev(e).clone(), dev(g).clone()
+    h = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(wd, dev(dy), Ad, Bd, s, dtype)], M, I, fmsa_hip.BWD_SWIGLU, e=e_d, g=g_d)
+    dh_ref = dy.float() @ wd["dense"].t() + (dy.float() @ Bd.to(dtype).float()) @ (s * Ad.to(dtype).float())
+    h_ref, dg_ref, de_ref = olora.swiglu_bwd(dh_ref.to(dtype), e, g)
+    assert olora.max_rel_err(h.cpu(), h_ref.float()) < 4e-3
+    assert olora.max_rel_err(e_d.cpu(), dg_ref.float()) < TOL
+    assert olora.max_rel_err(g_d.cpu(), de_ref.float()) < TOL
