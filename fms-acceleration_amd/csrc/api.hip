@@ -16,6 +16,10 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
 int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx, void* e,
                             void* g, void* h_out, int64_t ldeg, int act_dtype, hipStream_t st);
 
+int launch_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype, hipStream_t st);
+int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, int M, int I, int64_t ld, int act_dtype,
+                      hipStream_t st);
+
 namespace {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -185,6 +189,24 @@ int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mod
     if (!aligned16(dX) || lddx % 8 != 0) return FMSA_ERR_ALIGN;
   }
   return launch_gptq_lora_bwd_dx(projs, n_proj, M, mode, dX, lddx, e, g, h_out, ldeg, act_dtype, (hipStream_t)stream);
+}
+
+int fmsa_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype, void* stream) {
+  if (!e || !g || !h) return FMSA_ERR_NULL;
+  if (M <= 0 || I <= 0 || I % 8 != 0 || ld < I) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  if (!aligned16(e) || !aligned16(g) || !aligned16(h) || ld % 8 != 0) return FMSA_ERR_ALIGN;
+  return launch_swiglu_fwd(e, g, h, M, I, ld, act_dtype, (hipStream_t)stream);
+}
+
+int fmsa_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h_out, int M, int I, int64_t ld,
+                    int act_dtype, void* stream) {
+  if (!dh || !e || !g || !h_out) return FMSA_ERR_NULL;
+  if (M <= 0 || I <= 0 || I % 8 != 0 || ld < I || lddh < I) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  if (!aligned16(dh) || !aligned16(e) || !aligned16(g) || !aligned16(h_out) || ld % 8 != 0 || lddh % 8 != 0)
+    return FMSA_ERR_ALIGN;
+  return launch_swiglu_bwd(dh, lddh, e, g, h_out, M, I, ld, act_dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,472 @@
+"""Fused GPTQ-LoRA autograd functions on the gfx950 kernels of libfmsa_hip.
+
+Drop-in counterparts of the reference's `LoRA_MLP`, `LoRA_QKV`, `LoRA_W` and their module-level
+entry points (fused_ops/unsloth_lora/gptq/fast_lora.py: :174-435, :466-711, :742-846, entry points
+:438-463, :714-739, :849-859): same names, same positional argument order per projection
+(`qweight, scales, qzeros, g_idx, bits, bias, A, B, S`), same gradient tuple (None for every frozen
+or non-tensor input, dA / dB in the layouts of `lora_A.weight` [r, K] and `lora_B.weight` [N, r]).
+
+What differs is where the work happens.  The reference dequantises W to a dense fp16 matrix and
+calls torch.matmul plus ~20 small GEMMs and elementwise kernels per function; here each function
+is a handful of launches:
+
+  forward   U = Xd A^T                 (fmsa_lora_down, streams X once)
+            Y = X deq(W) + s U B^T     (fmsa_gptq_lora_fwd: nibble unpack in registers -> MFMA,
+                                        LoRA / bias / SwiGLU in the epilogue)
+  backward  T = dY B                   (fmsa_lora_down)
+            dA = s T^T Xd, dB = s dY^T U   (fmsa_lora_grad, deterministic)
+            dX = dY deq(W)^T + (Xd != 0) * T (s A)      (fmsa_gptq_lora_bwd_dx)
+
+There is no CPU or PyTorch fallback: tensors must live on the GPU and the library must be built.
+
+Known, documented departures from the reference text:
+  * LoRA_MLP.backward masks the LoRA part of dh with (dropout(h) != 0), the form the reference
+    uses for every other projection; its own line (:354-357) multiplies dY in place by a mask of
+    h's shape and cannot run when hidden != intermediate.
+  * Like the reference (UL/swiglu.py:86-88) the MLP backward overwrites the saved e and g, so a
+    graph can be back-propagated once (no retain_graph / double backward).
+  * 4-bit only (the reference's dequant also accepts 2 and 8 bits).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+import fmsa_hip
+
+
+# ----------------------------------------------------------------------------------------------
+# quantisation state (mirrors GPTQuantState / extract_gptq_state / get_lora_parameters, :19-116)
+# ----------------------------------------------------------------------------------------------
+@dataclass
+class GPTQuantState:
+    infeatures: int
+    outfeatures: int
+    bits: int
+    group_size: int
+    maxq: int
+    qweight: torch.Tensor
+    qzeros: torch.Tensor
+    scales: torch.Tensor
+    g_idx: torch.Tensor
+    bias: Optional[torch.Tensor] = None
+
+
+def unpack_gptqstate(qstate):
+    return qstate.qweight, qstate.scales, qstate.qzeros, qstate.g_idx, qstate.bits
+
+
+def _nonzero_bias(qmodule):
+    """The reference drops an all-zero bias (:63-67) with a count_nonzero per call; the answer is
+    cached on the tensor and refreshed when the tensor is modified."""
+    bias = getattr(qmodule, "bias", None)
+    if bias is None:
+        return None
+    cached = getattr(bias, "_fmsa_nonzero", None)
+    if cached is None or cached[0] != bias._version:
+        cached = (bias._version, bool(bias.count_nonzero() > 0))
+        bias._fmsa_nonzero = cached
+    return bias if cached[1] else None
+
+
+def extract_gptq_state(qmodule):
+    if hasattr(qmodule, "base_layer"):
+        qmodule = qmodule.base_layer
+    return GPTQuantState(
+        infeatures=qmodule.infeatures,
+        outfeatures=qmodule.outfeatures,
+        bits=qmodule.bits,
+        group_size=qmodule.group_size,
+        maxq=qmodule.maxq,
+        qweight=qmodule.qweight,
+        qzeros=qmodule.qzeros,
+        scales=qmodule.scales,
+        g_idx=qmodule.g_idx,
+        bias=_nonzero_bias(qmodule),
+    )
+
+
+def get_lora_parameters(proj):
+    """(qstate, bias, A, B, s, dropout) of a LoRA-wrapped (or bare) GPTQ linear; A = B = s = None
+    when the adapters are disabled or merged (:94-116)."""
+    base_layer = proj.base_layer if hasattr(proj, "base_layer") else proj
+    qstate = extract_gptq_state(base_layer)
+    bias = qstate.bias
+    if base_layer.__module__.startswith("auto_gptq"):
+        # checkpoints packed by the external auto_gptq library keep zero-1 in qzeros
+        setattr(qstate.qzeros, "offset", 1)
+    if not hasattr(proj, "disable_adapters") or proj.disable_adapters or proj.merged:
+        return qstate, bias, None, None, None, None
+    active = proj.active_adapters[0] if hasattr(proj, "active_adapters") else proj.active_adapter
+    A = proj.lora_A[active].weight
+    B = proj.lora_B[active].weight
+    s = proj.scaling[active]
+    dropout = proj.lora_dropout[active] if hasattr(proj, "lora_dropout") else None
+    return qstate, bias, A, B, s, dropout
+
+
+# ----------------------------------------------------------------------------------------------
+# per-weight preparation, cached on the qweight tensor
+# ----------------------------------------------------------------------------------------------
+class _PreparedWeight:
+    """The C-ABI view of one QuantLinear.  For an act-order g_idx the packed rows are re-ordered
+    once (fmsa_gptq_permute_rows) so that the group of row k' is k' // group_size; `perm` then
+    maps the kernels' row order back to the model's: row k' of the repacked weight is row
+    perm[k'] of the original."""
+
+    __slots__ = ("struct", "K", "N", "group_size", "perm", "_keep")
+
+    def __init__(self, qweight, scales, qzeros, g_idx, bits):
+        if bits != 4:
+            raise NotImplementedError(f"the gfx950 fused kernels cover 4-bit GPTQ only (got bits={bits})")
+        if not qweight.is_cuda:
+            raise RuntimeError("fused GPTQ-LoRA ops need the quantised weight on the GPU")
+        K, N, G = qweight.shape[0] * 8, qweight.shape[1], scales.shape[0]
+        if K % G != 0:
+            raise NotImplementedError(f"in_features {K} is not a multiple of the number of groups {G}")
+        gs = K // G
+        zero_offset = int(getattr(qzeros, "offset", 0) or 0)
+        qweight, scales, qzeros = qweight.contiguous(), scales.contiguous(), qzeros.contiguous()
+        ident = torch.arange(K, device=g_idx.device, dtype=torch.int64) // gs
+        g64 = g_idx.to(torch.int64)
+        g64 = torch.where(g64 < 0, g64 + G, g64)
+        perm = None
+        if not torch.equal(g64, ident):
+            perm64 = torch.argsort(g64, stable=True)
+            if not torch.equal(g64[perm64], ident):
+                raise NotImplementedError("act-order g_idx with groups of unequal size is not supported")
+            perm = perm64.to(torch.int32).contiguous()
+            qweight = fmsa_hip.gptq_permute_rows(qweight, perm)
+        self.K, self.N, self.group_size, self.perm = K, N, gs, perm
+        self._keep = (qweight, scales, qzeros)
+        self.struct = fmsa_hip.make_weight(qweight, scales, qzeros, None, gs, zero_offset)
+
+
+def _prepare(qweight, scales, qzeros, g_idx, bits) -> _PreparedWeight:
+    key = (qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(), g_idx.data_ptr(), g_idx._version,
+           qweight._version, int(getattr(qzeros, "offset", 0) or 0))
+    cached = getattr(qweight, "_fmsa_prepared", None)
+    if cached is None or cached[0] != key:
+        cached = (key, _PreparedWeight(qweight, scales, qzeros, g_idx, bits))
+        qweight._fmsa_prepared = cached
+    return cached[1]
+
+
+# ----------------------------------------------------------------------------------------------
+# small helpers shared by the three functions
+# ----------------------------------------------------------------------------------------------
+def _act_dtype(X):
+    if X.dtype in (torch.float16, torch.bfloat16):
+        return X.dtype
+    if torch.is_autocast_enabled():
+        return torch.get_autocast_gpu_dtype()
+    raise TypeError(f"fused GPTQ-LoRA ops compute in float16 / bfloat16, got {X.dtype} outside autocast")
+
+
+def _as2d(X, dtype):
+    X2 = X.reshape(-1, X.shape[-1])
+    if X2.dtype != dtype:
+        X2 = X2.to(dtype)
+    return X2 if X2.is_contiguous() else X2.contiguous()
+
+
+def _apply_dropout(X2, dropout):
+    """Post-dropout input of the LoRA branch (matmul_lora :155-163).  Returns X2 itself when the
+    module is absent or an identity."""
+    if dropout is None or isinstance(dropout, torch.nn.Identity):
+        return X2
+    if isinstance(dropout, torch.Tensor):
+        return X2 * dropout.reshape(X2.shape).to(X2.dtype)
+    Xd = dropout(X2)
+    return Xd if Xd.is_contiguous() else Xd.contiguous()
+
+
+class _Proj:
+    """One projection's operands in the forms the kernels take."""
+
+    def __init__(self, args, dtype):
+        qweight, scales, qzeros, g_idx, bits, bias, A, B, S = args
+        self.w = _prepare(qweight, scales, qzeros, g_idx, bits)
+        self.bias = None if bias is None else bias.to(dtype)
+        self.A_param, self.B_param = A, B
+        self.r = 0 if A is None else A.shape[0]
+        self.s = 0.0 if S is None else float(S)
+        self.A = None if A is None else A.detach().to(dtype).contiguous()  # [r, K]
+        self.B = None if B is None else B.detach().to(dtype).contiguous()  # [N, r]
+
+    # the kernels walk K in the repacked order for act-order weights
+    def to_kernel_order(self, X2):
+        return X2 if self.w.perm is None else fmsa_hip.permute_cols(X2, self.w.perm, gather=True)
+
+    def from_kernel_order(self, dXp):
+        return dXp if self.w.perm is None else fmsa_hip.permute_cols(dXp, self.w.perm, gather=False)
+
+    def fwd_dict(self, U):
+        return {"w": self.w.struct, "U": U, "B": self.B, "bias": self.bias, "r": self.r, "s": self.s}
+
+    def bwd_dict(self, dY2, T, mask_src):
+        At = None
+        if self.r:
+            At = self.A.t().contiguous()  # [K, r]
+            if self.w.perm is not None:
+                At = At[self.w.perm.long()].contiguous()
+                mask_src = None if mask_src is None else fmsa_hip.permute_cols(mask_src, self.w.perm, gather=True)
+        return {"w": self.w.struct, "dY": dY2, "T": T, "At": At, "mask_src": mask_src if self.r else None,
+                "r": self.r, "s": self.s}
+
+    def lora_grads(self, T, Xd, U, dY2):
+        """dA [r, K] = s T^T Xd and dB [N, r] = s dY^T U, in the dtypes of the parameters."""
+        if not self.r:
+            return None, None
+        dA = fmsa_hip.lora_grad(T, Xd, self.s, False, self.A_param.dtype)
+        dB = fmsa_hip.lora_grad(U, dY2, self.s, True, self.B_param.dtype)
+        return dA, dB
+
+
+def _linear_forward(projs, X2, Xds):
+    """Y_p = X deq(W_p) + s U_p B_p^T for projections sharing X2.  One launch when no weight is
+    act-order; otherwise one launch per projection on its own column-permuted copy of X."""
+    Us = [fmsa_hip.lora_down(Xd, p.A) if p.r else None for p, Xd in zip(projs, Xds)]
+    if all(p.w.perm is None for p in projs):
+        outs = fmsa_hip.gptq_lora_fwd(X2, [p.fwd_dict(U) for p, U in zip(projs, Us)])
+    else:
+        outs = [fmsa_hip.gptq_lora_fwd(p.to_kernel_order(X2), [p.fwd_dict(U)])[0] for p, U in zip(projs, Us)]
+    return outs, Us
+
+
+def _linear_backward_dx(projs, dYs, Ts, Xds, M, K):
+    if all(p.w.perm is None for p in projs):
+        return fmsa_hip.gptq_lora_bwd_dx([p.bwd_dict(dY, T, Xd) for p, dY, T, Xd in zip(projs, dYs, Ts, Xds)], M, K)
+    dX = None
+    for p, dY, T, Xd in zip(projs, dYs, Ts, Xds):
+        part = p.from_kernel_order(fmsa_hip.gptq_lora_bwd_dx([p.bwd_dict(dY, T, Xd)], M, K))
+        dX = part if dX is None else dX.add_(part)
+    return dX
+
+
+def _Bt(p):
+    return p.B.t().contiguous()  # [r, N]
+
+
+# ----------------------------------------------------------------------------------------------
+# LoRA_W  (o_proj)
+# ----------------------------------------------------------------------------------------------
+class LoRA_W(torch.autograd.Function):
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, X, O_qweight, O_scales, O_qzeros, O_g_idx, O_bits, O_bias, A, B, S, dropout_O=None):
+        dtype = _act_dtype(X)
+        X2 = _as2d(X, dtype)
+        p = _Proj((O_qweight, O_scales, O_qzeros, O_g_idx, O_bits, O_bias, A, B, S), dtype)
+        Xd = _apply_dropout(X2, dropout_O) if p.r else X2
+        (Y,), (U,) = _linear_forward([p], X2, [Xd])
+        ctx.proj = p
+        ctx.act_dtype = dtype
+        ctx.x_shape, ctx.x_dtype = X.shape, X.dtype
+        ctx.save_for_backward(Xd, U) if p.r else ctx.save_for_backward()
+        return Y.view(*X.shape[:-1], p.w.N)
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dY):
+        p = ctx.proj
+        dY2 = _as2d(dY, ctx.act_dtype)
+        M, K = dY2.shape[0], p.w.K
+        dA = dB = None
+        T = Xd = None
+        if p.r:
+            Xd, U = ctx.saved_tensors
+            T = fmsa_hip.lora_down(dY2, _Bt(p))
+            dA, dB = p.lora_grads(T, Xd, U, dY2)
+        dX = _linear_backward_dx([p], [dY2], [T], [Xd], M, K)
+        return (dX.view(ctx.x_shape).to(ctx.x_dtype), None, None, None, None, None, None, dA, dB, None, None)
+
+
+# ----------------------------------------------------------------------------------------------
+# LoRA_QKV
+# ----------------------------------------------------------------------------------------------
+class LoRA_QKV(torch.autograd.Function):
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(
+        ctx, X,
+        Q_qweight, Q_scales, Q_qzeros, Q_g_idx, Q_bits, Q_bias, QA, QB, QS,
+        K_qweight, K_scales, K_qzeros, K_g_idx, K_bits, K_bias, KA, KB, KS,
+        V_qweight, V_scales, V_qzeros, V_g_idx, V_bits, V_bias, VA, VB, VS,
+        dropout_Q=None, dropout_K=None, dropout_V=None,
+    ):
+        dtype = _act_dtype(X)
+        X2 = _as2d(X, dtype)
+        projs = [
+            _Proj((Q_qweight, Q_scales, Q_qzeros, Q_g_idx, Q_bits, Q_bias, QA, QB, QS), dtype),
+            _Proj((K_qweight, K_scales, K_qzeros, K_g_idx, K_bits, K_bias, KA, KB, KS), dtype),
+            _Proj((V_qweight, V_scales, V_qzeros, V_g_idx, V_bits, V_bias, VA, VB, VS), dtype),
+        ]
+        Xds = [_apply_dropout(X2, d) if p.r else X2 for p, d in zip(projs, (dropout_Q, dropout_K, dropout_V))]
+        outs, Us = _linear_forward(projs, X2, Xds)
+        ctx.projs = projs
+        ctx.act_dtype = dtype
+        ctx.x_shape, ctx.x_dtype = X.shape, X.dtype
+        # tensors that may be None (disabled adapters) cannot go through save_for_backward as a
+        # fixed-length tuple; store how many were saved per projection
+        saved, ctx.layout = [], []
+        for Xd, U, p in zip(Xds, Us, projs):
+            ctx.layout.append(bool(p.r))
+            if p.r:
+                saved += [Xd, U]
+        ctx.save_for_backward(*saved)
+        return tuple(y.view(*X.shape[:-1], p.w.N) for y, p in zip(outs, projs))
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dQ, dK, dV):
+        projs = ctx.projs
+        saved = list(ctx.saved_tensors)
+        K = projs[0].w.K
+        dYs, Ts, Xds, grads = [], [], [], []
+        for p, dY, has in zip(projs, (dQ, dK, dV), ctx.layout):
+            dY2 = _as2d(dY, ctx.act_dtype)  # dK may arrive non-contiguous (:631)
+            T = Xd = None
+            dA = dB = None
+            if has:
+                Xd, U = saved.pop(0), saved.pop(0)
+                T = fmsa_hip.lora_down(dY2, _Bt(p))
+                dA, dB = p.lora_grads(T, Xd, U, dY2)
+            dYs.append(dY2)
+            Ts.append(T)
+            Xds.append(Xd)
+            grads.append((dA, dB))
+        M = dYs[0].shape[0]
+        dX = _linear_backward_dx(projs, dYs, Ts, Xds, M, K)
+        n6 = (None,) * 6
+        return (
+            dX.view(ctx.x_shape).to(ctx.x_dtype),
+            *n6, grads[0][0], grads[0][1], None,
+            *n6, grads[1][0], grads[1][1], None,
+            *n6, grads[2][0], grads[2][1], None,
+            None, None, None,
+        )
+
+
+# ----------------------------------------------------------------------------------------------
+# LoRA_MLP  (SwiGLU)
+# ----------------------------------------------------------------------------------------------
+class LoRA_MLP(torch.autograd.Function):
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(
+        ctx, X,
+        gate_qweight, gate_scales, gate_qzeros, gate_g_idx, gate_bits, gate_bias, gateA, gateB, gateS,
+        up_qweight, up_scales, up_qzeros, up_g_idx, up_bits, up_bias, upA, upB, upS,
+        down_qweight, down_scales, down_qzeros, down_g_idx, down_bits, down_bias, downA, downB, downS,
+        dropout_gate=None, dropout_up=None, dropout_down=None,
+    ):
+        dtype = _act_dtype(X)
+        X2 = _as2d(X, dtype)
+        gate = _Proj((gate_qweight, gate_scales, gate_qzeros, gate_g_idx, gate_bits, gate_bias, gateA, gateB, gateS), dtype)
+        up = _Proj((up_qweight, up_scales, up_qzeros, up_g_idx, up_bits, up_bias, upA, upB, upS), dtype)
+        down = _Proj((down_qweight, down_scales, down_qzeros, down_g_idx, down_bits, down_bias, downA, downB, downS), dtype)
+        Xg = _apply_dropout(X2, dropout_gate) if gate.r else X2
+        Xu = _apply_dropout(X2, dropout_up) if up.r else X2
+        fused = gate.w.perm is None and up.w.perm is None
+        if fused:
+            Ug = fmsa_hip.lora_down(Xg, gate.A) if gate.r else None
+            Uu = fmsa_hip.lora_down(Xu, up.A) if up.r else None
+            e, g, h = fmsa_hip.gptq_lora_fwd(X2, [gate.fwd_dict(Ug), up.fwd_dict(Uu)], fmsa_hip.FWD_SWIGLU)
+        else:
+            (e, g), (Ug, Uu) = _linear_forward([gate, up], X2, [Xg, Xu])
+            h = fmsa_hip.swiglu_fwd(e, g)
+        hd = _apply_dropout(h, dropout_down) if down.r else h
+        (out,), (Ud,) = _linear_forward([down], h, [hd])
+        ctx.projs = (gate, up, down)
+        ctx.x_shape, ctx.x_dtype = X.shape, X.dtype
+        ctx.down_dropped = hd is not h
+        none = X2.new_empty(0)
+        ctx.save_for_backward(Xg, Xu, e, g, hd if ctx.down_dropped else none,
+                              Ug if gate.r else none, Uu if up.r else none, Ud if down.r else none)
+        return out.view(*X.shape[:-1], down.w.N)
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dY):
+        gate, up, down = ctx.projs
+        Xg, Xu, e, g, hd, Ug, Uu, Ud = ctx.saved_tensors
+        dY2 = _as2d(dY, e.dtype)
+        M, H, I = dY2.shape[0], gate.w.K, down.w.K
+
+        # ---- down projection: dh, then SwiGLU backward in place (e <- d_g, g <- d_e) -----------
+        Td = fmsa_hip.lora_down(dY2, _Bt(down)) if down.r else None
+        mask_h = hd if ctx.down_dropped else None
+        if down.w.perm is None:
+            h = fmsa_hip.gptq_lora_bwd_dx([down.bwd_dict(dY2, Td, mask_h)], M, I, fmsa_hip.BWD_SWIGLU, e=e, g=g)
+        else:
+            # un-fused epilogue for a repacked (act-order) weight: dh in kernel order, scatter back,
+            # then the standalone SwiGLU backward.  The mask of the LoRA part is (dropout(h) != 0).
+            h_now = fmsa_hip.swiglu_fwd(e, g)
+            dh = down.from_kernel_order(
+                fmsa_hip.gptq_lora_bwd_dx([down.bwd_dict(dY2, Td, mask_h if mask_h is not None else h_now)], M, I))
+            h = fmsa_hip.swiglu_bwd(dh, e, g)
+        d_g, d_e = e, g
+        dAd = dBd = None
+        if down.r:
+            # the reference forms both down-projection grads from the recomputed h (:369-370)
+            Ud_b = fmsa_hip.lora_down(h, down.A) if ctx.down_dropped else Ud
+            dAd, dBd = down.lora_grads(Td, h, Ud_b, dY2)
+
+        # ---- up / gate: adapter grads, then dX over the concatenated contraction ---------------
+        Tu = fmsa_hip.lora_down(d_g, _Bt(up)) if up.r else None
+        Tg = fmsa_hip.lora_down(d_e, _Bt(gate)) if gate.r else None
+        dAu, dBu = up.lora_grads(Tu, Xu, Uu, d_g)
+        dAg, dBg = gate.lora_grads(Tg, Xg, Ug, d_e)
+        dX = _linear_backward_dx([up, gate], [d_g, d_e], [Tu, Tg], [Xu, Xg], M, H)
+
+        n6 = (None,) * 6
+        return (
+            dX.view(ctx.x_shape).to(ctx.x_dtype),
+            *n6, dAg, dBg, None,
+            *n6, dAu, dBu, None,
+            *n6, dAd, dBd, None,
+            None, None, None,
+        )
+
+
+# ----------------------------------------------------------------------------------------------
+# module-level entry points (bound to modules with MethodType by the model patcher)
+# ----------------------------------------------------------------------------------------------
+def apply_lora_mlp(self, X):
+    gateQstate, gate_bias, gateA, gateB, gateS, dropout_gate = get_lora_parameters(self.gate_proj)
+    upQState, up_bias, upA, upB, upS, dropout_up = get_lora_parameters(self.up_proj)
+    downQState, down_bias, downA, downB, downS, dropout_down = get_lora_parameters(self.down_proj)
+    return LoRA_MLP.apply(
+        X,
+        *unpack_gptqstate(gateQstate), gate_bias, gateA, gateB, gateS,
+        *unpack_gptqstate(upQState), up_bias, upA, upB, upS,
+        *unpack_gptqstate(downQState), down_bias, downA, downB, downS,
+        dropout_gate, dropout_up, dropout_down,
+    )
+
+
+def apply_lora_qkv(self, X):
+    Qqstate, Q_bias, QA, QB, QS, Qdropout = get_lora_parameters(self.q_proj)
+    Kqstate, K_bias, KA, KB, KS, Kdropout = get_lora_parameters(self.k_proj)
+    Vqstate, V_bias, VA, VB, VS, Vdropout = get_lora_parameters(self.v_proj)
+    return LoRA_QKV.apply(
+        X,
+        *unpack_gptqstate(Qqstate), Q_bias, QA, QB, QS,
+        *unpack_gptqstate(Kqstate), K_bias, KA, KB, KS,
+        *unpack_gptqstate(Vqstate), V_bias, VA, VB, VS,
+        Qdropout, Kdropout, Vdropout,
+    )
+
+
+def apply_lora_o(self, X):
+    Oqstate, O_bias, OA, OB, OS, dropout = get_lora_parameters(self.o_proj)
+    return LoRA_W.apply(X, *unpack_gptqstate(Oqstate), O_bias, OA, OB, OS, dropout)
+
+
+def apply_lora_o_v2(self, X):
+    """Patched directly on the output linear (`self` is the LoRA layer itself, :856-859)."""
+    Oqstate, O_bias, OA, OB, OS, dropout = get_lora_parameters(self)
+    return LoRA_W.apply(X, *unpack_gptqstate(Oqstate), O_bias, OA, OB, OS, dropout)

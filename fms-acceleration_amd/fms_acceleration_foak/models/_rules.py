@@ -1,0 +1,57 @@
+"""Shared construction of the `<arch>-qkvo` / `<arch>-mlp` rules: the three dense architectures
+differ only in their attention / MLP classes (reference: models/llama.py:73-123, mistral.py:70-119,
+granite.py:78-128)."""
+from __future__ import annotations
+
+import warnings
+from functools import partial
+
+from fms_acceleration.model_patcher import (
+    ModelPatcherRule,
+    ModelPatcherTrigger,
+    combine_functions,
+    combine_triggers,
+)
+
+from ..utils import filter_mp_rules
+from .utils import KEY_MLP, KEY_O, KEY_QKV, build_lora_fused_ops, get_hidden_activation_fn_key, trigger_fused_ops
+
+QKV_NAMES = ["q_proj", "k_proj", "v_proj"]
+MLP_NAMES = ["up_proj", "down_proj", "gate_proj"]
+
+
+def fused_lora_rules(arch: str, attn_cls, mlp_cls, base_type: str, config=None, label: str = None):
+    rules = [
+        ModelPatcherRule(
+            rule_id=f"{arch}-qkvo",
+            trigger=combine_triggers(
+                ModelPatcherTrigger(check=partial(trigger_fused_ops, attn_cls=attn_cls, submodule_names=QKV_NAMES)),
+                ModelPatcherTrigger(check=partial(trigger_fused_ops, attn_cls=attn_cls, submodule_names=["o_proj"])),
+                logic="OR",
+            ),
+            forward_builder=combine_functions(
+                partial(build_lora_fused_ops, submodule_names=QKV_NAMES, fused_op=KEY_QKV, base_type=base_type),
+                partial(build_lora_fused_ops, submodule_names=["o_proj"], fused_op=KEY_O, base_type=base_type),
+                logic="APPEND",
+            ),
+        ),
+    ]
+    if mlp_cls is not None:
+        rules.append(
+            ModelPatcherRule(
+                rule_id=f"{arch}-mlp",
+                trigger=ModelPatcherTrigger(check=partial(trigger_fused_ops, attn_cls=mlp_cls, submodule_names=MLP_NAMES)),
+                forward_builder=partial(build_lora_fused_ops, submodule_names=MLP_NAMES, fused_op=KEY_MLP,
+                                        base_type=base_type),
+            )
+        )
+    # only SwiGLU is fused: any other activation drops the MLP rule (llama.py:164-172)
+    if config is not None and mlp_cls is not None:
+        act = get_hidden_activation_fn_key(config)
+        if act != "silu":
+            warnings.warn(
+                f"{label or arch}Rules: activation is {act}, thus disabling LoRA fused-op for MLP, since only "
+                "SwiGLU is supported. This only affects quantized-peft."
+            )
+            rules = filter_mp_rules(rules, {"mlp"}, drop=True)
+    return rules

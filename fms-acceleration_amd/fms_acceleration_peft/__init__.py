@@ -1,0 +1,5 @@
+"""Namesake of `fms_acceleration_peft`: the quantised base-layer data layouts (GPTQ QuantLinear,
+NF4 container), a stand-in LoRA wrapper, and the plugin configuration shells."""
+from .framework_plugin_autogptq import AutoGPTQAccelerationPlugin
+from .lora import LoraLinear
+from .qlinear import QuantLinear, QuantLinearFunction

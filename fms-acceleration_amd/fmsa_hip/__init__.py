@@ -33,6 +33,8 @@ EXPORTED_SYMBOLS = (
     "fmsa_lora_grad",
     "fmsa_gptq_lora_fwd",
     "fmsa_gptq_lora_bwd_dx",
+    "fmsa_swiglu_fwd",
+    "fmsa_swiglu_bwd",
 )
 
 
@@ -105,6 +107,8 @@ def lib() -> ctypes.CDLL:
                                      c_int, c_void_p]
     L.fmsa_gptq_lora_bwd_dx.argtypes = [POINTER(BwdProj), c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p,
                                         c_void_p, c_int64, c_int, c_void_p]
+    L.fmsa_swiglu_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
+    L.fmsa_swiglu_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
     for name in EXPORTED_SYMBOLS:
         getattr(L, name)  # AttributeError here means the library is stale: rebuild it
     _lib = L
@@ -260,3 +264,22 @@ def gptq_lora_bwd_dx(projs: Sequence[dict], M: int, K: int, mode: int = BWD_LINE
            lib().fmsa_gptq_lora_bwd_dx(arr, len(projs), M, mode, _ptr(dx), dx.stride(0), None, None, None, 0,
                                        act_enum(ref.dtype), _stream(ref)))
     return dx
+
+
+def swiglu_fwd(e, g):
+    """h = silu(e) * g with the reference's rounding points (standalone kernel)."""
+    M, I = e.shape
+    assert e.stride() == g.stride() and e.stride(1) == 1
+    h = torch.empty_like(e)
+    _check("fmsa_swiglu_fwd", lib().fmsa_swiglu_fwd(_ptr(e), _ptr(g), _ptr(h), M, I, e.stride(0), act_enum(e.dtype), _stream(e)))
+    return h
+
+
+def swiglu_bwd(dh, e, g):
+    """In place: e <- d_g, g <- d_e; returns h."""
+    M, I = e.shape
+    assert e.stride() == g.stride() and e.stride(1) == 1 and dh.stride(1) == 1
+    h = torch.empty_like(e)
+    _check("fmsa_swiglu_bwd", lib().fmsa_swiglu_bwd(_ptr(dh), dh.stride(0), _ptr(e), _ptr(g), _ptr(h), M, I, e.stride(0),
+                                                    act_enum(e.dtype), _stream(e)))
+    return h

@@ -156,6 +156,17 @@ int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs /*host*/, int n_proj, int M
                           void* dX, int64_t lddx, void* e, void* g, void* h_out, int64_t ldeg,
                           int act_dtype, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Standalone SwiGLU (UL/swiglu.py:20-47 and :50-98) for the paths whose GEMM epilogue cannot
+ * fuse it.  e, g, h share the leading dimension ld; I % 8 == 0.
+ *   fwd: h = RNE(silu_f32(e)) * g
+ *   bwd: in place, h_out <- f*g, e <- d_g = dh*f, g <- d_e = RNE(f32(dh*g) * s(e) * (1 + e(1 - s(e))))
+ * ------------------------------------------------------------------------------------------ */
+int fmsa_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype,
+                    void* stream);
+int fmsa_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h_out, int M, int I,
+                    int64_t ld, int act_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

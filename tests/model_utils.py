@@ -1,0 +1,41 @@
+"""Builders of small GPTQ + LoRA modules for the module-level tests."""
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from oracle import lora as olora
+from tests.helpers import make_gptq
+
+
+class MaskDropout(nn.Module):
+    """Deterministic stand-in for nn.Dropout: multiplies by a fixed 0/1 mask, no 1/(1-p) rescale
+    (the reference's test double, plugins/fused-ops-and-kernels/tests/test_fused_ops.py:68-83)."""
+
+    def __init__(self, p, shape, seed=0):
+        super().__init__()
+        gen = torch.Generator().manual_seed(seed)
+        self.register_buffer("mask", (torch.rand(shape, generator=gen) >= p).float())
+
+    def forward(self, x):
+        return x * self.mask.to(x.dtype).reshape(x.shape)
+
+
+def make_lora_gptq_linear(K, N, r, alpha, seed, group_size=128, act_order=False, bias=False, device="cpu",
+                          lora_dtype=torch.float32, dropout=None):
+    """LoraLinear(QuantLinear) with seeded weights.  Returns (module, dense fp32 W [K, N], A, B)."""
+    from fms_acceleration_peft import LoraLinear, QuantLinear
+
+    w = make_gptq(K, N, group_size, seed=seed, act_order=act_order)
+    ql = QuantLinear(4, w["group_size"], K, N, bias)
+    ql.load_packed(w["np"]["qweight"], w["np"]["qzeros"], w["np"]["scales"], w["np"]["g_idx"])
+    if bias:
+        gen = torch.Generator().manual_seed(seed + 77)
+        ql.bias.copy_((torch.randn(N, generator=gen) * 0.1).half())
+    lin = LoraLinear(ql, r, alpha, dtype=lora_dtype)
+    A, B = olora.make_lora(K, N, r, seed + 1)
+    lin.lora_A["default"].weight.data.copy_(A)
+    lin.lora_B["default"].weight.data.copy_(B)
+    if dropout is not None:
+        lin.lora_dropout["default"] = dropout
+    return lin.to(device), w["dense"], A, B
