@@ -33,9 +33,9 @@ int check_weight(const fmsa_gptq_weight* w, int group_multiple) {
   if (!aligned16(w->qweight) || !aligned16(w->scales) || !aligned16(w->qzeros)) return FMSA_ERR_ALIGN;
   if (group_multiple > 0) {
     // The fused kernels assume the group of row k is k / group_size: act-order weights must be
-    // repacked with fmsa_gptq_permute_rows first.  The forward reads scale/zero once per 64-wide
-    // K stage (group_size % 64 == 0); the input-gradient kernel needs one group per packed
-    // qweight row (group_size % 8 == 0).
+    // repacked with fmsa_gptq_permute_rows first.  The forward needs one group per 16-wide MFMA
+    // K step (group_size % 16 == 0); the input-gradient kernel one group per packed qweight row
+    // (group_size % 8 == 0).
     if (w->g_idx) return FMSA_ERR_UNSUPPORTED;
     if (w->group_size % group_multiple != 0) return FMSA_ERR_UNSUPPORTED;
   }
@@ -133,7 +133,7 @@ int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, in
   if (!aligned16(X) || ldx % 8 != 0) return FMSA_ERR_ALIGN;
   for (int p = 0; p < n_proj; ++p) {
     const fmsa_fwd_proj& s = projs[p];
-    if (int rc = check_weight(&s.w, 64)) return rc;
+    if (int rc = check_weight(&s.w, 16)) return rc;
     if (s.w.K != K) return FMSA_ERR_SHAPE;
     if (!s.Y) return FMSA_ERR_NULL;
     if (s.ldy < s.w.N) return FMSA_ERR_SHAPE;

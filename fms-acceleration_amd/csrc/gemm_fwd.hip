@@ -51,7 +51,8 @@ struct FwdArgs {
 // which would force a copy of it into scratch memory.
 FMSA_DEVI FwdProjDev select_proj(const FwdArgs& a, int p) { return p == 0 ? a.p[0] : (p == 1 ? a.p[1] : a.p[2]); }
 
-template <typename T>
+// GPS = scale groups per 64-wide K stage: 1 for group_size % 64 == 0, 2 / 4 for group sizes 32 / 16.
+template <typename T, int GPS>
 __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t lds[2][BM * LDS_STRIDE];
 
@@ -122,10 +123,10 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 
   u32x4 a_st[8];        // X staging: 8 x 16 B per lane per stage
   uint32_t q_cur[NT][4], q_nxt[NT][4];
-  float sf[NT], nsz[NT];
+  float sf[NT][GPS], nsz[NT][GPS];
   int g_cur[NT];
-  uint16_t sc_nxt[NT];
-  uint32_t zw_nxt[NT];
+  uint16_t sc_nxt[NT][GPS];
+  uint32_t zw_nxt[NT][GPS];
   bool g_changed[NT];
 
   auto load_stage = [&](int k0) {
@@ -146,10 +147,15 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
         q_nxt[j][t] = (8 * k8 < K) ? (uint32_t)qwp[j][(size_t)k8 * Np[j]] : 0u;
       }
       const int g = k0 / gs[j];
-      g_changed[j] = (g != g_cur[j]);
+      g_changed[j] = (GPS > 1) || (g != g_cur[j]);
       if (g_changed[j]) {
-        sc_nxt[j] = scp[j][(size_t)g * Np[j]];
-        zw_nxt[j] = (uint32_t)zp[j][(size_t)g * (Np[j] >> 3)];
+#pragma unroll
+        for (int u = 0; u < GPS; ++u) {
+          const int ku = k0 + u * (BK / GPS);
+          const int gu = (ku < K ? ku : k0) / gs[j];
+          sc_nxt[j][u] = scp[j][(size_t)gu * Np[j]];
+          zw_nxt[j][u] = (uint32_t)zp[j][(size_t)gu * (Np[j] >> 3)];
+        }
         g_cur[j] = g;
       }
     }
@@ -166,9 +172,12 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) q_cur[j][t] = q_nxt[j][t];
       if (g_changed[j]) {
-        sf[j] = fp16_bits_to_f32(sc_nxt[j]);
-        const float z = (float)((zw_nxt[j] >> zshift[j]) & 0xFu) + zoff[j];
-        nsz[j] = -sf[j] * z;  // exact: 11-bit x 5-bit
+#pragma unroll
+        for (int u = 0; u < GPS; ++u) {
+          sf[j][u] = fp16_bits_to_f32(sc_nxt[j][u]);
+          const float z = (float)((zw_nxt[j][u] >> zshift[j]) & 0xFu) + zoff[j];
+          nsz[j][u] = -sf[j][u] * z;  // exact: 11-bit x 5-bit
+        }
       }
     }
   };
@@ -187,7 +196,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     for (int t = 0; t < 4; ++t) {
       u32x4 wf[NT];
 #pragma unroll
-      for (int j = 0; j < NT; ++j) wf[j] = dequant8<T>(q_cur[j][t], sf[j], nsz[j]);
+      for (int j = 0; j < NT; ++j) wf[j] = dequant8<T>(q_cur[j][t], sf[j][t * GPS / 4], nsz[j][t * GPS / 4]);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         const u32x4 xf =
@@ -317,10 +326,22 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
   a.nbn = nb;
   a.nbm = (M + BM - 1) / BM;
   dim3 grid(a.nbm * a.nbn), block(256);
+  int gps = 1;
+  for (int p = 0; p < n_proj; ++p) {
+    const int gsz = projs[p].w.group_size;
+    if (gsz % 64 != 0) gps = (gsz % 32 == 0) ? (gps > 2 ? gps : 2) : 4;
+  }
+#define LAUNCH(TT)                                                                          \
+  do {                                                                                      \
+    if (gps == 1) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1>), grid, block, 0, st, a); \
+    else if (gps == 2) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 2>), grid, block, 0, st, a); \
+    else hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 4>), grid, block, 0, st, a);          \
+  } while (0)
   if (act_dtype == FMSA_BF16)
-    hipLaunchKernelGGL(gptq_lora_fwd_kernel<bf16_t>, grid, block, 0, st, a);
+    LAUNCH(bf16_t);
   else
-    hipLaunchKernelGGL(gptq_lora_fwd_kernel<f16_t>, grid, block, 0, st, a);
+    LAUNCH(f16_t);
+#undef LAUNCH
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }

@@ -170,3 +170,20 @@ def act_order_g_idx(K: int, group_size: int, seed: int = 4) -> np.ndarray:
     g = np.empty(K, dtype=np.int32)
     g[perm] = (np.arange(K) // group_size).astype(np.int32)
     return g
+
+
+def dequant_torch(qweight, scales, qzeros, g_idx, zero_offset: int = 0):
+    """The reference's pure-torch `dequant_ref` (UL/gptq/triton/kernels.py:15-40) restated: shift /
+    mask unpack of qzeros and qweight, then scales[g_idx] * (q - zeros[g_idx]).  `dequant_ref` adds 1
+    to the zeros unconditionally (v1 checkpoints); here that is `zero_offset`.  Returns fp32 [K, N].
+    Multi-threaded through torch: this is the dequant step of the CPU baseline."""
+    import torch
+
+    qweight, scales, qzeros, g_idx = (torch.as_tensor(t) for t in (qweight, scales, qzeros, g_idx))
+    wf = torch.arange(0, 32, BITS, dtype=torch.int32)
+    zeros = torch.bitwise_and(torch.bitwise_right_shift(qzeros.unsqueeze(2).expand(-1, -1, PF), wf.view(1, 1, -1)), MAXQ)
+    zeros = (zeros + zero_offset).reshape(scales.shape)
+    weights = torch.bitwise_and(torch.bitwise_right_shift(qweight.unsqueeze(1).expand(-1, PF, -1), wf.view(1, -1, 1)), MAXQ)
+    weights = weights.reshape(-1, weights.shape[2])
+    g = g_idx.long()
+    return scales.float()[g] * (weights - zeros[g]).float()
