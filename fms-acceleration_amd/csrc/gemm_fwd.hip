@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
       col0[j] = (bn - a.nblk_start[p]) * 256 + wave * 64 + j * 32;
     }
   }
-  const int32_t* qwp[NT];
+  const char* qbase[NT];
   const uint16_t* scp[NT];
   const int32_t* zp[NT];
   int Np[NT], zshift[NT], gs[NT];
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     const int col = col0[j] + l32;
     Np[j] = P.N;
     gs[j] = P.group_size;
-    qwp[j] = P.qweight + col;
+    qbase[j] = reinterpret_cast<const char*>(P.qweight);
     scp[j] = P.scales + col;
     zp[j] = P.qzeros + (col >> 3);
     zshift[j] = 4 * (col & 7);
@@ -121,92 +121,139 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
 
+  // ---- operand addressing: uniform 64-bit base + 32-bit per-lane byte offset --------------------
+  // X tile: lane owns chunk (row = tid/8 + 32*i, oct = tid%8), i = 0..7.  Rows past M are clamped to
+  // the last valid row (their results are never stored), so the loads need no predication.
+  uint32_t x_off[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = min(m0 + (tid >> 3) + 32 * i, a.M - 1) - m0;
+    x_off[i] = (uint32_t)(((int64_t)row * a.ldx) * 2);
+  }
+  const char* x_base = reinterpret_cast<const char*>(a.X) + (size_t)m0 * a.ldx * 2;
+  const int oct = tid & 7;
+  const uint32_t lds_w_off = (uint32_t)(((tid >> 3) * LDS_STRIDE + oct * 8) * 2);
+  const uint32_t lds_r_off = (uint32_t)((l32 * LDS_STRIDE + 8 * half) * 2);
+  uint32_t q_off[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) q_off[j] = (uint32_t)(((int64_t)half * Np[j] + col0[j] + l32) * 4);
+  const int k8_last = (K >> 3) - 1;
+
   u32x4 a_st[8];        // X staging: 8 x 16 B per lane per stage
   uint32_t q_cur[NT][4], q_nxt[NT][4];
   float sf[NT][GPS], nsz[NT][GPS];
-  int g_cur[NT];
   uint16_t sc_nxt[NT][GPS];
   uint32_t zw_nxt[NT][GPS];
-  bool g_changed[NT];
 
-  auto load_stage = [&](int k0) {
+  // issue the global loads of stage `st` (clamped to the last stage: the surplus loads of the final
+  // iterations re-read valid data and are never used)
+  auto load_stage = [&](int st) {
+    const int k0 = min(st, n_stages - 1) * BK;
+    const int gk = k0 + 8 * oct;
+    const bool k_ok = gk < K;
+    const char* xb = x_base + (size_t)(k_ok ? gk : (K - 8)) * 2;
+    // nothing may touch the loaded registers here: any use would make the wave wait for the load
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c >> 3, oct = c & 7;
-      const int gm = m0 + row, gk = k0 + 8 * oct;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (gm < a.M && gk < K) v = *reinterpret_cast<const u32x4*>(a.X + (size_t)gm * a.ldx + gk);
-      a_st[i] = v;
-    }
+    for (int i = 0; i < 8; ++i) a_st[i] = *reinterpret_cast<const u32x4*>(xb + x_off[i]);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const int k8 = (k0 >> 3) + 2 * t + half;
-        q_nxt[j][t] = (8 * k8 < K) ? (uint32_t)qwp[j][(size_t)k8 * Np[j]] : 0u;
+        const int k8u = min((k0 >> 3) + 2 * t, k8_last - 1);  // uniform part; + half per lane
+        q_nxt[j][t] = *reinterpret_cast<const uint32_t*>(qbase[j] + (size_t)k8u * Np[j] * 4 + q_off[j]);
       }
-      const int g = k0 / gs[j];
-      g_changed[j] = (GPS > 1) || (g != g_cur[j]);
-      if (g_changed[j]) {
 #pragma unroll
-        for (int u = 0; u < GPS; ++u) {
-          const int ku = k0 + u * (BK / GPS);
-          const int gu = (ku < K ? ku : k0) / gs[j];
-          sc_nxt[j][u] = scp[j][(size_t)gu * Np[j]];
-          zw_nxt[j][u] = (uint32_t)zp[j][(size_t)gu * (Np[j] >> 3)];
-        }
-        g_cur[j] = g;
+      for (int u = 0; u < GPS; ++u) {
+        const int ku = k0 + u * (BK / GPS);
+        const int gu = (ku < K ? ku : k0) / gs[j];
+        sc_nxt[j][u] = scp[j][(size_t)gu * Np[j]];
+        zw_nxt[j][u] = (uint32_t)zp[j][(size_t)gu * (Np[j] >> 3)];
       }
     }
   };
-  auto commit_stage = [&](int buf) {
+  // registers -> LDS buffer `buf`, and make the prefetched weight words / scales current
+  auto commit_stage = [&](int buf, int st) {
+    char* lw = reinterpret_cast<char*>(lds[buf]) + lds_w_off;
+    const bool k_ok = (min(st, n_stages - 1) * BK + 8 * oct) < K;  // K tail: zero columns past K
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c >> 3, oct = c & 7;
-      *reinterpret_cast<u32x4*>(&lds[buf][row * LDS_STRIDE + oct * 8]) = a_st[i];
-    }
+    for (int i = 0; i < 8; ++i)
+      *reinterpret_cast<u32x4*>(lw + i * 32 * LDS_STRIDE * 2) = k_ok ? a_st[i] : u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) q_cur[j][t] = q_nxt[j][t];
-      if (g_changed[j]) {
 #pragma unroll
-        for (int u = 0; u < GPS; ++u) {
-          sf[j][u] = fp16_bits_to_f32(sc_nxt[j][u]);
-          const float z = (float)((zw_nxt[j][u] >> zshift[j]) & 0xFu) + zoff[j];
-          nsz[j][u] = -sf[j][u] * z;  // exact: 11-bit x 5-bit
-        }
+      for (int u = 0; u < GPS; ++u) {
+        sf[j][u] = fp16_bits_to_f32(sc_nxt[j][u]);
+        const float z = (float)((zw_nxt[j][u] >> zshift[j]) & 0xFu) + zoff[j];
+        nsz[j][u] = -sf[j][u] * z;  // exact: 11-bit x 5-bit
       }
     }
   };
 
+  // Software pipeline at the granularity of one 16-wide MFMA K step: while the 16 MFMAs of step t
+  // run, the 8 X fragments of step t+1 are read from LDS and its 2 weight fragments are unpacked,
+  // into the other half of xf / wf.  The stage barrier sits after step 2, so step 3 can already
+  // fetch step 0 of the next stage from the other LDS buffer.
+  u32x4 xf[2][MT], wf[2][NT];
+  auto prefetch = [&](int buf, int t, auto par_c) {
+    constexpr int par = decltype(par_c)::value;
+    const char* lr = reinterpret_cast<const char*>(lds[buf]) + lds_r_off + t * 32;
 #pragma unroll
-  for (int j = 0; j < NT; ++j) g_cur[j] = -1;
+    for (int mt = 0; mt < MT; ++mt)
+      xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * LDS_STRIDE * 2);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) wf[par][j] = dequant8<T>(q_cur[j][t], sf[j][t * GPS / 4], nsz[j][t * GPS / 4]);
+  };
+  auto mfma_step = [&](auto par_c) {
+    constexpr int par = decltype(par_c)::value;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[par][j], xf[par][mt], acc[mt][j]);
+  };
+  // interleave: 1 MFMA, 3 VALU, and an LDS read after every second MFMA
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+      if ((i & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // nothing from the next step (or the stage hand-over) moves up
+  };
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+
   load_stage(0);
-  commit_stage(0);
+  commit_stage(0, 0);
   __syncthreads();
+  prefetch(0, 0, P0{});
 
   for (int s = 0; s < n_stages; ++s) {
     const int buf = s & 1;
-    if (s + 1 < n_stages) load_stage((s + 1) * BK);
-    const uint16_t* lb = lds[buf];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      u32x4 wf[NT];
-#pragma unroll
-      for (int j = 0; j < NT; ++j) wf[j] = dequant8<T>(q_cur[j][t], sf[j][t * GPS / 4], nsz[j][t * GPS / 4]);
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const u32x4 xf =
-            *reinterpret_cast<const u32x4*>(&lb[(32 * mt + l32) * LDS_STRIDE + 16 * t + 8 * half]);
-#pragma unroll
-        for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[j], xf, acc[mt][j]);
-      }
-    }
-    if (s + 1 < n_stages) commit_stage(buf ^ 1);
+    // Global loads of the next stage are issued and consumed inside one iteration (steps 0-2 hide
+    // their latency): a load that stayed in flight across the loop back-edge would be waited for
+    // at the back-edge, where the compiler copies loop-carried registers.
+    load_stage(s + 1);
+    // step 0
+    prefetch(buf, 1, P1{});
+    mfma_step(P0{});
+    interleave();
+    // step 1
+    prefetch(buf, 2, P0{});
+    mfma_step(P1{});
+    interleave();
+    // step 2, then hand the next stage over
+    prefetch(buf, 3, P1{});
+    mfma_step(P0{});
+    interleave();
+    commit_stage(buf ^ 1, s + 1);
     __syncthreads();
+    // step 3
+    prefetch(buf ^ 1, 0, P0{});
+    mfma_step(P1{});
+    interleave();
   }
 
   // ---- epilogue ---------------------------------------------------------------------------
