@@ -36,18 +36,17 @@ FMSA_DEVI float fp16_bits_to_f32(uint16_t h) {
 }
 FMSA_DEVI float bf16_bits_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
 
-// Two fp32 -> packed storage type, RNE, low half = a.
+// Two fp32 -> packed storage type, RNE, low half = a.  Written as vector conversions so that the
+// compiler selects v_cvt_pk_bf16_f32 / v_cvt_f16_f32 itself and can schedule around them.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 template <typename T> FMSA_DEVI uint32_t pack2(float a, float b);
 template <> FMSA_DEVI uint32_t pack2<bf16_t>(float a, float b) {
-  uint32_t r;
-  asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){a, b}, bf16x2));
 }
 template <> FMSA_DEVI uint32_t pack2<f16_t>(float a, float b) {
-  union { f16_t h[2]; uint32_t u; } c;
-  c.h[0] = (f16_t)a;  // v_cvt_f16_f32 is RNE under the default mode
-  c.h[1] = (f16_t)b;
-  return c.u;
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){a, b}, f16x2));
 }
 template <typename T> FMSA_DEVI uint16_t pack1(float a) { return (uint16_t)(pack2<T>(a, 0.f) & 0xffffu); }
 
@@ -59,25 +58,32 @@ template <> FMSA_DEVI float unpack_lo<f16_t>(uint32_t v) { return fp16_bits_to_f
 template <> FMSA_DEVI float unpack_hi<f16_t>(uint32_t v) { return fp16_bits_to_f32((uint16_t)(v >> 16)); }
 template <typename T> FMSA_DEVI float unpack1(uint16_t v) { return unpack_lo<T>((uint32_t)v); }
 
-// byte j of x as fp32 (one VALU op each)
-FMSA_DEVI float ubyte0(uint32_t x) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(x)); return r; }
-FMSA_DEVI float ubyte1(uint32_t x) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(x)); return r; }
-FMSA_DEVI float ubyte2(uint32_t x) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(x)); return r; }
-FMSA_DEVI float ubyte3(uint32_t x) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(x)); return r; }
+// byte j of x as fp32: the shift-and-mask form is what the compiler turns into v_cvt_f32_ubyte<j>
+FMSA_DEVI float ubyte0(uint32_t x) { return (float)(x & 0xffu); }
+FMSA_DEVI float ubyte1(uint32_t x) { return (float)((x >> 8) & 0xffu); }
+FMSA_DEVI float ubyte2(uint32_t x) { return (float)((x >> 16) & 0xffu); }
+FMSA_DEVI float ubyte3(uint32_t x) { return (float)(x >> 24); }
+// Stops the optimiser from narrowing the byte masks above back into nibble masks (which would
+// cost a shift + and + convert per value instead of one convert).  Emits no instruction.
+FMSA_DEVI uint32_t opaque(uint32_t x) {
+  asm("" : "+v"(x));
+  return x;
+}
 
 // ---- GPTQ: eight nibbles of one int32 -> eight storage-type values --------------------------
 // value_j = RNE( sf * nib_j + nsz ) with nsz = -sf * (z + zero_offset).  sf is an fp16 scale
 // widened to fp32 (11 significant bits) and nib, z are < 32, so sf*nib, nsz and their sum are
 // all exact in fp32: the only rounding is the final conversion, as in
-// UL/gptq/triton/kernels.py:118-122.
-template <typename T> FMSA_DEVI u32x4 dequant8(uint32_t w, float sf, float nsz) {
-  const uint32_t lo = w & 0x0F0F0F0Fu;         // nibbles 0,2,4,6 in bytes 0..3
-  const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;  // nibbles 1,3,5,7
+// UL/gptq/triton/kernels.py:118-122.  The odd nibbles are used in place (16 * nib in the high
+// half of each byte) with the scale pre-divided by 16 -- a power of two, so still exact.
+template <typename T> FMSA_DEVI u32x4 dequant8(uint32_t w, float sf, float sf16, float nsz) {
+  const uint32_t lo = opaque(w & 0x0F0F0F0Fu);  // nibbles 0,2,4,6 in bytes 0..3
+  const uint32_t hi = opaque(w & 0xF0F0F0F0u);  // 16 * nibbles 1,3,5,7
   u32x4 r;
-  r[0] = pack2<T>(__builtin_fmaf(sf, ubyte0(lo), nsz), __builtin_fmaf(sf, ubyte0(hi), nsz));
-  r[1] = pack2<T>(__builtin_fmaf(sf, ubyte1(lo), nsz), __builtin_fmaf(sf, ubyte1(hi), nsz));
-  r[2] = pack2<T>(__builtin_fmaf(sf, ubyte2(lo), nsz), __builtin_fmaf(sf, ubyte2(hi), nsz));
-  r[3] = pack2<T>(__builtin_fmaf(sf, ubyte3(lo), nsz), __builtin_fmaf(sf, ubyte3(hi), nsz));
+  r[0] = pack2<T>(__builtin_fmaf(sf, ubyte0(lo), nsz), __builtin_fmaf(sf16, ubyte0(hi), nsz));
+  r[1] = pack2<T>(__builtin_fmaf(sf, ubyte1(lo), nsz), __builtin_fmaf(sf16, ubyte1(hi), nsz));
+  r[2] = pack2<T>(__builtin_fmaf(sf, ubyte2(lo), nsz), __builtin_fmaf(sf16, ubyte2(hi), nsz));
+  r[3] = pack2<T>(__builtin_fmaf(sf, ubyte3(lo), nsz), __builtin_fmaf(sf16, ubyte3(hi), nsz));
   return r;
 }
 
@@ -100,6 +106,14 @@ template <> FMSA_DEVI f32x4 mfma16<bf16_t>(u32x4 a, u32x4 b, f32x4 c) {
 }
 template <> FMSA_DEVI f32x4 mfma16<f16_t>(u32x4 a, u32x4 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// ---- buffer resources ----------------------------------------------------------------------------
+// Raw buffer descriptor over [base, base + bytes): loads through it take a 32-bit per-lane offset
+// plus a scalar offset, and a lane offset at or past `bytes` returns zero instead of faulting.
+FMSA_DEVI __amdgpu_buffer_rsrc_t make_rsrc(const void* base, size_t bytes) {
+  const uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
 }
 
 // ---- workgroup-id remap: consecutive ids land on different XCDs (id % 8), each with its own

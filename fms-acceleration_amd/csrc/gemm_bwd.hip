@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     for (int t = 0; t < 4; ++t) {
       // per-column scale and -scale*zero for the lane's 8 columns
       float sfv[8], nszv[8];
-      const uint32_t zlo = zwc[t] & 0x0F0F0F0Fu, zhi = (zwc[t] >> 4) & 0x0F0F0F0Fu;
+      const uint32_t zlo = opaque(zwc[t] & 0x0F0F0F0Fu), zhi = opaque((zwc[t] >> 4) & 0x0F0F0F0Fu);
       const float zf[8] = {ubyte0(zlo), ubyte0(zhi), ubyte1(zlo), ubyte1(zhi),
                            ubyte2(zlo), ubyte2(zhi), ubyte3(zlo), ubyte3(zhi)};
 #pragma unroll
@@ -194,8 +194,8 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       }
       u32x4 wf[NT];
       {
-        const uint32_t lo0 = qc[t][0] & 0x0F0F0F0Fu, hi0 = (qc[t][0] >> 4) & 0x0F0F0F0Fu;
-        const uint32_t lo1 = qc[t][1] & 0x0F0F0F0Fu, hi1 = (qc[t][1] >> 4) & 0x0F0F0F0Fu;
+        const uint32_t lo0 = opaque(qc[t][0] & 0x0F0F0F0Fu), hi0 = opaque((qc[t][0] >> 4) & 0x0F0F0F0Fu);
+        const uint32_t lo1 = opaque(qc[t][1] & 0x0F0F0F0Fu), hi1 = opaque((qc[t][1] >> 4) & 0x0F0F0F0Fu);
         // tile 0 = low nibble (k = 8*k8 + 2*wave), tile 1 = high nibble (k + 1); element i <-> column n+i
         wf[0][0] = pack2<T>(__builtin_fmaf(sfv[0], ubyte0(lo0), nszv[0]), __builtin_fmaf(sfv[1], ubyte1(lo0), nszv[1]));
         wf[0][1] = pack2<T>(__builtin_fmaf(sfv[2], ubyte2(lo0), nszv[2]), __builtin_fmaf(sfv[3], ubyte3(lo0), nszv[3]));

@@ -52,7 +52,7 @@ struct FwdArgs {
 FMSA_DEVI FwdProjDev select_proj(const FwdArgs& a, int p) { return p == 0 ? a.p[0] : (p == 1 ? a.p[1] : a.p[2]); }
 
 // GPS = scale groups per 64-wide K stage: 1 for group_size % 64 == 0, 2 / 4 for group sizes 32 / 16.
-template <typename T, int GPS>
+template <typename T, int GPS, bool KTAIL>
 __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t lds[2][BM * LDS_STRIDE];
 
@@ -91,8 +91,8 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     }
   }
   const char* qbase[NT];
-  const uint16_t* scp[NT];
-  const int32_t* zp[NT];
+  const char* scbase[NT];
+  const char* zbase[NT];
   int Np[NT], zshift[NT], gs[NT];
   float zoff[NT];
 #pragma unroll
@@ -101,11 +101,12 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     active[j] = col0[j] < P.N;
     if (!active[j]) col0[j] = 0;
     const int col = col0[j] + l32;
-    Np[j] = P.N;
-    gs[j] = P.group_size;
+    // wave-uniform by construction; readfirstlane tells the compiler so (scalar offsets below)
+    Np[j] = __builtin_amdgcn_readfirstlane(P.N);
+    gs[j] = __builtin_amdgcn_readfirstlane(P.group_size);
     qbase[j] = reinterpret_cast<const char*>(P.qweight);
-    scp[j] = P.scales + col;
-    zp[j] = P.qzeros + (col >> 3);
+    scbase[j] = reinterpret_cast<const char*>(P.scales);
+    zbase[j] = reinterpret_cast<const char*>(P.qzeros);
     zshift[j] = 4 * (col & 7);
     zoff[j] = (float)P.zero_offset;
   }
@@ -121,63 +122,91 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
 
-  // ---- operand addressing: uniform 64-bit base + 32-bit per-lane byte offset --------------------
-  // X tile: lane owns chunk (row = tid/8 + 32*i, oct = tid%8), i = 0..7.  Rows past M are clamped to
-  // the last valid row (their results are never stored), so the loads need no predication.
+  // ---- operand addressing: buffer loads (SGPR resource + 32-bit lane offset + SGPR offset) -----
+  // No 64-bit address arithmetic in the loop, and lanes whose offset falls outside the resource
+  // read zeros: rows past M need no predication.
+  // X tile: lane owns chunk (row = tid/8 + 32*i, oct = tid%8), i = 0..7.
+  const int oct = tid & 7;
+  const int rows_valid = min(BM, a.M - m0);
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(a.X + (size_t)m0 * a.ldx, (size_t)rows_valid * a.ldx * 2);
   uint32_t x_off[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = min(m0 + (tid >> 3) + 32 * i, a.M - 1) - m0;
-    x_off[i] = (uint32_t)(((int64_t)row * a.ldx) * 2);
-  }
-  const char* x_base = reinterpret_cast<const char*>(a.X) + (size_t)m0 * a.ldx * 2;
-  const int oct = tid & 7;
+  for (int i = 0; i < 8; ++i) x_off[i] = (uint32_t)((((tid >> 3) + 32 * i) * a.ldx + 8 * oct) * 2);
   const uint32_t lds_w_off = (uint32_t)(((tid >> 3) * LDS_STRIDE + oct * 8) * 2);
   const uint32_t lds_r_off = (uint32_t)((l32 * LDS_STRIDE + 8 * half) * 2);
-  uint32_t q_off[NT];
+  // weights: word (k8, col) at k8*N*4 + col*4; the lane part is (half*N + col)*4
+  __amdgpu_buffer_rsrc_t q_rsrc[NT], sc_rsrc[NT], z_rsrc[NT];
+  uint32_t q_off[NT], sc_off[NT], z_off[NT];
+  uint32_t q_stage_bytes[NT], q_step_bytes[NT], q_last[NT];
 #pragma unroll
-  for (int j = 0; j < NT; ++j) q_off[j] = (uint32_t)(((int64_t)half * Np[j] + col0[j] + l32) * 4);
-  const int k8_last = (K >> 3) - 1;
+  for (int j = 0; j < NT; ++j) {
+    const int n_groups = (K + gs[j] - 1) / gs[j];
+    q_rsrc[j] = make_rsrc(qbase[j], (size_t)(K >> 3) * Np[j] * 4);
+    sc_rsrc[j] = make_rsrc(scbase[j], (size_t)n_groups * Np[j] * 2);
+    z_rsrc[j] = make_rsrc(zbase[j], (size_t)n_groups * (Np[j] >> 3) * 4);
+    q_off[j] = (uint32_t)((half * Np[j] + col0[j] + l32) * 4);
+    sc_off[j] = (uint32_t)((col0[j] + l32) * 2);
+    z_off[j] = (uint32_t)(((col0[j] + l32) >> 3) * 4);
+    q_step_bytes[j] = (uint32_t)Np[j] * 8;    // two packed rows per 16-wide K step
+    q_stage_bytes[j] = (uint32_t)Np[j] * 32;  // eight packed rows per stage
+    q_last[j] = (uint32_t)((K >> 3) - 2) * Np[j] * 4;
+  }
 
   u32x4 a_st[8];        // X staging: 8 x 16 B per lane per stage
   uint32_t q_cur[NT][4], q_nxt[NT][4];
-  float sf[NT][GPS], nsz[NT][GPS];
+  float sf[NT][GPS], sf16[NT][GPS], nsz[NT][GPS];
   uint16_t sc_nxt[NT][GPS];
   uint32_t zw_nxt[NT][GPS];
-
-  // issue the global loads of stage `st` (clamped to the last stage: the surplus loads of the final
-  // iterations re-read valid data and are never used)
-  auto load_stage = [&](int st) {
-    const int k0 = min(st, n_stages - 1) * BK;
-    const int gk = k0 + 8 * oct;
-    const bool k_ok = gk < K;
-    const char* xb = x_base + (size_t)(k_ok ? gk : (K - 8)) * 2;
-    // nothing may touch the loaded registers here: any use would make the wave wait for the load
+  // group index of the stage being loaded, advanced without a division when GPS == 1
+  int g_ld[NT], k_in_g[NT];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) a_st[i] = *reinterpret_cast<const u32x4*>(xb + x_off[i]);
+  for (int j = 0; j < NT; ++j) g_ld[j] = k_in_g[j] = 0;
+
+  // issue the global loads of stage `st` (0 <= st < n_stages); nothing here may read the loaded
+  // registers, or the wave would wait for the load on the spot
+  auto load_stage = [&](int st) {
+    const uint32_t x_soff = (uint32_t)st * (BK * 2);
+    // K % 64 == 32 (KTAIL): in the last stage the upper half of the stage lies past K.  Its X
+    // columns are forced out of range (zeros); the weight rows are clamped to valid memory.
+    uint32_t poison = 0;
+    if constexpr (KTAIL) poison = ((st * BK + 8 * oct) < K) ? 0u : 0x80000000u;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a_st[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_off[i] | poison, x_soff, 0);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
+      const uint32_t qs = (uint32_t)st * q_stage_bytes[j];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const int k8u = min((k0 >> 3) + 2 * t, k8_last - 1);  // uniform part; + half per lane
-        q_nxt[j][t] = *reinterpret_cast<const uint32_t*>(qbase[j] + (size_t)k8u * Np[j] * 4 + q_off[j]);
+        uint32_t so = qs + t * q_step_bytes[j];
+        if constexpr (KTAIL) so = min(so, q_last[j]);
+        q_nxt[j][t] = __builtin_amdgcn_raw_buffer_load_b32(q_rsrc[j], q_off[j], so, 0);
       }
 #pragma unroll
       for (int u = 0; u < GPS; ++u) {
-        const int ku = k0 + u * (BK / GPS);
-        const int gu = (ku < K ? ku : k0) / gs[j];
-        sc_nxt[j][u] = scp[j][(size_t)gu * Np[j]];
-        zw_nxt[j][u] = (uint32_t)zp[j][(size_t)gu * (Np[j] >> 3)];
+        int gu;
+        if constexpr (GPS == 1) {
+          gu = g_ld[j];
+        } else {
+          const int ku = st * BK + u * (BK / GPS);
+          gu = (ku < K ? ku : st * BK) / gs[j];
+        }
+        sc_nxt[j][u] = __builtin_amdgcn_raw_buffer_load_b16(sc_rsrc[j], sc_off[j], (uint32_t)gu * Np[j] * 2, 0);
+        zw_nxt[j][u] = __builtin_amdgcn_raw_buffer_load_b32(z_rsrc[j], z_off[j], (uint32_t)gu * (Np[j] >> 3) * 4, 0);
+      }
+      if constexpr (GPS == 1) {
+        k_in_g[j] += BK;
+        if (k_in_g[j] >= gs[j]) {
+          k_in_g[j] -= gs[j];
+          ++g_ld[j];
+        }
       }
     }
   };
   // registers -> LDS buffer `buf`, and make the prefetched weight words / scales current
-  auto commit_stage = [&](int buf, int st) {
+  auto commit_stage = [&](int buf) {
     char* lw = reinterpret_cast<char*>(lds[buf]) + lds_w_off;
-    const bool k_ok = (min(st, n_stages - 1) * BK + 8 * oct) < K;  // K tail: zero columns past K
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      *reinterpret_cast<u32x4*>(lw + i * 32 * LDS_STRIDE * 2) = k_ok ? a_st[i] : u32x4{0u, 0u, 0u, 0u};
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(lw + i * 32 * LDS_STRIDE * 2) = a_st[i];
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
 #pragma unroll
@@ -185,6 +214,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int u = 0; u < GPS; ++u) {
         sf[j][u] = fp16_bits_to_f32(sc_nxt[j][u]);
+        sf16[j][u] = sf[j][u] * 0.0625f;
         const float z = (float)((zw_nxt[j][u] >> zshift[j]) & 0xFu) + zoff[j];
         nsz[j][u] = -sf[j][u] * z;  // exact: 11-bit x 5-bit
       }
@@ -203,7 +233,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     for (int mt = 0; mt < MT; ++mt)
       xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * LDS_STRIDE * 2);
 #pragma unroll
-    for (int j = 0; j < NT; ++j) wf[par][j] = dequant8<T>(q_cur[j][t], sf[j][t * GPS / 4], nsz[j][t * GPS / 4]);
+    for (int j = 0; j < NT; ++j) wf[par][j] = dequant8<T>(q_cur[j][t], sf[j][t * GPS / 4], sf16[j][t * GPS / 4], nsz[j][t * GPS / 4]);
   };
   auto mfma_step = [&](auto par_c) {
     constexpr int par = decltype(par_c)::value;
@@ -226,7 +256,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   using P1 = std::integral_constant<int, 1>;
 
   load_stage(0);
-  commit_stage(0, 0);
+  commit_stage(0);
   __syncthreads();
   prefetch(0, 0, P0{});
 
@@ -234,8 +264,9 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     const int buf = s & 1;
     // Global loads of the next stage are issued and consumed inside one iteration (steps 0-2 hide
     // their latency): a load that stayed in flight across the loop back-edge would be waited for
-    // at the back-edge, where the compiler copies loop-carried registers.
-    load_stage(s + 1);
+    // at the back-edge, where the compiler copies loop-carried registers.  In the last iteration
+    // nothing is loaded and the hand-over below just re-commits stale registers, unused.
+    if (s + 1 < n_stages) load_stage(s + 1);
     // step 0
     prefetch(buf, 1, P1{});
     mfma_step(P0{});
@@ -248,7 +279,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     prefetch(buf, 3, P1{});
     mfma_step(P0{});
     interleave();
-    commit_stage(buf ^ 1, s + 1);
+    commit_stage(buf ^ 1);
     __syncthreads();
     // step 3
     prefetch(buf ^ 1, 0, P0{});
@@ -378,17 +409,24 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
     const int gsz = projs[p].w.group_size;
     if (gsz % 64 != 0) gps = (gsz % 32 == 0) ? (gps > 2 ? gps : 2) : 4;
   }
-#define LAUNCH(TT)                                                                          \
-  do {                                                                                      \
-    if (gps == 1) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1>), grid, block, 0, st, a); \
-    else if (gps == 2) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 2>), grid, block, 0, st, a); \
-    else hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 4>), grid, block, 0, st, a);          \
+  const bool ktail = (a.K % BK) != 0;
+#define LAUNCH2(TT, KT)                                                                          \
+  do {                                                                                           \
+    if (gps == 1) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, KT>), grid, block, 0, st, a);  \
+    else if (gps == 2) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 2, KT>), grid, block, 0, st, a); \
+    else hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 4, KT>), grid, block, 0, st, a);           \
+  } while (0)
+#define LAUNCH(TT)            \
+  do {                        \
+    if (ktail) LAUNCH2(TT, true); \
+    else LAUNCH2(TT, false);  \
   } while (0)
   if (act_dtype == FMSA_BF16)
     LAUNCH(bf16_t);
   else
     LAUNCH(f16_t);
 #undef LAUNCH
+#undef LAUNCH2
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }
