@@ -138,9 +138,11 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   __amdgpu_buffer_rsrc_t q_rsrc[NT], sc_rsrc[NT], z_rsrc[NT];
   uint32_t q_off[NT], sc_off[NT], z_off[NT];
   uint32_t q_stage_bytes[NT], q_step_bytes[NT], q_last[NT];
+  int n_groups_j[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
     const int n_groups = (K + gs[j] - 1) / gs[j];
+    n_groups_j[j] = n_groups;
     q_rsrc[j] = make_rsrc(qbase[j], (size_t)(K >> 3) * Np[j] * 4);
     sc_rsrc[j] = make_rsrc(scbase[j], (size_t)n_groups * Np[j] * 2);
     z_rsrc[j] = make_rsrc(zbase[j], (size_t)n_groups * (Np[j] >> 3) * 4);
@@ -185,7 +187,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
       for (int u = 0; u < GPS; ++u) {
         int gu;
         if constexpr (GPS == 1) {
-          gu = g_ld[j];
+          gu = min(g_ld[j], n_groups_j[j] - 1);
         } else {
           const int ku = st * BK + u * (BK / GPS);
           gu = (ku < K ? ku : st * BK) / gs[j];
@@ -193,12 +195,11 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
         sc_nxt[j][u] = __builtin_amdgcn_raw_buffer_load_b16(sc_rsrc[j], sc_off[j], (uint32_t)gu * Np[j] * 2, 0);
         zw_nxt[j][u] = __builtin_amdgcn_raw_buffer_load_b32(z_rsrc[j], z_off[j], (uint32_t)gu * (Np[j] >> 3) * 4, 0);
       }
-      if constexpr (GPS == 1) {
+      if constexpr (GPS == 1) {  // uniform scalar bookkeeping, no division
         k_in_g[j] += BK;
-        if (k_in_g[j] >= gs[j]) {
-          k_in_g[j] -= gs[j];
-          ++g_ld[j];
-        }
+        const bool wrap = k_in_g[j] >= gs[j];
+        k_in_g[j] -= wrap ? gs[j] : 0;
+        g_ld[j] += wrap ? 1 : 0;
       }
     }
   };
@@ -242,16 +243,28 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[par][j], xf[par][mt], acc[mt][j]);
   };
-  // interleave: 1 MFMA, 3 VALU, and an LDS read after every second MFMA
-  auto interleave = [&]() {
+  // One wave per SIMD issues strictly in order, and an MFMA that finds the matrix pipe busy stalls
+  // everything behind it.  The other instructions of a step therefore have to sit BETWEEN its 16
+  // MFMAs (each occupies the pipe for 8 issue slots): per MFMA 3 VALU, every second one an LDS
+  // read, and in step 0 also the global loads of the next stage with their scalar offset math.
+  auto interleave = [&](auto with_vmem_c) {
+    constexpr bool with_vmem = decltype(with_vmem_c)::value;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
       if ((i & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (with_vmem) {
+        if (i < 6)
+          __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        else
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);  // nothing from the next step (or the stage hand-over) moves up
   };
+  using WithVmem = std::integral_constant<bool, true>;
+  using NoVmem = std::integral_constant<bool, false>;
   using P0 = std::integral_constant<int, 0>;
   using P1 = std::integral_constant<int, 1>;
 
@@ -262,29 +275,30 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 
   for (int s = 0; s < n_stages; ++s) {
     const int buf = s & 1;
-    // Global loads of the next stage are issued and consumed inside one iteration (steps 0-2 hide
+    // Global loads of the next stage are issued and consumed inside one iteration (steps 1-2 hide
     // their latency): a load that stayed in flight across the loop back-edge would be waited for
-    // at the back-edge, where the compiler copies loop-carried registers.  In the last iteration
-    // nothing is loaded and the hand-over below just re-commits stale registers, unused.
-    if (s + 1 < n_stages) load_stage(s + 1);
+    // at the back-edge, where the compiler copies loop-carried registers.  The last iteration
+    // re-loads the final stage (no branch, so the loads can be interleaved with step 0's MFMAs);
+    // that data is committed to the idle LDS buffer and never read.
     // step 0
+    load_stage(min(s + 1, n_stages - 1));
     prefetch(buf, 1, P1{});
     mfma_step(P0{});
-    interleave();
+    interleave(WithVmem{});
     // step 1
     prefetch(buf, 2, P0{});
     mfma_step(P1{});
-    interleave();
+    interleave(NoVmem{});
     // step 2, then hand the next stage over
     prefetch(buf, 3, P1{});
     mfma_step(P0{});
-    interleave();
+    interleave(NoVmem{});
     commit_stage(buf ^ 1);
     __syncthreads();
     // step 3
     prefetch(buf ^ 1, 0, P0{});
     mfma_step(P1{});
-    interleave();
+    interleave(NoVmem{});
   }
 
   // ---- epilogue ---------------------------------------------------------------------------
