@@ -113,11 +113,11 @@ int fmsa_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, int 
                    int act_dtype, int out_dtype, void* out, void* workspace, size_t workspace_bytes, void* stream) {
   if (!L || !R || !out) return FMSA_ERR_NULL;
   if (M <= 0 || C <= 0 || r <= 0 || ldr < C) return FMSA_ERR_SHAPE;
-  if (C % 2 != 0 || ldr % 2 != 0) return FMSA_ERR_SHAPE;
+  if (C % 8 != 0 || ldr % 8 != 0 || r % 8 != 0 || r > 128) return FMSA_ERR_SHAPE;
   if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
   if (out_dtype != FMSA_F16 && out_dtype != FMSA_BF16 && out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
   if (!workspace || workspace_bytes < fmsa_lora_grad_workspace(M, C, r)) return FMSA_ERR_WORKSPACE;
-  if ((reinterpret_cast<uintptr_t>(R) & 3u) || (reinterpret_cast<uintptr_t>(workspace) & 7u)) return FMSA_ERR_ALIGN;
+  if (!aligned16(R) || !aligned16(L) || !aligned16(workspace)) return FMSA_ERR_ALIGN;
   return launch_lora_grad(L, R, ldr, M, C, r, scale, transpose_out, act_dtype, out_dtype, out, workspace,
                           (hipStream_t)stream);
 }

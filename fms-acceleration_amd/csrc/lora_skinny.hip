@@ -60,63 +60,118 @@ __global__ __launch_bounds__(256) void lora_down_kernel(const uint16_t* __restri
 }
 
 // ---- lora_grad ----------------------------------------------------------------------------------
-// Pass 1: a wave owns 128 adjacent columns of R (one bf16x2 per lane: 256 B rows) and a fixed
-// range of tokens; the token's r coefficients L[m, :] are wave-uniform (scalar loads) and each
-// R element is used for 16 FMAs.  Partial sums are written to partial[split][r][C] (fp32).
-// Pass 2 adds the splits in index order, so the result does not depend on scheduling.
-template <typename T>
+// out[j, c] = sum_m L[m, j] * R[m, c]: the contraction runs over tokens, which is the row index of
+// both row-major operands, so each MFMA fragment (8 consecutive contraction elements per lane) is a
+// column walk.  Tiles of 32 tokens are staged through LDS (coalesced 16-byte global loads in, 16-bit
+// column reads out); the 32 tokens of a tile are assigned to the MFMA's contraction index as
+// k = 8*kg + e  <->  token 4*e + kg, and rows are padded by 32 B, which makes the four kg groups of a
+// wave hit disjoint banks.
+// Pass 1: workgroup = 128 columns of R x one fixed range of tokens (split); wave w owns columns
+// 32w .. 32w+31 (two 16-wide MFMA tiles) and all r ranks.  Partial sums go to partial[split][r][C]
+// (fp32).  Pass 2 adds the splits in index order, so the result does not depend on scheduling.
+constexpr int LG_TM = 32;               // tokens per tile
+constexpr int LG_TC = 128;              // columns of R per workgroup
+constexpr int LG_RSTRIDE = LG_TC + 16;  // elements: 256 B + 32 B pad
+
+template <typename T, int RT>
 __global__ __launch_bounds__(256) void lora_grad_partial_kernel(const uint16_t* __restrict__ L,
                                                                 const uint16_t* __restrict__ R, int64_t ldr, int M,
                                                                 int C, int r, int rows_per_split,
                                                                 float* __restrict__ partial) {
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int split = blockIdx.y * 4 + wave;
-  const int c = blockIdx.x * 128 + 2 * lane;
-  const bool c_ok = c < C;
+  constexpr int LSTRIDE = (RT == 1) ? 16 : RT * 16 + 16;  // elements; row pitch = 8 banks mod 32
+  __shared__ __attribute__((aligned(16))) uint16_t r_lds[2][LG_TM * LG_RSTRIDE];
+  __shared__ __attribute__((aligned(16))) uint16_t l_lds[2][LG_TM * LSTRIDE];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int l16 = lane & 15, kg = lane >> 4;
+  const int split = blockIdx.y;
+  const int c0 = blockIdx.x * LG_TC;
   const int m_begin = split * rows_per_split;
   const int m_end = min(M, m_begin + rows_per_split);
-  const uint16_t* rp = R + (c_ok ? c : 0);
+  const int n_tiles = (m_end - m_begin + LG_TM - 1) / LG_TM;
 
-  for (int j0 = 0; j0 < r; j0 += 16) {
-    float acc0[16], acc1[16];
+  // global -> LDS assignment: R tile = 32 rows x 16 chunks of 16 B -> 2 chunks per thread;
+  // L tile = 32 rows x (RT*2) chunks -> threads 0 .. 64*RT-1, one chunk each
+  const int r_row = tid >> 4, r_chunk = tid & 15;
+  const bool r_col_ok = (c0 + 8 * r_chunk) < C;  // C % 8 == 0
+  const int l_row = tid / (2 * RT), l_chunk = tid % (2 * RT);
+  const bool l_thread = tid < 64 * RT;
+  const bool l_col_ok = 8 * l_chunk < r;  // r % 8 == 0
+
+  u32x4 rst[2], lst;
+  auto load_tile = [&](int tile) {
+    const int m0 = m_begin + tile * LG_TM;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) acc0[j] = acc1[j] = 0.f;
-    int m = m_begin;
-    for (; m + 4 <= m_end; m += 4) {
-      uint32_t rv[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) rv[u] = *reinterpret_cast<const uint32_t*>(rp + (size_t)(m + u) * ldr);
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float r0 = unpack_lo<T>(rv[u]), r1 = unpack_hi<T>(rv[u]);
-        const uint16_t* lrow = L + (size_t)(m + u) * r + j0;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const float lj = (j0 + j < r) ? unpack1<T>(lrow[j]) : 0.f;
-          acc0[j] = __builtin_fmaf(lj, r0, acc0[j]);
-          acc1[j] = __builtin_fmaf(lj, r1, acc1[j]);
-        }
-      }
+    for (int p = 0; p < 2; ++p) {
+      const int m = m0 + r_row + 16 * p;
+      rst[p] = u32x4{0u, 0u, 0u, 0u};
+      if (m < m_end && r_col_ok) rst[p] = *reinterpret_cast<const u32x4*>(R + (size_t)m * ldr + c0 + 8 * r_chunk);
     }
-    for (; m < m_end; ++m) {
-      const uint32_t rv = *reinterpret_cast<const uint32_t*>(rp + (size_t)m * ldr);
-      const float r0 = unpack_lo<T>(rv), r1 = unpack_hi<T>(rv);
-      const uint16_t* lrow = L + (size_t)m * r + j0;
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const float lj = (j0 + j < r) ? unpack1<T>(lrow[j]) : 0.f;
-        acc0[j] = __builtin_fmaf(lj, r0, acc0[j]);
-        acc1[j] = __builtin_fmaf(lj, r1, acc1[j]);
-      }
+    lst = u32x4{0u, 0u, 0u, 0u};
+    if (l_thread) {
+      const int m = m0 + l_row;
+      if (m < m_end && l_col_ok) lst = *reinterpret_cast<const u32x4*>(L + (size_t)m * r + 8 * l_chunk);
     }
-    if (c_ok) {
+  };
+  auto commit_tile = [&](int buf) {
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        if (j0 + j < r) {
-          float2 v = make_float2(acc0[j], acc1[j]);
-          *reinterpret_cast<float2*>(partial + ((size_t)split * r + j0 + j) * C + c) = v;
-        }
+    for (int p = 0; p < 2; ++p)
+      *reinterpret_cast<u32x4*>(&r_lds[buf][(r_row + 16 * p) * LG_RSTRIDE + 8 * r_chunk]) = rst[p];
+    if (l_thread) *reinterpret_cast<u32x4*>(&l_lds[buf][l_row * LSTRIDE + 8 * l_chunk]) = lst;
+  };
+  // 8 contraction elements of column `col`: tokens 4*e + kg, e = 0..7
+  auto column_frag = [&](const uint16_t* base, int stride, int col) {
+    u32x4 f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t lo = base[(8 * e + kg) * stride + col];
+      const uint32_t hi = base[(8 * e + 4 + kg) * stride + col];
+      f[e] = lo | (hi << 16);
+    }
+    return f;
+  };
+
+  f32x4 acc[2][RT];
+#pragma unroll
+  for (int g = 0; g < 2; ++g)
+#pragma unroll
+    for (int t = 0; t < RT; ++t) acc[g][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (n_tiles > 0) {
+    load_tile(0);
+    commit_tile(0);
+  }
+  __syncthreads();
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    const int buf = tile & 1;
+    if (tile + 1 < n_tiles) load_tile(tile + 1);
+    u32x4 lf[RT], rf[2];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) lf[t] = column_frag(l_lds[buf], LSTRIDE, 16 * t + l16);
+#pragma unroll
+    for (int g = 0; g < 2; ++g) rf[g] = column_frag(r_lds[buf], LG_RSTRIDE, 32 * wave + 16 * g + l16);
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+      for (int t = 0; t < RT; ++t) acc[g][t] = mfma16<T>(rf[g], lf[t], acc[g][t]);  // D[c][j]
+    if (tile + 1 < n_tiles) commit_tile(buf ^ 1);
+    __syncthreads();
+  }
+  // lane holds D[c = 4*kg + i][j = l16]: four consecutive columns -> one 16-byte store
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+    const int c = c0 + 32 * wave + 16 * g + 4 * kg;
+    if (c >= C) continue;
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      const int j = 16 * t + l16;
+      if (j >= r) continue;
+      float* dst = partial + ((size_t)split * r + j) * C + c;
+      if (c + 4 <= C) {
+        *reinterpret_cast<f32x4*>(dst) = acc[g][t];
+      } else {
+        for (int i = 0; i < 4; ++i)
+          if (c + i < C) dst[i] = acc[g][t][i];
       }
     }
   }
@@ -142,12 +197,11 @@ __global__ __launch_bounds__(256) void lora_grad_reduce_kernel(const float* __re
 }  // namespace
 
 int lora_grad_splits(int M, int C) {
-  const int ncb = (C + 127) / 128;
-  int splits = 1536 / ncb;
-  const int max_splits = (M + 31) / 32;
+  const int ncb = (C + LG_TC - 1) / LG_TC;
+  int splits = 2048 / ncb;
+  const int max_splits = (M + 63) / 64;  // at least two 32-token tiles per split
   if (splits > max_splits) splits = max_splits;
-  splits = (splits / 4) * 4;
-  if (splits < 4) splits = 4;
+  if (splits < 1) splits = 1;
   return splits;
 }
 
@@ -179,14 +233,27 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
 int launch_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
                      int act_dtype, int out_dtype, void* out, void* workspace, hipStream_t st) {
   const int splits = lora_grad_splits(M, C);
-  const int rows_per_split = (M + splits - 1) / splits;
-  dim3 grid1((C + 127) / 128, splits / 4), block(256);
-  if (act_dtype == FMSA_BF16)
-    hipLaunchKernelGGL(lora_grad_partial_kernel<bf16_t>, grid1, block, 0, st, (const uint16_t*)L, (const uint16_t*)R,
-                       ldr, M, C, r, rows_per_split, (float*)workspace);
-  else
-    hipLaunchKernelGGL(lora_grad_partial_kernel<f16_t>, grid1, block, 0, st, (const uint16_t*)L, (const uint16_t*)R,
-                       ldr, M, C, r, rows_per_split, (float*)workspace);
+  int rows_per_split = (M + splits - 1) / splits;
+  rows_per_split = ((rows_per_split + LG_TM - 1) / LG_TM) * LG_TM;
+  dim3 grid1((C + LG_TC - 1) / LG_TC, splits), block(256);
+  const int rt = (r + 15) / 16;
+#define LAUNCH(TT, RT)                                                                                            \
+  hipLaunchKernelGGL((lora_grad_partial_kernel<TT, RT>), grid1, block, 0, st, (const uint16_t*)L, (const uint16_t*)R, \
+                     ldr, M, C, r, rows_per_split, (float*)workspace)
+#define DISPATCH(TT)                      \
+  switch (rt) {                           \
+    case 1: LAUNCH(TT, 1); break;         \
+    case 2: LAUNCH(TT, 2); break;         \
+    case 3: case 4: LAUNCH(TT, 4); break; \
+    default: LAUNCH(TT, 8); break;        \
+  }
+  if (act_dtype == FMSA_BF16) {
+    DISPATCH(bf16_t)
+  } else {
+    DISPATCH(f16_t)
+  }
+#undef DISPATCH
+#undef LAUNCH
   FMSA_CHECK_LAUNCH();
   dim3 grid2((r * C + 255) / 256);
   if (out_dtype == FMSA_F32)

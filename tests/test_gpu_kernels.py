@@ -58,7 +58,7 @@ def test_lora_down(M, C, r, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,C,r,tr", [(512, 2048, 16, False), (200, 1056, 8, True), (4096, 4096, 16, True), (96, 130, 24, False)])
+@pytest.mark.parametrize("M,C,r,tr", [(512, 2048, 16, False), (200, 1056, 8, True), (4096, 4096, 16, True), (96, 136, 24, False), (70, 4104, 64, True)])
 def test_lora_grad(M, C, r, tr, dtype):
     import fmsa_hip
 
