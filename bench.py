@@ -140,10 +140,10 @@ def time_kernels(M, device, dtype):
     Ud = fmsa_hip.lora_down(h, A_i)
     pd = {"w": Wd, "U": Ud, "B": B_h, "bias": None, "r": r, "s": 1.0}
     Td = fmsa_hip.lora_down(dy, B_h.t().contiguous())
-    bd = {"w": Wd, "dY": dy, "T": Td, "At": A_i.t().contiguous(), "mask_src": None, "r": r, "s": 1.0}
+    bd = {"w": Wd, "nsz": fmsa_hip.gptq_make_nsz(Wd, dy.device), "dY": dy, "T": Td, "At": A_i.t().contiguous(), "mask_src": None, "r": r, "s": 1.0}
     Tu = fmsa_hip.lora_down(dgi, B_i.t().contiguous())
-    bu = {"w": Wu, "dY": dgi, "T": Tu, "At": A_h.t().contiguous(), "mask_src": x, "r": r, "s": 1.0}
-    bg = dict(bu, w=Wg)
+    bu = {"w": Wu, "nsz": fmsa_hip.gptq_make_nsz(Wu, dgi.device), "dY": dgi, "T": Tu, "At": A_h.t().contiguous(), "mask_src": x, "r": r, "s": 1.0}
+    bg = dict(bu, w=Wg, nsz=fmsa_hip.gptq_make_nsz(Wg, x.device))
     e2, g2 = e.clone(), g.clone()
     out = {}
     f1 = 2.0 * M * H * I
@@ -216,7 +216,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--tokens", type=int, default=M_TOKENS)
-    ap.add_argument("--cpu-sample-tokens", type=int, default=512)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     args = ap.parse_args()

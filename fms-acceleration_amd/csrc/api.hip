@@ -16,6 +16,7 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
 int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx, void* e,
                             void* g, void* h_out, int64_t ldeg, int act_dtype, hipStream_t st);
 
+int launch_gptq_nsz(const fmsa_gptq_weight* w, float* out, hipStream_t st);
 int launch_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype, hipStream_t st);
 int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, int M, int I, int64_t ld, int act_dtype,
                       hipStream_t st);
@@ -161,21 +162,28 @@ int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mod
   if (mode != FMSA_BWD_LINEAR && mode != FMSA_BWD_SWIGLU) return FMSA_ERR_SHAPE;
   if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
   const int K = projs[0].w.K;
+  const void* mask = nullptr;
+  int64_t ldmask = 0;
   for (int p = 0; p < n_proj; ++p) {
     const fmsa_bwd_proj& s = projs[p];
     if (int rc = check_weight(&s.w, 8)) return rc;
     if (s.w.K != K) return FMSA_ERR_SHAPE;
-    if (!s.dY) return FMSA_ERR_NULL;
+    if (!s.dY || !s.nsz) return FMSA_ERR_NULL;
     if (s.lddy < s.w.N) return FMSA_ERR_SHAPE;
+    if (!aligned16(s.nsz)) return FMSA_ERR_ALIGN;
     if (!aligned16(s.dY) || s.lddy % 8 != 0) return FMSA_ERR_ALIGN;
     if (int rc = check_rank(s.r)) return rc;
     if (s.r > 0) {
       if (!s.T || !s.At) return FMSA_ERR_NULL;
       if (!aligned16(s.T) || !aligned16(s.At)) return FMSA_ERR_ALIGN;
     }
-    if (s.mask_src) {
+    if (s.mask_src && s.r > 0) {
       if (s.ldmask < K) return FMSA_ERR_SHAPE;
-      if ((reinterpret_cast<uintptr_t>(s.mask_src) & 3u) || s.ldmask % 2 != 0) return FMSA_ERR_ALIGN;
+      if (!aligned16(s.mask_src) || s.ldmask % 8 != 0) return FMSA_ERR_ALIGN;
+      // one mask per call: the LoRA terms of all projections are summed before it is applied
+      if (mask && (mask != s.mask_src || ldmask != s.ldmask)) return FMSA_ERR_UNSUPPORTED;
+      mask = s.mask_src;
+      ldmask = s.ldmask;
     }
   }
   if (mode == FMSA_BWD_SWIGLU) {
@@ -207,6 +215,13 @@ int fmsa_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h_out,
   if (!aligned16(dh) || !aligned16(e) || !aligned16(g) || !aligned16(h_out) || ld % 8 != 0 || lddh % 8 != 0)
     return FMSA_ERR_ALIGN;
   return launch_swiglu_bwd(dh, lddh, e, g, h_out, M, I, ld, act_dtype, (hipStream_t)stream);
+}
+
+int fmsa_gptq_make_nsz(const fmsa_gptq_weight* w, float* out, void* stream) {
+  if (!w || !out) return FMSA_ERR_NULL;
+  if (int rc = check_weight(w, 0)) return rc;
+  if (!aligned16(out)) return FMSA_ERR_ALIGN;
+  return launch_gptq_nsz(w, out, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -111,9 +111,16 @@ template <> FMSA_DEVI f32x4 mfma16<f16_t>(u32x4 a, u32x4 b, f32x4 c) {
 // ---- buffer resources ----------------------------------------------------------------------------
 // Raw buffer descriptor over [base, base + bytes): loads through it take a 32-bit per-lane offset
 // plus a scalar offset, and a lane offset at or past `bytes` returns zero instead of faulting.
+// The descriptor must live in scalar registers: base and size are wave-uniform by construction and
+// readfirstlane states that to the compiler (otherwise every load is wrapped in a waterfall loop).
 FMSA_DEVI __amdgpu_buffer_rsrc_t make_rsrc(const void* base, size_t bytes) {
-  const uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)bytes;
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+  uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)bytes;
+  n = __builtin_amdgcn_readfirstlane(n);
+  void* ub = reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
+  return __builtin_amdgcn_make_buffer_rsrc(ub, 0, (int)n, 0x00020000);
 }
 
 // ---- workgroup-id remap: consecutive ids land on different XCDs (id % 8), each with its own

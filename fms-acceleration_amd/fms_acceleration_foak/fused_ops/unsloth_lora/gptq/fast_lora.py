@@ -116,7 +116,7 @@ class _PreparedWeight:
     maps the kernels' row order back to the model's: row k' of the repacked weight is row
     perm[k'] of the original."""
 
-    __slots__ = ("struct", "K", "N", "group_size", "perm", "_keep")
+    __slots__ = ("struct", "K", "N", "group_size", "perm", "nsz", "_keep")
 
     def __init__(self, qweight, scales, qzeros, g_idx, bits):
         if bits != 4:
@@ -142,6 +142,9 @@ class _PreparedWeight:
         self.K, self.N, self.group_size, self.perm = K, N, gs, perm
         self._keep = (qweight, scales, qzeros)
         self.struct = fmsa_hip.make_weight(qweight, scales, qzeros, None, gs, zero_offset)
+        # -scale * zero per (group, column), fp32: read by the input-gradient kernel (frozen weight,
+        # so it is built once)
+        self.nsz = fmsa_hip.gptq_make_nsz(self.struct, qweight.device)
 
 
 def _prepare(qweight, scales, qzeros, g_idx, bits) -> _PreparedWeight:
@@ -213,7 +216,7 @@ class _Proj:
             if self.w.perm is not None:
                 At = At[self.w.perm.long()].contiguous()
                 mask_src = None if mask_src is None else fmsa_hip.permute_cols(mask_src, self.w.perm, gather=True)
-        return {"w": self.w.struct, "dY": dY2, "T": T, "At": At, "mask_src": mask_src if self.r else None,
+        return {"w": self.w.struct, "nsz": self.w.nsz, "dY": dY2, "T": T, "At": At, "mask_src": mask_src if self.r else None,
                 "r": self.r, "s": self.s}
 
     def lora_grads(self, T, Xd, U, dY2):

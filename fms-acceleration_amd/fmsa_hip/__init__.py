@@ -35,6 +35,7 @@ EXPORTED_SYMBOLS = (
     "fmsa_gptq_lora_bwd_dx",
     "fmsa_swiglu_fwd",
     "fmsa_swiglu_bwd",
+    "fmsa_gptq_make_nsz",
 )
 
 
@@ -67,6 +68,7 @@ class FwdProj(Structure):
 class BwdProj(Structure):
     _fields_ = [
         ("w", GptqWeight),
+        ("nsz", c_void_p),
         ("dY", c_void_p),
         ("lddy", c_int64),
         ("T", c_void_p),
@@ -109,6 +111,7 @@ def lib() -> ctypes.CDLL:
                                         c_void_p, c_int64, c_int, c_void_p]
     L.fmsa_swiglu_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
     L.fmsa_swiglu_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
+    L.fmsa_gptq_make_nsz.argtypes = [POINTER(GptqWeight), c_void_p, c_void_p]
     for name in EXPORTED_SYMBOLS:
         getattr(L, name)  # AttributeError here means the library is stale: rebuild it
     _lib = L
@@ -161,6 +164,14 @@ def gptq_dequant(qweight, scales, qzeros, g_idx, group_size, zero_offset=0, out_
     w = make_weight(qweight, scales, qzeros, g_idx, group_size, zero_offset)
     out = torch.empty((w.K, w.N), dtype=out_dtype, device=qweight.device)
     _check("fmsa_gptq_dequant", lib().fmsa_gptq_dequant(ctypes.byref(w), _DTYPE_ENUM[out_dtype], _ptr(out), _stream(out)))
+    return out
+
+
+def gptq_make_nsz(w: GptqWeight, device) -> torch.Tensor:
+    """fp32 [G, N] table -scale * (zero + zero_offset) read by the input-gradient kernel."""
+    G = (w.K + w.group_size - 1) // w.group_size
+    out = torch.empty((G, w.N), dtype=torch.float32, device=device)
+    _check("fmsa_gptq_make_nsz", lib().fmsa_gptq_make_nsz(ctypes.byref(w), _ptr(out), _stream(out)))
     return out
 
 
@@ -242,7 +253,7 @@ def gptq_lora_fwd(x2d, projs: Sequence[dict], mode: int = FWD_LINEAR):
 
 
 def gptq_lora_bwd_dx(projs: Sequence[dict], M: int, K: int, mode: int = BWD_LINEAR, e=None, g=None):
-    """projs: dicts with keys w, dY, T, At, mask_src, r, s.  LINEAR mode returns dX [M, K];
+    """projs: dicts with keys w, nsz, dY, T, At, mask_src, r, s.  LINEAR mode returns dX [M, K];
     SWIGLU mode overwrites e <- d_g, g <- d_e and returns h."""
     arr = (BwdProj * len(projs))()
     ref = projs[0]["dY"]
@@ -250,7 +261,7 @@ def gptq_lora_bwd_dx(projs: Sequence[dict], M: int, K: int, mode: int = BWD_LINE
         dy = p["dY"]
         assert dy.stride(1) == 1
         ms = p.get("mask_src")
-        arr[i] = BwdProj(p["w"], _ptr(dy), dy.stride(0), _ptr(p.get("T")) if p["r"] else None,
+        arr[i] = BwdProj(p["w"], _ptr(p["nsz"]), _ptr(dy), dy.stride(0), _ptr(p.get("T")) if p["r"] else None,
                          _ptr(p.get("At")) if p["r"] else None, _ptr(ms), 0 if ms is None else ms.stride(0),
                          int(p["r"]), float(p["s"] or 0.0))
     if mode == BWD_SWIGLU:

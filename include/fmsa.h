@@ -131,7 +131,7 @@ int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs /*host*/, int n_proj, const vo
 /* ------------------------------------------------------------------------------------------
  * Fused input-gradient:
  *   dX = sum_p [ dY_p * deq(W_p)^T + mask_p (.) ( T_p * (s_p A_p) ) ],  T_p = dY_p * B_p
- * for 1..3 projections sharing the input (LoRA_W / LoRA_QKV / the gate+up half of LoRA_MLP
+ * (one mask for the whole call) for 1..3 projections sharing the input (LoRA_W / LoRA_QKV / the gate+up half of LoRA_MLP
  * backward, UL/gptq/fast_lora.py:828-831, 657-674, 388-398).  mask_p = (mask_src_p != 0)
  * element-wise over [M, K] (the post-dropout input; NULL = no mask).
  * Mode FMSA_BWD_SWIGLU is the down-projection half of LoRA_MLP backward (:351-366): the result
@@ -140,17 +140,23 @@ int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs /*host*/, int n_proj, const vo
  * ------------------------------------------------------------------------------------------ */
 typedef struct fmsa_bwd_proj {
   fmsa_gptq_weight w;
-  const void* dY;   /* [M, N] act_dtype */
+  const float* nsz;  /* [G, N] fp32 = -scale * (zero + zero_offset), from fmsa_gptq_make_nsz */
+  const void* dY;    /* [M, N] act_dtype */
   int64_t lddy;
-  const void* T;    /* [M, r] act_dtype = dY * B; NULL when r == 0 */
-  const void* At;   /* [K, r] act_dtype = lora_A.weight^T (contiguous) */
-  const void* mask_src; /* [M, K] act_dtype or NULL */
+  const void* T;     /* [M, r] act_dtype = dY * B; NULL when r == 0 */
+  const void* At;    /* [K, r] act_dtype = lora_A.weight^T (contiguous) */
+  const void* mask_src; /* [M, K] act_dtype or NULL; every non-NULL entry of one call must be the same */
   int64_t ldmask;
   int32_t r;
   float s;
 } fmsa_bwd_proj;
 
 enum fmsa_bwd_mode { FMSA_BWD_LINEAR = 0, FMSA_BWD_SWIGLU = 1 };
+
+/* Per-weight table read by the input-gradient kernel: out[g, n] = -fp32(scales[g, n]) *
+ * (z[g, n] + zero_offset), fp32 [G, N] (exact: 11-bit x 5-bit).  The base weight is frozen, so a
+ * caller builds it once per weight. */
+int fmsa_gptq_make_nsz(const fmsa_gptq_weight* w /*host*/, float* out, void* stream);
 
 int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs /*host*/, int n_proj, int M, int mode,
                           void* dX, int64_t lddx, void* e, void* g, void* h_out, int64_t ldeg,

@@ -163,7 +163,9 @@ def test_fwd_swiglu(M, H, I, dtype):
 def _proj_bwd(w, dy_dev, A, B, s, dtype, mask_src=None):
     import fmsa_hip
 
-    p = {"w": gweight(w), "r": A.shape[0], "s": s, "dY": dy_dev, "mask_src": mask_src}
+    gw = gweight(w)
+    p = {"w": gw, "nsz": fmsa_hip.gptq_make_nsz(gw, dy_dev.device), "r": A.shape[0], "s": s, "dY": dy_dev,
+         "mask_src": mask_src}
     p["T"] = fmsa_hip.lora_down(dy_dev, dev(B.to(dtype).t().contiguous()))
     p["At"] = dev(A.to(dtype).t().contiguous())
     return p
@@ -204,7 +206,8 @@ def test_bwd_dx_three_projections(dtype):
     ws = [make_gptq(K, N, 128, seed=10 + i) for i, N in enumerate(Ns)]
     ABs = [olora.make_lora(K, N, r, 20 + i) for i, N in enumerate(Ns)]
     dys = [randn((M, N), 30 + i, dtype) for i, N in enumerate(Ns)]
-    projs = [_proj_bwd(w, dev(dy), A, B, s, dtype, mask_src=dev(x)) for w, (A, B), dy in zip(ws, ABs, dys)]
+    xd = dev(x)  # one mask source for the whole call
+    projs = [_proj_bwd(w, dev(dy), A, B, s, dtype, mask_src=xd) for w, (A, B), dy in zip(ws, ABs, dys)]
     dx = fmsa_hip.gptq_lora_bwd_dx(projs, M, K)
     ref, _ = olora.lora_qkv_manual(x.float(), [(w["dense"], A.to(dtype).float(), B.to(dtype).float(), s)
                                                  for w, (A, B) in zip(ws, ABs)], [d.float() for d in dys])
@@ -226,7 +229,14 @@ def test_bwd_swiglu(M, H, I, dtype):
     e_d, g_d = dev(e).clone(), dev(g).clone()
     h = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(wd, dev(dy), Ad, Bd, s, dtype)], M, I, fmsa_hip.BWD_SWIGLU, e=e_d, g=g_d)
     dh_ref = dy.float() @ wd["dense"].t() + (dy.float() @ Bd.to(dtype).float()) @ (s * Ad.to(dtype).float())
-    h_ref, dg_ref, de_ref = olora.swiglu_bwd(dh_ref.to(dtype), e, g)
+    # h does not depend on the GEMM: it must match the reference's rounding points closely
+    h_ref, _, _ = olora.swiglu_bwd(dh_ref.to(dtype), e, g)
     assert olora.max_rel_err(h.cpu(), h_ref.float()) < 4e-3
-    assert olora.max_rel_err(e_d.cpu(), dg_ref.float()) < TOL
-    assert olora.max_rel_err(g_d.cpu(), de_ref.float()) < TOL
+    # d_g, d_e against the un-rounded fp32 math (the kernel rounds dh, dh*g and the results to the
+    # storage type as the reference does; each rounding is <= 2^-9 relative)
+    e32, g32 = e.float(), g.float()
+    se = torch.sigmoid(e32)
+    dg_ref = dh_ref * (se * e32)
+    de_ref = dh_ref * g32 * se * (1.0 + e32 * (1.0 - se))
+    assert olora.max_rel_err(e_d.cpu(), dg_ref) < TOL
+    assert olora.max_rel_err(g_d.cpu(), de_ref) < TOL
