@@ -1,0 +1,112 @@
+"""The C-ABI library: every symbol declared in include/fmsa.h is exported, and argument validation
+returns error codes before any HIP call (so it runs on a machine without a GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import fmsa_hip
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "fmsa.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fmsa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_library_agree():
+    names = declared_functions()
+    assert set(names) == set(fmsa_hip.EXPORTED_SYMBOLS)
+    lib = fmsa_hip.lib()
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert lib.fmsa_abi_version() >= 1
+    assert lib.fmsa_strerror(0) == b"ok" and b"NULL" in lib.fmsa_strerror(-1)
+
+
+def test_struct_layouts_match_the_header():
+    assert ctypes.sizeof(fmsa_hip.GptqWeight) == 48
+    assert ctypes.sizeof(fmsa_hip.FwdProj) == 96
+    assert ctypes.sizeof(fmsa_hip.BwdProj) == 112
+
+
+def _w(K=64, N=64, gs=64, q=0x1000, s=0x2000, z=0x3000, g=None, zo=0):
+    return fmsa_hip.GptqWeight(q, s, z, g, K, N, gs, zo)
+
+
+def test_dequant_validation():
+    lib = fmsa_hip.lib()
+    f = lib.fmsa_gptq_dequant
+    assert f(None, 0, 0x1000, None) == -1
+    assert f(ctypes.byref(_w()), 0, None, None) == -1
+    assert f(ctypes.byref(_w(q=None)), 0, 0x1000, None) == -1
+    assert f(ctypes.byref(_w(K=40)), 0, 0x1000, None) == -2      # K % 32
+    assert f(ctypes.byref(_w(N=0)), 0, 0x1000, None) == -2
+    assert f(ctypes.byref(_w(zo=2)), 0, 0x1000, None) == -2
+    assert f(ctypes.byref(_w(q=0x1004)), 0, 0x1000, None) == -3  # alignment
+    assert f(ctypes.byref(_w()), 7, 0x1000, None) == -4          # dtype
+
+
+def test_fused_forward_validation():
+    lib = fmsa_hip.lib()
+    f = lib.fmsa_gptq_lora_fwd
+
+    def proj(**kw):
+        d = dict(w=_w(), U=0x4000, B=0x5000, bias=None, Y=0x6000, ldy=64, r=16, s=1.0)
+        d.update(kw)
+        return fmsa_hip.FwdProj(d["w"], d["U"], d["B"], d["bias"], d["Y"], d["ldy"], d["r"], d["s"])
+
+    def call(p, n=1, X=0x7000, ldx=64, M=8, mode=0, H=None, ldh=0, dt=1):
+        arr = (fmsa_hip.FwdProj * 3)(*([p] * 3))
+        return f(arr, n, X, ldx, M, mode, H, ldh, dt, None)
+
+    assert call(proj(), X=None) == -1
+    assert call(proj(), n=4) == -2
+    assert call(proj(), M=0) == -2
+    assert call(proj(), dt=2) == -4                       # fp32 is not an activation type
+    assert call(proj(), ldx=32) == -2
+    assert call(proj(w=_w(g=0x8000))) == -5               # act-order must be repacked first
+    assert call(proj(w=_w(gs=24, K=96)), ldx=96) == -5            # group size not a multiple of 16
+    assert call(proj(r=12)) == -5
+    assert call(proj(U=None)) == -1
+    assert call(proj(Y=None)) == -1
+    assert call(proj(ldy=32)) == -2
+    assert call(proj(), n=1, mode=1) == -2                # SwiGLU needs exactly gate + up
+    assert call(proj(), n=2, mode=1, H=None) == -1
+
+
+def test_bwd_and_skinny_validation():
+    lib = fmsa_hip.lib()
+    p = fmsa_hip.BwdProj(_w(), 0x9000, 0xA000, 64, 0xB000, 0xC000, None, 0, 16, 1.0)
+    arr = (fmsa_hip.BwdProj * 3)(p, p, p)
+    f = lib.fmsa_gptq_lora_bwd_dx
+    assert f(arr, 1, 8, 0, None, 0, None, None, None, 0, 1, None) == -1       # dX missing
+    assert f(arr, 1, 8, 1, None, 0, None, None, None, 0, 1, None) == -1       # e/g/h missing
+    assert f(arr, 2, 8, 1, None, 0, 0x1000, 0x2000, 0x3000, 64, 1, None) == -2  # SwiGLU takes one projection
+    p2 = fmsa_hip.BwdProj(_w(), None, 0xA000, 64, 0xB000, 0xC000, None, 0, 16, 1.0)
+    assert f((fmsa_hip.BwdProj * 1)(p2), 1, 8, 0, 0xD000, 64, None, None, None, 0, 1, None) == -1  # nsz missing
+    m1 = fmsa_hip.BwdProj(_w(), 0x9000, 0xA000, 64, 0xB000, 0xC000, 0xE000, 64, 16, 1.0)
+    m2 = fmsa_hip.BwdProj(_w(), 0x9000, 0xA000, 64, 0xB000, 0xC000, 0xF000, 64, 16, 1.0)
+    assert f((fmsa_hip.BwdProj * 2)(m1, m2), 2, 8, 0, 0xD000, 64, None, None, None, 0, 1, None) == -5  # two masks
+    assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 64, 12, 1, 0x3000, None) == -5
+    assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 60, 16, 1, 0x3000, None) == -2
+    assert lib.fmsa_lora_grad_workspace(8192, 4096, 16) > 0
+    assert lib.fmsa_lora_grad(0x1000, 0x2000, 64, 8, 64, 16, 1.0, 0, 1, 2, 0x3000, None, 0, None) == -6
+    assert lib.fmsa_swiglu_fwd(0x1000, 0x2000, 0x3000, 8, 60, 64, 1, None) == -2
+    assert lib.fmsa_gptq_permute_rows(0x1000, 0x2000, 64, 64, 0x1000, None) == -5  # in place
+
+
+def test_product_path_refuses_cpu_tensors():
+    """There is no CPU fallback: the binding raises instead of computing elsewhere."""
+    import torch
+
+    with pytest.raises(RuntimeError, match="GPU"):
+        fmsa_hip.lora_down(torch.zeros(8, 64, dtype=torch.bfloat16), torch.zeros(8, 64, dtype=torch.bfloat16))
+    from fms_acceleration_peft import QuantLinear
+
+    ql = QuantLinear(4, 64, 64, 64, False)
+    with pytest.raises(RuntimeError):
+        ql(torch.zeros(2, 64, dtype=torch.float16))

@@ -1,0 +1,223 @@
+"""ModelPatcher behaviours (mirrors plugins/framework/tests/test_model_patcher.py of the reference)
+and the fused-LoRA patch rules applied to real transformers modules on the CPU."""
+import warnings
+
+import pytest
+import torch
+
+from fms_acceleration.model_patcher import (
+    ModelPatcher,
+    ModelPatcherRule,
+    ModelPatcherTrigger,
+    ModelPatcherTriggerType,
+    combine_functions,
+    combine_triggers,
+    patch_model,
+)
+from fms_acceleration.utils.test_utils import instantiate_model_patcher
+
+
+class Leaf(torch.nn.Module):
+    def forward(self, x):
+        return x + 1
+
+
+class Other(torch.nn.Module):
+    def forward(self, x):
+        return x
+
+
+class Net(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.a = Leaf()
+        self.b = Leaf()
+        self.c = Other()
+
+    def forward(self, x):
+        return self.c(self.b(self.a(x)))
+
+
+def test_trigger_typing():
+    assert ModelPatcherTrigger(check=Leaf).type == ModelPatcherTriggerType.module
+    assert ModelPatcherTrigger(check=lambda m: True).type == ModelPatcherTriggerType.callable
+    with pytest.raises(TypeError):
+        ModelPatcherTrigger(check=3)
+    with pytest.raises(AssertionError):
+        ModelPatcherTrigger(check=Leaf, type=ModelPatcherTriggerType.callable)
+    t = ModelPatcherTrigger(check=Leaf, module_name="a")
+    assert t.is_triggered(Leaf(), "a") and not t.is_triggered(Leaf(), "b") and not t.is_triggered(Other(), "a")
+
+    def raises(m):
+        raise AttributeError("no such child")
+
+    assert not ModelPatcherTrigger(check=raises).is_triggered(Leaf())
+
+
+def test_combine_triggers_and_functions():
+    is_leaf = ModelPatcherTrigger(check=Leaf)
+    named_a = ModelPatcherTrigger(check=lambda m: True, module_name="a")
+    assert combine_triggers(is_leaf, named_a, logic="OR").is_triggered(Other(), "a") is False  # name not passed on
+    assert combine_triggers(is_leaf, ModelPatcherTrigger(check=Other), logic="OR").is_triggered(Other())
+    assert not combine_triggers(is_leaf, ModelPatcherTrigger(check=Other), logic="AND").is_triggered(Other())
+    with pytest.raises(AssertionError):
+        combine_triggers(is_leaf, logic="XOR")
+    f = combine_functions(lambda m: [1], lambda m: [2, 3])
+    assert f(None) == [1, 2, 3]
+
+
+def test_rule_validation_and_duplicates():
+    with pytest.raises(ValueError, match="at most one"):
+        ModelPatcherRule("r", trigger=ModelPatcherTrigger(check=Leaf), forward=lambda s, x: x, forward_builder=lambda m: None)
+    with pytest.raises(ValueError, match="trigger must be None"):
+        ModelPatcherRule("r", trigger=ModelPatcherTrigger(check=Leaf), import_and_maybe_reload=("a.b", object, None))
+    with instantiate_model_patcher():
+        ModelPatcher.register(ModelPatcherRule("dup", trigger=ModelPatcherTrigger(check=Leaf)))
+        with pytest.raises(AssertionError, match="already exists"):
+            ModelPatcher.register(ModelPatcherRule("dup", trigger=ModelPatcherTrigger(check=Leaf)))
+    assert "dup" not in ModelPatcher.rules  # isolation restored the singleton
+
+
+def test_forward_replacement_first_rule_wins():
+    with instantiate_model_patcher():
+        ModelPatcher.register(ModelPatcherRule("plus10", trigger=ModelPatcherTrigger(check=Leaf), forward=lambda self, x: x + 10))
+        ModelPatcher.register(ModelPatcherRule("plus100", trigger=ModelPatcherTrigger(check=Leaf), forward=lambda self, x: x + 100))
+        net = Net()
+        with warnings.catch_warnings(record=True) as w:
+            warnings.simplefilter("always")
+            patch_model(net)
+        assert any("is ignored" in str(x.message) for x in w)
+        assert net(torch.zeros(1)).item() == 20
+        assert [h.rule_id for h in ModelPatcher.history] == ["plus10", "plus10"]
+        assert "plus10" in ModelPatcher.summary() and "Leaf" in ModelPatcher.summary()
+        assert len(ModelPatcher.summary(raw=True)) == 2
+
+
+def test_forward_builder_list_becomes_sub_rules():
+    calls = []
+
+    def builder(mod):
+        calls.append(type(mod).__name__)
+        return [
+            (ModelPatcherTrigger(check=Leaf, module_name="a"), lambda self, x: x + 2),
+            (ModelPatcherTrigger(check=Leaf, module_name="b"), lambda self, x: x + 3),
+        ]
+
+    with instantiate_model_patcher():
+        ModelPatcher.register(ModelPatcherRule("net", trigger=ModelPatcherTrigger(check=Net), forward_builder=builder))
+        net = Net()
+        patch_model(net)
+        assert calls == ["Net"]
+        assert net(torch.zeros(1)).item() == 5
+        assert sorted(h.rule_id for h in ModelPatcher.history) == ["net-1", "net-2"]
+        assert set(ModelPatcher.rules) == {"net"}  # temporary sub-rules are gone
+
+
+def _tiny_llama_layer():
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaAttention, LlamaMLP
+
+    from fms_acceleration_peft import LoraLinear, QuantLinear
+
+    cfg = LlamaConfig(hidden_size=128, intermediate_size=256, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=64, hidden_act="silu")
+    cfg.architectures = ["LlamaForCausalLM"]
+
+    def wrap(lin):
+        return LoraLinear(QuantLinear(4, 64, lin.in_features, lin.out_features, False), r=8, lora_alpha=16)
+
+    block = torch.nn.Module()
+    block.self_attn = LlamaAttention(cfg, layer_idx=0)
+    block.mlp = LlamaMLP(cfg)
+    for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
+        setattr(block.self_attn, name, wrap(getattr(block.self_attn, name)))
+    for name in ("gate_proj", "up_proj", "down_proj"):
+        setattr(block.mlp, name, wrap(getattr(block.mlp, name)))
+    block.config = cfg
+    return block, cfg
+
+
+def test_fused_lora_rules_patch_llama_modules():
+    """The FOAK plugin registers llama-qkvo / llama-mlp (and the mistral / granite twins); patching a
+    Llama attention + MLP whose projections are LoRA-wrapped QuantLinears rebinds q/k/v/o and the MLP."""
+    from fms_acceleration_foak import FastKernelsAccelerationPlugin
+    from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_mlp, apply_lora_o_v2
+
+    block, cfg = _tiny_llama_layer()
+    block.quantization_method = "gptq"
+    plugin = FastKernelsAccelerationPlugin({"training": {"fused_ops_and_kernels": {"fused_lora": True, "fast_loss": True}}})
+    train_args = type("T", (), {"bf16": True, "fp16": False})()
+    with instantiate_model_patcher():
+        plugin.augmentation(block, train_args, ())
+        assert set(ModelPatcher.rules) == {"llama-qkvo", "llama-mlp", "mistral-qkvo", "mistral-mlp", "granite-qkvo", "granite-mlp"}
+        patch_model(block)
+        ids = sorted(h.rule_id for h in ModelPatcher.history)
+        assert ids == ["llama-mlp", "llama-qkvo-1", "llama-qkvo-2", "llama-qkvo-3", "llama-qkvo-4"]
+        assert block.mlp.forward.__func__ is apply_lora_mlp
+        assert block.self_attn.o_proj.forward.__func__ is apply_lora_o_v2
+        for name in ("q_proj", "k_proj", "v_proj"):
+            assert "forward" in vars(getattr(block.self_attn, name))  # instance-level rebinding
+        assert plugin.get_callbacks_and_ready_for_train(block, None) == []
+    # without a quantised base the fused-LoRA rules are not registered at all
+    block2, _ = _tiny_llama_layer()
+    with instantiate_model_patcher():
+        plugin.augmentation(block2, train_args, ())
+        assert set(ModelPatcher.rules) == set()
+    # mixed precision is mandatory on a quantised base
+    with instantiate_model_patcher():
+        with pytest.raises(AssertionError, match="mixed precision"):
+            plugin.augmentation(block, type("T", (), {"bf16": False, "fp16": False})(), ())
+
+
+def test_mlp_rule_dropped_for_non_silu_activation():
+    from fms_acceleration_foak.models import llama
+
+    cfg = type("C", (), {"hidden_act": "gelu", "architectures": ["LlamaForCausalLM"]})()
+    with warnings.catch_warnings(record=True):
+        warnings.simplefilter("always")
+        ids = [r.rule_id for r in llama.get_mp_rules("auto_gptq", cfg)]
+    assert ids == ["llama-qkvo"]
+
+
+def test_partial_lora_follows_the_reference_rule_logic():
+    """The qkvo trigger is an OR of "q, k, v all LoRA" and "o is LoRA", and its builder APPENDs the
+    sub-rules of both branches (models/llama.py:75-108 of the reference): with an adapter-less k_proj
+    the rule still fires through o_proj, and the per-projection sub-rules then patch exactly the
+    children that are LoRA layers (q, v, o).  Same behaviour as the reference, kept as is."""
+    from fms_acceleration_foak.models import llama
+
+    block, cfg = _tiny_llama_layer()
+    block.self_attn.k_proj = block.self_attn.k_proj.base_layer  # k loses its adapter
+    with instantiate_model_patcher():
+        for r in llama.get_mp_rules("auto_gptq", cfg):
+            ModelPatcher.register(r)
+        patch_model(block)
+        ids = sorted(h.rule_id for h in ModelPatcher.history)
+        assert ids == ["llama-mlp", "llama-qkvo-1", "llama-qkvo-3", "llama-qkvo-4"]
+
+
+def test_qkv_wrapper_protocol():
+    from fms_acceleration_foak.models.utils import _build_fused_forwards
+
+    calls = []
+
+    def fused(attn, X):
+        calls.append(1)
+        return X + 1, X + 2, X + 3
+
+    fwd = dict(_build_fused_forwards(None, fused, ["q_proj", "k_proj", "v_proj"]))
+    x = torch.zeros(1)
+    assert fwd["q_proj"](None, x).item() == 1
+    assert fwd["k_proj"](None, x).item() == 2
+    with pytest.raises(AssertionError):
+        fwd["k_proj"](None, x)  # k called twice before v
+    assert fwd["v_proj"](None, x).item() == 3
+    assert fwd["v_proj"](None, x).item() == 3 and len(calls) == 2  # a new round starts with whoever comes first
+
+
+def test_filter_mp_rules():
+    from fms_acceleration_foak.utils import filter_mp_rules
+
+    rules = [ModelPatcherRule(rule_id=i) for i in ("a-qkvo", "a-mlp", "a-rms")]
+    assert [r.rule_id for r in filter_mp_rules(rules, {"qkvo", "mlp"})] == ["a-qkvo", "a-mlp"]
+    assert [r.rule_id for r in filter_mp_rules(rules, {"mlp"}, drop=True)] == ["a-qkvo", "a-rms"]
