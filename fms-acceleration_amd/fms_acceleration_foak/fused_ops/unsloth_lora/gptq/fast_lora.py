@@ -240,13 +240,18 @@ def _linear_forward(projs, X2, Xds):
 
 
 def _linear_backward_dx(projs, dYs, Ts, Xds, M, K):
-    if all(p.w.perm is None for p in projs):
+    """dX = sum_p dY_p deq(W_p)^T + mask (.) sum_p s_p T_p A_p.  One launch when the projections share
+    one mask source (no dropout, or one dropout module applied once) and none is act-order; otherwise
+    one launch per projection (each with its own mask / column order) and a sum."""
+    masks = [Xd for p, Xd in zip(projs, Xds) if p.r]
+    one_mask = all(m is masks[0] for m in masks)
+    if one_mask and all(p.w.perm is None for p in projs):
         return fmsa_hip.gptq_lora_bwd_dx([p.bwd_dict(dY, T, Xd) for p, dY, T, Xd in zip(projs, dYs, Ts, Xds)], M, K)
     dX = None
     for p, dY, T, Xd in zip(projs, dYs, Ts, Xds):
         part = p.from_kernel_order(fmsa_hip.gptq_lora_bwd_dx([p.bwd_dict(dY, T, Xd)], M, K))
-        dX = part if dX is None else dX.add_(part)
-    return dX
+        dX = part.float() if dX is None else dX.add_(part)  # summed in fp32, rounded once
+    return dX.to(dYs[0].dtype) if len(projs) > 1 else part
 
 
 def _Bt(p):

@@ -1,0 +1,113 @@
+"""Patched (fused) versus unpatched (unfused QuantLinear + LoRA) transformers modules, the
+reference's own parity test design (plugins/fused-ops-and-kernels/tests/test_fused_ops.py:355-438):
+deep-copy a Llama attention / MLP whose projections are LoRA-wrapped GPTQ linears, patch one copy
+through the ModelPatcher rules, run both under autocast, loss = out.norm(), compare the loss and
+the adapter gradients -- plus the input gradient, which the reference computes but never asserts."""
+import copy
+
+import pytest
+import torch
+
+from fms_acceleration.model_patcher import ModelPatcher, patch_model
+from fms_acceleration.utils.test_utils import instantiate_model_patcher
+from tests.helpers import randn
+from tests.model_utils import MaskDropout, make_lora_gptq_linear
+
+pytestmark = pytest.mark.gpu
+
+# the reference's sizes and LoRA settings (test_fused_ops.py:61-64)
+SIZES = [(1, 128, 2048), (2, 256, 2048)]
+R, ALPHA = 8, 1.0
+
+
+def _llama_cfg(hidden):
+    from transformers import LlamaConfig
+
+    cfg = LlamaConfig(hidden_size=hidden, intermediate_size=2 * hidden, num_attention_heads=16, num_key_value_heads=4,
+                      num_hidden_layers=1, vocab_size=64, hidden_act="silu", attention_dropout=0.0)
+    cfg._attn_implementation = "eager"
+    return cfg
+
+
+def _wrap(mod, names, seed, dropout_p=0.0, tokens=None):
+    for i, name in enumerate(names):
+        lin = getattr(mod, name)
+        drop = MaskDropout(dropout_p, (tokens, lin.in_features), seed=seed + 50 + i) if dropout_p else None
+        wrapped, _, _, _ = make_lora_gptq_linear(lin.in_features, lin.out_features, R, ALPHA, seed=seed + i, dropout=drop)
+        setattr(mod, name, wrapped)
+
+
+def _patched_copy(module, cfg):
+    from fms_acceleration_foak.models import llama
+
+    twin = copy.deepcopy(module)
+    with instantiate_model_patcher():
+        for rule in llama.get_mp_rules("auto_gptq", cfg):
+            ModelPatcher.register(rule)
+        patch_model(twin)
+        n_patched = len(ModelPatcher.history)
+    return twin, n_patched
+
+
+def _lora_grads(module):
+    return {n: p.grad.float().cpu() for n, p in module.named_parameters() if "lora_" in n}
+
+
+def _compare(ref_mod, fused_mod, run, x, dtype):
+    outs = []
+    for mod in (ref_mod, fused_mod):
+        xi = x.clone().requires_grad_(True)
+        with torch.autocast(device_type="cuda", dtype=dtype):
+            out = run(mod, xi)
+            loss = out.float().norm()
+        loss.backward()
+        outs.append((loss.item(), xi.grad.float().cpu(), _lora_grads(mod), out.float().detach().cpu()))
+    (l0, dx0, g0, o0), (l1, dx1, g1, o1) = outs
+    # fp16: the reference's own tolerances (loss abs diff < 1e-3, grads allclose rtol 1e-3 / atol 1e-4,
+    # test_fused_ops.py:51-53).  bf16 keeps 3 fewer mantissa bits than fp16, so the same criteria are
+    # scaled by 8.  Both sides are 16-bit pipelines that round at different places; the <= 1e-2 gate
+    # against the fp32 oracle is tests/test_gpu_fused_ops.py.
+    k = 1.0 if dtype == torch.float16 else 8.0
+    assert abs(l0 - l1) < 1e-3 * k * max(1.0, abs(l0) / 10), (l0, l1)
+    assert torch.allclose(o0, o1, rtol=1e-3 * k, atol=2e-3 * k * o0.abs().max().item())
+    assert torch.allclose(dx0, dx1, rtol=1e-3 * k, atol=1e-4 * k)
+    assert g0.keys() == g1.keys() and len(g0) > 0
+    for name in g0:
+        assert torch.allclose(g0[name], g1[name], rtol=1e-3 * k, atol=1e-4 * k), name
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dropout_p", [0.0, 0.1, 0.5])
+@pytest.mark.parametrize("bsz,seq,hidden", SIZES)
+def test_attention_qkvo(bsz, seq, hidden, dropout_p, dtype):
+    from transformers.models.llama.modeling_llama import LlamaAttention, LlamaRotaryEmbedding
+
+    cfg = _llama_cfg(hidden)
+    attn = LlamaAttention(cfg, layer_idx=0)
+    _wrap(attn, ("q_proj", "k_proj", "v_proj", "o_proj"), seed=3, dropout_p=dropout_p, tokens=bsz * seq)
+    attn = attn.cuda()
+    fused, n_patched = _patched_copy(attn, cfg)
+    assert n_patched == 4
+    x = randn((bsz, seq, hidden), 2, dtype).cuda()
+    pos = torch.arange(seq, device="cuda")[None].expand(bsz, -1)
+    cos, sin = LlamaRotaryEmbedding(cfg).cuda()(x, pos)
+
+    def run(mod, xi):
+        return mod(xi, position_embeddings=(cos, sin), attention_mask=None)[0]
+
+    _compare(attn, fused, run, x, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bsz,seq,hidden", SIZES)
+def test_mlp(bsz, seq, hidden, dtype):
+    from transformers.models.llama.modeling_llama import LlamaMLP
+
+    cfg = _llama_cfg(hidden)
+    mlp = LlamaMLP(cfg)
+    _wrap(mlp, ("gate_proj", "up_proj", "down_proj"), seed=9)
+    mlp = mlp.cuda()
+    fused, n_patched = _patched_copy(mlp, cfg)
+    assert n_patched == 1
+    x = randn((bsz, seq, hidden), 2, dtype).cuda()
+    _compare(mlp, fused, lambda mod, xi: mod(xi), x, dtype)
