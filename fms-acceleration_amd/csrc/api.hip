@@ -17,6 +17,7 @@ int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int m
                             void* g, void* h_out, int64_t ldeg, int act_dtype, hipStream_t st);
 
 int launch_gptq_nsz(const fmsa_gptq_weight* w, float* out, hipStream_t st);
+int launch_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, hipStream_t st);
 int launch_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype, hipStream_t st);
 int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, int M, int I, int64_t ld, int act_dtype,
                       hipStream_t st);
@@ -222,6 +223,16 @@ int fmsa_gptq_make_nsz(const fmsa_gptq_weight* w, float* out, void* stream) {
   if (int rc = check_weight(w, 0)) return rc;
   if (!aligned16(out)) return FMSA_ERR_ALIGN;
   return launch_gptq_nsz(w, out, (hipStream_t)stream);
+}
+
+int fmsa_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, void* stream) {
+  if (!w || !out) return FMSA_ERR_NULL;
+  if (!w->packed || !w->absmax_q || !w->absmax2 || !w->code2 || !w->code) return FMSA_ERR_NULL;
+  if (w->N <= 0 || w->K <= 0 || w->blocksize <= 0 || w->blocksize2 <= 0) return FMSA_ERR_SHAPE;
+  if (w->blocksize % 16 != 0 || ((int64_t)w->N * w->K) % w->blocksize != 0) return FMSA_ERR_SHAPE;
+  if (out_dtype != FMSA_F16 && out_dtype != FMSA_BF16 && out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
+  if (!aligned16(out) || (reinterpret_cast<uintptr_t>(w->packed) & 7u)) return FMSA_ERR_ALIGN;
+  return launch_nf4_dequant(w, out_dtype, out, (hipStream_t)stream);
 }
 
 }  // extern "C"

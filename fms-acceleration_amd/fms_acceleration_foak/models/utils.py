@@ -13,6 +13,9 @@ import torch
 
 from fms_acceleration.model_patcher import ModelPatcherTrigger
 
+from ..fused_ops.unsloth_lora.bnb.fast_lora import apply_lora_mlp_swiglu as fused_op_mlp_bnb
+from ..fused_ops.unsloth_lora.bnb.fast_lora import apply_lora_o_v2 as fused_op_o_bnb
+from ..fused_ops.unsloth_lora.bnb.fast_lora import apply_lora_qkv as fused_op_qkv_bnb
 from ..fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_mlp as fused_op_mlp_gptq
 from ..fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_o_v2 as fused_op_o_gptq
 from ..fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_qkv as fused_op_qkv_gptq
@@ -25,6 +28,7 @@ KEY_HIDDEN_ACTIVATIONS = ["hidden_act", "activation_function"]
 
 FUSED_OPS = {
     "auto_gptq": {KEY_QKV: fused_op_qkv_gptq, KEY_O: fused_op_o_gptq, KEY_MLP: fused_op_mlp_gptq},
+    "bitsandbytes": {KEY_QKV: fused_op_qkv_bnb, KEY_O: fused_op_o_bnb, KEY_MLP: fused_op_mlp_bnb},
 }
 
 

@@ -1,5 +1,7 @@
 """Namesake of `fms_acceleration_peft`: the quantised base-layer data layouts (GPTQ QuantLinear,
 NF4 container), a stand-in LoRA wrapper, and the plugin configuration shells."""
 from .framework_plugin_autogptq import AutoGPTQAccelerationPlugin
+from .framework_plugin_bnb import BNBAccelerationPlugin
 from .lora import LoraLinear
 from .qlinear import QuantLinear, QuantLinearFunction
+from .nf4 import Linear4bit, Params4bit, QuantState, quantize_nf4

@@ -20,7 +20,7 @@ class LoraLinear(nn.Module):
                  adapter_name: str = "default", dtype=torch.float32):
         super().__init__()
         self.base_layer = base_layer
-        in_f = getattr(base_layer, "infeatures", None) or base_layer.in_features
+        in_f = getattr(base_layer, "infeatures", None) or base_layer.in_features  # QuantLinear / Linear4bit
         out_f = getattr(base_layer, "outfeatures", None) or base_layer.out_features
         self.in_features, self.out_features = in_f, out_f
         self.r = {adapter_name: r}

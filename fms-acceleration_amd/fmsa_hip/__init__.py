@@ -36,6 +36,7 @@ EXPORTED_SYMBOLS = (
     "fmsa_swiglu_fwd",
     "fmsa_swiglu_bwd",
     "fmsa_gptq_make_nsz",
+    "fmsa_nf4_dequant",
 )
 
 
@@ -49,6 +50,21 @@ class GptqWeight(Structure):
         ("N", c_int32),
         ("group_size", c_int32),
         ("zero_offset", c_int32),
+    ]
+
+
+class Nf4Weight(Structure):
+    _fields_ = [
+        ("packed", c_void_p),
+        ("absmax_q", c_void_p),
+        ("absmax2", c_void_p),
+        ("code2", c_void_p),
+        ("code", c_void_p),
+        ("offset", c_float),
+        ("N", c_int32),
+        ("K", c_int32),
+        ("blocksize", c_int32),
+        ("blocksize2", c_int32),
     ]
 
 
@@ -112,6 +128,7 @@ def lib() -> ctypes.CDLL:
     L.fmsa_swiglu_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
     L.fmsa_swiglu_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
     L.fmsa_gptq_make_nsz.argtypes = [POINTER(GptqWeight), c_void_p, c_void_p]
+    L.fmsa_nf4_dequant.argtypes = [POINTER(Nf4Weight), c_int, c_void_p, c_void_p]
     for name in EXPORTED_SYMBOLS:
         getattr(L, name)  # AttributeError here means the library is stale: rebuild it
     _lib = L
@@ -294,3 +311,14 @@ def swiglu_bwd(dh, e, g):
     _check("fmsa_swiglu_bwd", lib().fmsa_swiglu_bwd(_ptr(dh), dh.stride(0), _ptr(e), _ptr(g), _ptr(h), M, I, e.stride(0),
                                                     act_enum(e.dtype), _stream(e)))
     return h
+
+
+def nf4_dequant(packed, absmax_q, absmax2, code2, code, offset: float, shape, blocksize: int, blocksize2: int,
+                out_dtype=torch.bfloat16):
+    """Dense [N, K] weight of a bitsandbytes NF4 tensor with double-quantised absmax."""
+    N, K = shape
+    w = Nf4Weight(packed.data_ptr(), absmax_q.data_ptr(), absmax2.data_ptr(), code2.data_ptr(), code.data_ptr(),
+                  float(offset), N, K, blocksize, blocksize2)
+    out = torch.empty((N, K), dtype=out_dtype, device=packed.device)
+    _check("fmsa_nf4_dequant", lib().fmsa_nf4_dequant(ctypes.byref(w), _DTYPE_ENUM[out_dtype], _ptr(out), _stream(out)))
+    return out

@@ -173,6 +173,28 @@ int fmsa_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t
 int fmsa_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h_out, int M, int I,
                     int64_t ld, int act_dtype, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * bitsandbytes NF4 weight with double-quantised absmax, as fast_dequantize reads it from a
+ * quant_state (UL/utils.py:86-141): weight [N, K] row-major, flattened, `blocksize` weights per
+ * absmax, two 4-bit codes per byte with the EVEN element in the high nibble.
+ *   absmax[b] = code2[absmax_q[b]] * absmax2[b / blocksize2] + offset        (fp32)
+ *   W[i]      = code[nibble(i)] * absmax[i / blocksize]                      (fp32, one RNE to out)
+ * fmsa_nf4_dequant replaces cdequantize_blockwise_fp32 + cdequantize_blockwise_{fp16,bf16,fp32}_nf4
+ * (:119-136) in one pass; out is [N, K] row-major (the reference returns its transpose as a view).
+ * blocksize % 16 == 0, N*K % blocksize == 0.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct fmsa_nf4_weight {
+  const uint8_t* packed;   /* [N*K/2]                                  quant_state weight   */
+  const uint8_t* absmax_q; /* [N*K/blocksize]                          quant_state.absmax   */
+  const float* absmax2;    /* [ceil(N*K/blocksize/blocksize2)]         state2.absmax        */
+  const float* code2;      /* [256]                                    state2.code          */
+  const float* code;       /* [16] NF4 code book                       quant_state.code     */
+  float offset;            /*                                          quant_state.offset   */
+  int32_t N, K, blocksize, blocksize2;
+} fmsa_nf4_weight;
+
+int fmsa_nf4_dequant(const fmsa_nf4_weight* w /*host*/, int out_dtype, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -39,3 +39,33 @@ def make_lora_gptq_linear(K, N, r, alpha, seed, group_size=128, act_order=False,
     if dropout is not None:
         lin.lora_dropout["default"] = dropout
     return lin.to(device), w["dense"], A, B
+
+
+def make_lora_nf4_linear(K, N, r, alpha, seed, bias=False, device="cpu", lora_dtype=torch.float32, dropout=None,
+                         compute_dtype=torch.bfloat16):
+    """LoraLinear(Linear4bit) with seeded weights; the NF4 tensors come from the oracle's quantiser.
+    Returns (module, dense fp32 W [K, N] from the oracle's dequantisation, A, B)."""
+    import numpy as np
+
+    from fms_acceleration_peft import Linear4bit, LoraLinear
+    from fms_acceleration_peft.nf4 import Params4bit, QuantState, QuantState2
+    from oracle import nf4 as onf4
+
+    rng = np.random.default_rng(seed)
+    Wd = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    q = onf4.quantize(Wd)
+    base = Linear4bit(K, N, bias, compute_dtype)
+    state = QuantState(torch.from_numpy(q["absmax_q"]), (N, K), compute_dtype, q["blocksize"],
+                       torch.from_numpy(onf4.NF4.copy()), torch.tensor(float(q["offset"])),
+                       QuantState2(torch.from_numpy(q["absmax2"]), torch.from_numpy(q["code2"]), q["blocksize2"]))
+    base.weight = Params4bit(torch.from_numpy(q["packed"]), state)
+    if bias:
+        gen = torch.Generator().manual_seed(seed + 77)
+        base.bias.data.copy_((torch.randn(N, generator=gen) * 0.1).to(compute_dtype))
+    lin = LoraLinear(base, r, alpha, dtype=lora_dtype)
+    A, B = olora.make_lora(K, N, r, seed + 1)
+    lin.lora_A["default"].weight.data.copy_(A)
+    lin.lora_B["default"].weight.data.copy_(B)
+    if dropout is not None:
+        lin.lora_dropout["default"] = dropout
+    return lin.to(device), onf4.dequant(q, "fp32").t().contiguous(), A, B

@@ -1,0 +1,157 @@
+"""NF4 path: the dequantisation kernel bit-exact against the CPU oracle (whose own parity with
+bitsandbytes is unpinned: the library is absent and the reference holds no NF4 vectors), and the
+bitsandbytes-flavoured fused operators against the oracle's unfused graph."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import lora as olora
+from oracle import nf4 as onf4
+from tests.helpers import randn
+from tests.model_utils import MaskDropout, make_lora_nf4_linear
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+_NAME = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}
+
+
+def _q(t, dtype):
+    return t.to(dtype).float()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,K", [(96, 512), (1, 64), (256, 4096), (1000, 192)])
+def test_nf4_dequant_bit_exact(N, K, dtype):
+    import fmsa_hip
+
+    rng = np.random.default_rng(N * 7 + K)
+    W = (rng.standard_normal((N, K)) * rng.uniform(0.005, 0.05, size=(N, 1))).astype(np.float32)
+    q = onf4.quantize(W)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    out = fmsa_hip.nf4_dequant(dev(q["packed"]), dev(q["absmax_q"]), dev(q["absmax2"]), dev(q["code2"]),
+                               dev(onf4.NF4), float(q["offset"]), (N, K), 64, 256, dtype)
+    ref = onf4.dequant(q, _NAME[dtype])
+    assert out.shape == (N, K) and out.dtype == dtype
+    assert torch.equal(out.cpu(), ref)
+
+
+def test_nf4_dequant_rejects_bad_shapes():
+    import fmsa_hip
+
+    z = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    f = torch.zeros(256, device="cuda")
+    with pytest.raises(fmsa_hip.FmsaError):
+        fmsa_hip.nf4_dequant(z, z, f, f, f[:16], 0.0, (1, 72), 64, 256, torch.bfloat16)  # N*K % blocksize
+
+
+def test_linear4bit_unfused_forward():
+    lin, W, _, _ = make_lora_nf4_linear(256, 128, 8, 16.0, seed=5, device="cuda", bias=True)
+    x = randn((4, 10, 256), 1, torch.bfloat16)
+    y = lin.base_layer(x.cuda())
+    ref = x.float() @ W + lin.base_layer.bias.float().cpu()
+    assert olora.max_rel_err(y.cpu(), ref) < TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("B_,S_,K,N,r", [(1, 128, 1024, 2048, 8), (3, 50, 256, 96, 32)])
+def test_lora_w(B_, S_, K, N, r, dtype, bias):
+    from fms_acceleration_foak.fused_ops.unsloth_lora.bnb.fast_lora import apply_lora_o_v2
+
+    alpha = 2.0 * r
+    lin, W, A, B = make_lora_nf4_linear(K, N, r, alpha, seed=3, device="cuda", bias=bias, compute_dtype=dtype)
+    x = randn((B_, S_, K), 2, dtype)
+    dy = randn((B_, S_, N), 3, dtype)
+    xg = x.cuda().requires_grad_(True)
+    y = apply_lora_o_v2(lin, xg)
+    y.backward(dy.cuda())
+    b = lin.base_layer.bias.float().cpu() if bias else None
+    y_ref, dx_ref, dA_ref, dB_ref = olora.lora_w_autograd(
+        x.float().reshape(-1, K), W, _q(A, dtype), _q(B, dtype), alpha / r, dy.float().reshape(-1, N), b)
+    assert y.shape == (B_, S_, N) and y.dtype == dtype
+    assert olora.max_rel_err(y.reshape(-1, N), y_ref) < TOL
+    assert olora.max_rel_err(xg.grad.reshape(-1, K), dx_ref) < TOL
+    gA, gB = lin.lora_A["default"].weight.grad, lin.lora_B["default"].weight.grad
+    assert gA.dtype == torch.float32
+    assert olora.max_rel_err(gA, dA_ref) < TOL
+    assert olora.max_rel_err(gB, dB_ref) < TOL
+    assert lin.base_layer.weight.grad is None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_lora_qkv(dtype):
+    from fms_acceleration_foak.fused_ops.unsloth_lora.bnb.fast_lora import apply_lora_qkv
+
+    Bz, S, K, r, alpha = 2, 96, 1024, 16, 32.0
+    Ns = {"q_proj": 1024, "k_proj": 256, "v_proj": 256}
+    attn = torch.nn.Module()
+    projs = []
+    for i, (name, N) in enumerate(Ns.items()):
+        lin, W, A, B = make_lora_nf4_linear(K, N, r, alpha, seed=10 + i, device="cuda", compute_dtype=dtype)
+        setattr(attn, name, lin)
+        projs.append((W, _q(A, dtype), _q(B, dtype), alpha / r))
+    x = randn((Bz, S, K), 2, dtype)
+    douts = [randn((Bz, S, N), 30 + i, dtype) for i, N in enumerate(Ns.values())]
+    xg = x.cuda().requires_grad_(True)
+    outs = apply_lora_qkv(attn, xg)
+    torch.autograd.backward(outs, [d.cuda() for d in douts])
+    outs_ref, dx_ref, grads_ref = olora.lora_qkv_autograd(
+        x.float().reshape(-1, K), projs, [d.float().reshape(-1, d.shape[-1]) for d in douts])
+    for o, o_ref in zip(outs, outs_ref):
+        assert olora.max_rel_err(o.reshape(o_ref.shape), o_ref) < TOL
+    assert olora.max_rel_err(xg.grad.reshape(-1, K), dx_ref) < TOL
+    for name, (dA_ref, dB_ref) in zip(Ns, grads_ref):
+        lin = getattr(attn, name)
+        assert olora.max_rel_err(lin.lora_A["default"].weight.grad, dA_ref) < TOL
+        assert olora.max_rel_err(lin.lora_B["default"].weight.grad, dB_ref) < TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,H,I,r", [(256, 512, 1024, 16), (100, 256, 704, 8)])
+def test_lora_mlp(M, H, I, r, dtype):
+    from fms_acceleration_foak.fused_ops.unsloth_lora.bnb.fast_lora import apply_lora_mlp_swiglu
+
+    alpha = 2.0 * r
+    mlp = torch.nn.Module()
+    ps = []
+    for i, (name, K, N) in enumerate((("gate_proj", H, I), ("up_proj", H, I), ("down_proj", I, H))):
+        lin, W, A, B = make_lora_nf4_linear(K, N, r, alpha, seed=20 + i, device="cuda", compute_dtype=dtype)
+        setattr(mlp, name, lin)
+        ps.append((W, _q(A, dtype), _q(B, dtype), alpha / r))
+    x = randn((1, M, H), 4, dtype) * 4.0
+    dy = randn((1, M, H), 5, dtype)
+    xg = x.cuda().requires_grad_(True)
+    out = apply_lora_mlp_swiglu(mlp, xg)
+    out.backward(dy.cuda())
+    out_ref, dx_ref, grads_ref, _ = olora.lora_mlp_autograd(x.float().reshape(-1, H), *ps, dy.float().reshape(-1, H))
+    assert olora.max_rel_err(out.reshape(-1, H), out_ref) < TOL
+    assert olora.max_rel_err(xg.grad.reshape(-1, H), dx_ref) < TOL
+    for name, (dA_ref, dB_ref) in zip(("gate_proj", "up_proj", "down_proj"), grads_ref):
+        lin = getattr(mlp, name)
+        assert olora.max_rel_err(lin.lora_A["default"].weight.grad, dA_ref) < 2 * TOL, name
+        assert olora.max_rel_err(lin.lora_B["default"].weight.grad, dB_ref) < 2 * TOL, name
+
+
+def test_lora_w_dropout_mask():
+    """dX's LoRA term is masked by (dropout(X) != 0) and dA uses the dropped activations
+    (fused_ops/unsloth_lora/bnb/fast_lora.py:431-456 of the reference)."""
+    from fms_acceleration_foak.fused_ops.unsloth_lora.bnb.fast_lora import apply_lora_o_v2
+
+    dtype, K, N, r, alpha, M = torch.bfloat16, 512, 256, 16, 32.0, 64
+    drop = MaskDropout(0.3, (M, K), seed=9)
+    lin, W, A, B = make_lora_nf4_linear(K, N, r, alpha, seed=3, device="cuda", dropout=drop.cuda())
+    x = randn((M, K), 2, dtype)
+    dy = randn((M, N), 3, dtype)
+    xg = x.cuda().requires_grad_(True)
+    y = apply_lora_o_v2(lin, xg)
+    y.backward(dy.cuda())
+    xd = x.float() * drop.mask.cpu()
+    Aq, Bq, s = _q(A, dtype), _q(B, dtype), alpha / r
+    y_ref = x.float() @ W + s * (xd @ Aq.t()) @ Bq.t()
+    dx_ref, dA_ref, dB_ref = olora.lora_w_manual(x.float(), W, Aq, Bq, s, dy.float(), xd=xd)
+    # lora_w_manual takes W as the matrix of the forward product; its dX uses W^T
+    assert olora.max_rel_err(y, y_ref) < TOL
+    assert olora.max_rel_err(xg.grad, dx_ref) < TOL
+    assert olora.max_rel_err(lin.lora_A["default"].weight.grad, dA_ref) < TOL
+    assert olora.max_rel_err(lin.lora_B["default"].weight.grad, dB_ref) < TOL
