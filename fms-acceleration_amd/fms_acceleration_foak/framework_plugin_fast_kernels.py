@@ -17,12 +17,17 @@ from .utils import filter_mp_rules
 def register_foak_model_patch_rules(base_type: str, filter_endswith: Set[str] = None, config=None):
     from fms_acceleration.model_patcher import ModelPatcher  # pylint: disable=import-outside-toplevel
 
-    from .models import granite, llama, mistral  # pylint: disable=import-outside-toplevel
+    # pylint: disable=import-outside-toplevel
+    from .models import granite, granitemoe, granitemoehybrid, granitemoeshared, llama, mistral, mixtral
 
     rules = [
         *granite.get_mp_rules(base_type, config),
+        *granitemoe.get_mp_rules(base_type),
+        *granitemoeshared.get_mp_rules(base_type),
+        *granitemoehybrid.get_mp_rules(base_type),
         *llama.get_mp_rules(base_type, config),
         *mistral.get_mp_rules(base_type, config),
+        *mixtral.get_mp_rules(base_type),
     ]
     if filter_endswith:
         rules = filter_mp_rules(rules, filter_endswith)

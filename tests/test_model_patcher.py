@@ -149,7 +149,9 @@ def test_fused_lora_rules_patch_llama_modules():
     train_args = type("T", (), {"bf16": True, "fp16": False})()
     with instantiate_model_patcher():
         plugin.augmentation(block, train_args, ())
-        assert set(ModelPatcher.rules) == {"llama-qkvo", "llama-mlp", "mistral-qkvo", "mistral-mlp", "granite-qkvo", "granite-mlp"}
+        assert set(ModelPatcher.rules) == {
+            "llama-qkvo", "llama-mlp", "mistral-qkvo", "mistral-mlp", "granite-qkvo", "granite-mlp",
+            "mixtral-qkvo", "granitemoe-qkvo", "granitemoeshared-qkvo", "granitemoehybrid-qkvo"}
         patch_model(block)
         ids = sorted(h.rule_id for h in ModelPatcher.history)
         assert ids == ["llama-mlp", "llama-qkvo-1", "llama-qkvo-2", "llama-qkvo-3", "llama-qkvo-4"]
