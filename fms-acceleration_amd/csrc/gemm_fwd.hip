@@ -3,8 +3,11 @@
 // Tiling (one workgroup = 4 waves = 256 lanes, one workgroup per CU):
 //   workgroup tile  256 tokens x 256 output columns, K walked in stages of 64
 //   wave tile       256 tokens x 64 columns = 8 x 2 MFMA 32x32x16 tiles, 256 fp32 accumulators
-//   X operand       global -> registers -> LDS (row stride 72 elements = 144 B, conflict-free for
-//                   16-byte fragment reads), double buffered, one barrier per stage
+//   X operand       global -> LDS directly (buffer loads with the LDS bit: no staging registers, no
+//                   ds_write), two stage buffers of 256 rows x 128 B, loaded one stage ahead.
+//                   A direct load places lane p's 16 bytes at slot p of a 1 KB block, so the
+//                   bank-conflict-free layout is obtained on the global side: slot c of row r holds
+//                   the 8-element chunk c ^ ((r >> 1) & 7) of that row.  One barrier per stage.
 //   W operand       never touches LDS: one packed int32 (8 nibbles along K at one column) is
 //                   exactly the 8-element MFMA fragment of the lane that owns that column, so each
 //                   lane loads its own words (a wave reads 2 x 128 B contiguous per load), unpacks
@@ -20,7 +23,7 @@ namespace {
 
 constexpr int BM = 256;
 constexpr int BK = 64;
-constexpr int LDS_STRIDE = BK + 8;  // elements
+constexpr int NBUF = 2;  // LDS stage buffers / register slots for the weight words
 constexpr int MT = 8;
 constexpr int NT = 2;
 
@@ -54,7 +57,15 @@ FMSA_DEVI FwdProjDev select_proj(const FwdArgs& a, int p) { return p == 0 ? a.p[
 // GPS = scale groups per 64-wide K stage: 1 for group_size % 64 == 0, 2 / 4 for group sizes 32 / 16.
 template <typename T, int GPS, bool KTAIL>
 __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t lds[2][BM * LDS_STRIDE];
+  // two separate arrays (not one 2-D array): every access names its buffer statically, which is
+  // what lets the compiler see that fragment reads of one buffer do not depend on the direct loads
+  // in flight into the other
+  __shared__ __attribute__((aligned(1024))) uint16_t lds0[BM * BK];
+  __shared__ __attribute__((aligned(1024))) uint16_t lds1[BM * BK];
+  auto lds_buf = [&](auto b_c) -> char* {
+    constexpr int b = decltype(b_c)::value;
+    return reinterpret_cast<char*>(b == 0 ? lds0 : lds1);
+  };
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -125,15 +136,24 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // ---- operand addressing: buffer loads (SGPR resource + 32-bit lane offset + SGPR offset) -----
   // No 64-bit address arithmetic in the loop, and lanes whose offset falls outside the resource
   // read zeros: rows past M need no predication.
-  // X tile: lane owns chunk (row = tid/8 + 32*i, oct = tid%8), i = 0..7.
-  const int oct = tid & 7;
+  // X tile: wave w fills rows 64w .. 64w+63 of a stage buffer with 8 direct loads; load i covers
+  // rows 64w+8i .. +7, lane p writes slot (p & 7) of row 64w + 8i + (p >> 3), which holds chunk
+  // (p & 7) ^ ((row >> 1) & 7) of that row.
+  const int uwave = __builtin_amdgcn_readfirstlane(wave);
   const int rows_valid = min(BM, a.M - m0);
   const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(a.X + (size_t)m0 * a.ldx, (size_t)rows_valid * a.ldx * 2);
   uint32_t x_off[8];
+  const int chunk_even = (lane & 7) ^ (lane >> 4);  // chunk fetched by loads 0, 2, 4, 6; odd loads: ^ 4
 #pragma unroll
-  for (int i = 0; i < 8; ++i) x_off[i] = (uint32_t)((((tid >> 3) + 32 * i) * a.ldx + 8 * oct) * 2);
-  const uint32_t lds_w_off = (uint32_t)(((tid >> 3) * LDS_STRIDE + oct * 8) * 2);
-  const uint32_t lds_r_off = (uint32_t)((l32 * LDS_STRIDE + 8 * half) * 2);
+  for (int i = 0; i < 8; ++i) {
+    const int row = 64 * wave + 8 * i + (lane >> 3);
+    const int chunk = chunk_even ^ (4 * (i & 1));
+    x_off[i] = (uint32_t)((row * a.ldx + 8 * chunk) * 2);
+  }
+  // fragment reads: row 32*mt + l32, chunk 2t + half -> slot (2t + half) ^ ((l32 >> 1) & 7)
+  uint32_t lds_r_off[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) lds_r_off[t] = (uint32_t)(l32 * (BK * 2) + 16 * ((2 * t + half) ^ ((l32 >> 1) & 7)));
   // weights: word (k8, col) at k8*N*4 + col*4; the lane part is (half*N + col)*4
   __amdgpu_buffer_rsrc_t q_rsrc[NT], sc_rsrc[NT], z_rsrc[NT];
   uint32_t q_off[NT], sc_off[NT], z_off[NT];
@@ -154,26 +174,33 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     q_last[j] = (uint32_t)((K >> 3) - 2) * Np[j] * 4;
   }
 
-  u32x4 a_st[8];        // X staging: 8 x 16 B per lane per stage
-  uint32_t q_cur[NT][4], q_nxt[NT][4];
+  // Weight words, scales and zero words in two register slots (slot = stage % 2), loaded one
+  // stage ahead together with X.
+  uint32_t qw[NBUF][NT][4];
+  uint16_t sc_raw[NBUF][NT][GPS];
+  uint32_t zw_raw[NBUF][NT][GPS];
   float sf[NT][GPS], sf16[NT][GPS], nsz[NT][GPS];
-  uint16_t sc_nxt[NT][GPS];
-  uint32_t zw_nxt[NT][GPS];
   // group index of the stage being loaded, advanced without a division when GPS == 1
   int g_ld[NT], k_in_g[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) g_ld[j] = k_in_g[j] = 0;
-
-  // issue the global loads of stage `st` (0 <= st < n_stages); nothing here may read the loaded
-  // registers, or the wave would wait for the load on the spot
-  auto load_stage = [&](int st) {
+  // issue the global loads of stage `st` (0 <= st < n_stages) into slot SB; nothing here may read
+  // the loaded registers, or the wave would wait for the load on the spot
+  auto load_stage = [&](int st, auto sb_c) {
+    constexpr int SB = decltype(sb_c)::value;
     const uint32_t x_soff = (uint32_t)st * (BK * 2);
     // K % 64 == 32 (KTAIL): in the last stage the upper half of the stage lies past K.  Its X
     // columns are forced out of range (zeros); the weight rows are clamped to valid memory.
-    uint32_t poison = 0;
-    if constexpr (KTAIL) poison = ((st * BK + 8 * oct) < K) ? 0u : 0x80000000u;
+    uint32_t poison[2] = {0u, 0u};
+    if constexpr (KTAIL) {
+      poison[0] = ((st * BK + 8 * chunk_even) < K) ? 0u : 0x80000000u;
+      poison[1] = ((st * BK + 8 * (chunk_even ^ 4)) < K) ? 0u : 0x80000000u;
+    }
+    char* lw = lds_buf(sb_c) + uwave * (64 * BK * 2);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) a_st[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_off[i] | poison, x_soff, 0);
+    for (int i = 0; i < 8; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (__attribute__((address_space(3))) void*)(lw + i * (8 * BK * 2)),
+                                               16, x_off[i] | poison[i & 1], x_soff, 0, 0);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       const uint32_t qs = (uint32_t)st * q_stage_bytes[j];
@@ -181,7 +208,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
       for (int t = 0; t < 4; ++t) {
         uint32_t so = qs + t * q_step_bytes[j];
         if constexpr (KTAIL) so = min(so, q_last[j]);
-        q_nxt[j][t] = __builtin_amdgcn_raw_buffer_load_b32(q_rsrc[j], q_off[j], so, 0);
+        qw[SB][j][t] = __builtin_amdgcn_raw_buffer_load_b32(q_rsrc[j], q_off[j], so, 0);
       }
 #pragma unroll
       for (int u = 0; u < GPS; ++u) {
@@ -192,8 +219,9 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
           const int ku = st * BK + u * (BK / GPS);
           gu = (ku < K ? ku : st * BK) / gs[j];
         }
-        sc_nxt[j][u] = __builtin_amdgcn_raw_buffer_load_b16(sc_rsrc[j], sc_off[j], (uint32_t)gu * Np[j] * 2, 0);
-        zw_nxt[j][u] = __builtin_amdgcn_raw_buffer_load_b32(z_rsrc[j], z_off[j], (uint32_t)gu * (Np[j] >> 3) * 4, 0);
+        gu = __builtin_amdgcn_readfirstlane(gu);  // uniform; keeps the scalar offsets out of vector registers
+        sc_raw[SB][j][u] = __builtin_amdgcn_raw_buffer_load_b16(sc_rsrc[j], sc_off[j], (uint32_t)gu * Np[j] * 2, 0);
+        zw_raw[SB][j][u] = __builtin_amdgcn_raw_buffer_load_b32(z_rsrc[j], z_off[j], (uint32_t)gu * (Np[j] >> 3) * 4, 0);
       }
       if constexpr (GPS == 1) {  // uniform scalar bookkeeping, no division
         k_in_g[j] += BK;
@@ -203,20 +231,16 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
       }
     }
   };
-  // registers -> LDS buffer `buf`, and make the prefetched weight words / scales current
-  auto commit_stage = [&](int buf) {
-    char* lw = reinterpret_cast<char*>(lds[buf]) + lds_w_off;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(lw + i * 32 * LDS_STRIDE * 2) = a_st[i];
+  // make the scales / zeros of slot SB current
+  auto commit_stage = [&](auto sb_c) {
+    constexpr int SB = decltype(sb_c)::value;
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) q_cur[j][t] = q_nxt[j][t];
-#pragma unroll
       for (int u = 0; u < GPS; ++u) {
-        sf[j][u] = fp16_bits_to_f32(sc_nxt[j][u]);
+        sf[j][u] = fp16_bits_to_f32(sc_raw[SB][j][u]);
         sf16[j][u] = sf[j][u] * 0.0625f;
-        const float z = (float)((zw_nxt[j][u] >> zshift[j]) & 0xFu) + zoff[j];
+        const float z = (float)((zw_raw[SB][j][u] >> zshift[j]) & 0xFu) + zoff[j];
         nsz[j][u] = -sf[j][u] * z;  // exact: 11-bit x 5-bit
       }
     }
@@ -225,16 +249,17 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // Software pipeline at the granularity of one 16-wide MFMA K step: while the 16 MFMAs of step t
   // run, the 8 X fragments of step t+1 are read from LDS and its 2 weight fragments are unpacked,
   // into the other half of xf / wf.  The stage barrier sits after step 2, so step 3 can already
-  // fetch step 0 of the next stage from the other LDS buffer.
+  // fetch step 0 of the next stage from the next LDS buffer.
   u32x4 xf[2][MT], wf[2][NT];
-  auto prefetch = [&](int buf, int t, auto par_c) {
+  auto prefetch = [&](auto sb_c, auto t_c, auto par_c) {
+    constexpr int SB = decltype(sb_c)::value;
+    constexpr int t = decltype(t_c)::value;
     constexpr int par = decltype(par_c)::value;
-    const char* lr = reinterpret_cast<const char*>(lds[buf]) + lds_r_off + t * 32;
+    const char* lr = lds_buf(sb_c) + lds_r_off[t];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-      xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * LDS_STRIDE * 2);
+    for (int mt = 0; mt < MT; ++mt) xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2);
 #pragma unroll
-    for (int j = 0; j < NT; ++j) wf[par][j] = dequant8<T>(q_cur[j][t], sf[j][t * GPS / 4], sf16[j][t * GPS / 4], nsz[j][t * GPS / 4]);
+    for (int j = 0; j < NT; ++j) wf[par][j] = dequant8<T>(qw[SB][j][t], sf[j][t * GPS / 4], sf16[j][t * GPS / 4], nsz[j][t * GPS / 4]);
   };
   auto mfma_step = [&](auto par_c) {
     constexpr int par = decltype(par_c)::value;
@@ -246,7 +271,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // One wave per SIMD issues strictly in order, and an MFMA that finds the matrix pipe busy stalls
   // everything behind it.  The other instructions of a step therefore have to sit BETWEEN its 16
   // MFMAs (each occupies the pipe for 8 issue slots): per MFMA 3 VALU, every second one an LDS
-  // read, and in step 0 also the global loads of the next stage with their scalar offset math.
+  // read, and in step 0 also the global loads of a later stage with their scalar offset math.
   auto interleave = [&](auto with_vmem_c) {
     constexpr bool with_vmem = decltype(with_vmem_c)::value;
 #pragma unroll
@@ -265,41 +290,54 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   };
   using WithVmem = std::integral_constant<bool, true>;
   using NoVmem = std::integral_constant<bool, false>;
-  using P0 = std::integral_constant<int, 0>;
-  using P1 = std::integral_constant<int, 1>;
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
 
-  load_stage(0);
-  commit_stage(0);
-  __syncthreads();
-  prefetch(0, 0, P0{});
-
-  for (int s = 0; s < n_stages; ++s) {
-    const int buf = s & 1;
-    // Global loads of the next stage are issued and consumed inside one iteration (steps 1-2 hide
-    // their latency): a load that stayed in flight across the loop back-edge would be waited for
-    // at the back-edge, where the compiler copies loop-carried registers.  The last iteration
-    // re-loads the final stage (no branch, so the loads can be interleaved with step 0's MFMAs);
-    // that data is committed to the idle LDS buffer and never read.
-    // step 0
-    load_stage(min(s + 1, n_stages - 1));
-    prefetch(buf, 1, P1{});
-    mfma_step(P0{});
-    interleave(WithVmem{});
-    // step 1
-    prefetch(buf, 2, P0{});
-    mfma_step(P1{});
+  // One 64-wide K stage out of LDS buffer / register slot SB = s % 2.  Steps 0-2 read the stage's
+  // fragments; then every wave waits for its own loads of stage s + 1 (issued one stage earlier),
+  // and the barrier makes all four waves' parts visible and closes the reads of buffer SB.  Step 3
+  // therefore is where the loads of stage s + 2 go out, into the buffer and register slot this
+  // stage has just vacated.  The last two stages re-load the final stage (no branch); that data
+  // is never read.
+  constexpr int WAIT_VM0 = 0x0F70;  // s_waitcnt vmcnt(0) only
+  auto stage = [&](int s, auto sb_c) {
+    constexpr int SB = decltype(sb_c)::value;
+    using S1 = std::integral_constant<int, SB ^ 1>;
+    prefetch(sb_c, I1{}, I1{});
+    mfma_step(I0{});
     interleave(NoVmem{});
-    // step 2, then hand the next stage over
-    prefetch(buf, 3, P1{});
-    mfma_step(P0{});
+    prefetch(sb_c, I2{}, I0{});
+    mfma_step(I1{});
     interleave(NoVmem{});
-    commit_stage(buf ^ 1);
+    prefetch(sb_c, I3{}, I1{});
+    mfma_step(I0{});
+    interleave(NoVmem{});
+    __builtin_amdgcn_s_waitcnt(WAIT_VM0);
+    commit_stage(S1{});
     __syncthreads();
-    // step 3
-    prefetch(buf ^ 1, 0, P0{});
-    mfma_step(P1{});
-    interleave(NoVmem{});
+    load_stage(min(s + 2, n_stages - 1), sb_c);
+    prefetch(S1{}, I0{}, I0{});
+    mfma_step(I1{});
+    interleave(WithVmem{});
+  };
+
+  load_stage(0, I0{});
+  __builtin_amdgcn_s_waitcnt(WAIT_VM0);
+  commit_stage(I0{});
+  __syncthreads();
+  load_stage(min(1, n_stages - 1), I1{});
+  prefetch(I0{}, I0{}, I0{});
+
+  // whole pairs in a single-exit loop (slots 0, 1), then the odd stage
+  const int n_full = n_stages & ~1;
+  int s = 0;
+  for (; s < n_full; s += NBUF) {
+    stage(s, I0{});
+    stage(s + 1, I1{});
   }
+  if (s < n_stages) stage(s, I0{});
 
   // ---- epilogue ---------------------------------------------------------------------------
   // accumulator register 4*i0+i1 of acc[mt][j] is Y[m0 + 32*mt + l32][col0[j] + 8*i0 + 4*half + i1]
