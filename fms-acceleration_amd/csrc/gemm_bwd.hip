@@ -10,14 +10,19 @@
 // Tiling (one workgroup = 4 waves, one workgroup per CU):
 //   workgroup tile  256 tokens x 256 output columns (32 qweight rows x 8 nibbles)
 //   wave w          nibbles 2w, 2w+1 of every word -> 256 tokens x 2 column tiles, 256 accumulators
-//                   (all four waves read the same words -- 4-bit data, served by L1/L2 -- but every
-//                   weight is unpacked by exactly one wave)
-//   dY operand      global -> registers -> LDS, double buffered, stages of 64 along N
-//   W operand       per 16-wide step and lane: 8 words, 8 fp16 scales and 8 fp32 (-scale*zero)
-//                   values of its row's group, fetched two steps ahead with buffer loads
-// Main loop: software pipeline at the granularity of one MFMA K step, as in the forward kernel
-// (LDS fragments and unpacked weights of step t+1 are produced while the 16 MFMAs of step t run,
-// and all other instructions are interleaved between those MFMAs).
+//                   (every weight is unpacked by exactly one wave)
+//   operands        everything a stage of 64 contraction columns needs is loaded straight into LDS
+//                   (buffer loads with the LDS bit), once per workgroup, double buffered:
+//                     dY tile   256 rows x 128 B, slot c of row r holds chunk c ^ ((r >> 1) & 7)
+//                     words     32 qweight rows x 256 B, slot c of row r holds chunk c ^ (r & 15)
+//                     scales    [8 groups][64] fp16 and (-scale*zero) [8 groups][64] fp32 of the
+//                               at most 8 quantisation groups the tile's 256 columns span
+//                   A direct load puts lane p's 16 bytes at slot p of a 1 KB block; the swizzles are
+//                   applied on the global side, and make the 16-byte fragment reads conflict-free.
+// Main loop: software pipeline at the granularity of one 16-wide MFMA K step.  While the 16 MFMAs
+// of step t run, the wave reads its 8 words, 8 scales and 8 offsets of step t+1 and the 8 dY
+// fragments from LDS and unpacks the two weight fragments; the loads of stage s+2 are issued in
+// the last step of stage s, after the barrier that closes the reads of the buffer they overwrite.
 // Epilogue: 64 tokens at a time the accumulators (and, separately, the LoRA term) are rounded to
 // the storage type, transposed through LDS and written as 16-byte row segments; mask and SwiGLU
 // backward are applied on that coalesced form.
@@ -27,7 +32,7 @@ namespace {
 
 constexpr int BM = 256;
 constexpr int BK = 64;
-constexpr int LDS_STRIDE = BK + 8;
+constexpr int MAX_TILE_GROUPS = 8;  // quantisation groups per 256 output columns (group_size >= 32)
 constexpr int MT = 8;
 constexpr int NT = 2;
 constexpr int EP_ROWS = 64;     // tokens per epilogue pass
@@ -60,21 +65,27 @@ struct BwdArgs {
 
 FMSA_DEVI BwdProjDev select_proj(const BwdArgs& a, int p) { return p == 0 ? a.p[0] : (p == 1 ? a.p[1] : a.p[2]); }
 
-// per-step weight operands of one lane: 8 words, 8 fp16 scales, 8 fp32 (-scale*zero)
-struct BSet {
-  u32x4 q0, q1, sc, nz0, nz1;
-};
-
 template <typename T, bool NTAIL>
 __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t lds[2][BM * LDS_STRIDE];
+  // separate arrays per stage buffer: every access names its buffer statically, so the compiler
+  // can tell fragment reads of one buffer from the direct loads in flight into the other
+  __shared__ __attribute__((aligned(1024))) uint16_t dy0[BM * BK];
+  __shared__ __attribute__((aligned(1024))) uint16_t dy1[BM * BK];
+  __shared__ __attribute__((aligned(1024))) uint32_t wq0[32 * BK];
+  __shared__ __attribute__((aligned(1024))) uint32_t wq1[32 * BK];
+  // per buffer 4 KB: scales [8][64] fp16 | offsets [8][64] fp32 | 1 KB written by the idle wave
+  __shared__ __attribute__((aligned(1024))) uint32_t tb0[1024];
+  __shared__ __attribute__((aligned(1024))) uint32_t tb1[1024];
+  __shared__ __attribute__((aligned(16))) uint16_t ep_planes[2 * EP_ROWS * EP_STRIDE];
+  auto dy_buf = [&](auto b_c) -> char* { return reinterpret_cast<char*>(decltype(b_c)::value == 0 ? dy0 : dy1); };
+  auto wq_buf = [&](auto b_c) -> char* { return reinterpret_cast<char*>(decltype(b_c)::value == 0 ? wq0 : wq1); };
+  auto tb_buf = [&](auto b_c) -> char* { return reinterpret_cast<char*>(decltype(b_c)::value == 0 ? tb0 : tb1); };
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int l32 = lane & 31;
   const int half = lane >> 5;
-  const int oct = tid & 7;
 
   int pid = xcd_remap(blockIdx.x, a.nbm * a.nbk);
   constexpr int GROUP_M = 8;
@@ -101,10 +112,22 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
 
-  const uint32_t lds_w_off = (uint32_t)(((tid >> 3) * LDS_STRIDE + oct * 8) * 2);
-  const uint32_t lds_r_off = (uint32_t)((l32 * LDS_STRIDE + 8 * half) * 2);
-  using P0 = std::integral_constant<int, 0>;
-  using P1 = std::integral_constant<int, 1>;
+  // ---- LDS read offsets (bytes) ----------------------------------------------------------------
+  // dY fragment of step t: row 32*mt + l32, chunk 2t + half
+  uint32_t dy_r[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) dy_r[t] = (uint32_t)(l32 * (BK * 2) + 16 * ((2 * t + half) ^ ((l32 >> 1) & 7)));
+  // words of step t: row l32, chunks 4t + 2*half + {0, 1}
+  uint32_t wq_r[4][2];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) wq_r[t][u] = (uint32_t)(l32 * 256 + 16 * ((4 * t + 2 * half + u) ^ (l32 & 15)));
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  constexpr int WAIT_VM0 = 0x0F70;  // s_waitcnt vmcnt(0) only
 
   for (int p = 0; p < a.n_proj; ++p) {
     const BwdProjDev P = select_proj(a, p);
@@ -113,62 +136,92 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     const int n_stages = (N + BK - 1) / BK;
     const int n_groups = (K + gs - 1) / gs;
 
-    // ---- operand addressing: buffer resources + 32-bit lane offsets + scalar offsets ----------
+    // ---- direct-load addressing: buffer resources + 32-bit lane offsets + scalar offsets ---------
+    // dY: wave w fills rows 64w .. 64w+63 with 8 loads; load i covers rows 64w+8i .. +7, lane q
+    // writes slot (q & 7) of row 64w + 8i + (q >> 3), i.e. fetches chunk (q & 7) ^ ((row >> 1) & 7).
     const __amdgpu_buffer_rsrc_t dy_rsrc = make_rsrc(P.dY + (size_t)m0 * P.lddy, (size_t)rows_valid * P.lddy * 2);
-    const uint32_t a_off = (uint32_t)(((tid >> 3) * P.lddy + 8 * oct) * 2);    // lane part
-    const uint32_t a_blk = __builtin_amdgcn_readfirstlane((uint32_t)(32 * P.lddy * 2));  // 32 rows further
+    const int dy_chunk_even = (lane & 7) ^ (lane >> 4);  // loads 0, 2, 4, 6; odd loads: ^ 4
+    uint32_t dy_off[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = 64 * wave + 8 * i + (lane >> 3);
+      dy_off[i] = (uint32_t)((row * P.lddy + 8 * (dy_chunk_even ^ (4 * (i & 1)))) * 2);
+    }
+    // words: wave w fills rows 8w .. 8w+7 with 2 loads of 4 rows; lane q writes slot (q & 15) of
+    // row 8w + 4i + (q >> 4), i.e. fetches the 4-word chunk (q & 15) ^ (row & 15).
     const __amdgpu_buffer_rsrc_t q_rsrc = make_rsrc(P.qweight, (size_t)(K >> 3) * N * 4);
+    uint32_t wq_off[2];
+    int wq_chunk[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = 8 * wave + 4 * i + (lane >> 4);
+      wq_chunk[i] = (lane & 15) ^ (row & 15);
+      const uint32_t dead_row = (k8base + row) < (K >> 3) ? 0u : 0x80000000u;  // rows past K read as zeros
+      wq_off[i] = (uint32_t)(((k8base + row) * N + 4 * wq_chunk[i]) * 4) | dead_row;
+    }
+    // tables: wave 0 loads the scales (lane q: group q >> 3, 8-column chunk q & 7), waves 1 and 2
+    // the offsets of groups 0-3 / 4-7 (lane q: group q >> 4, 4-column chunk q & 15); wave 3 issues
+    // the same instruction fully out of range, into the spare 1 KB.
+    const int g0 = (8 * k8base) / gs;
+    const int tb_elem = (wave == 0) ? 2 : 4;  // bytes per table element
+    const int tb_g = (wave == 0) ? (lane >> 3) : (4 * (wave - 1) + (lane >> 4));
+    const int tb_col = (wave == 0) ? 8 * (lane & 7) : 4 * (lane & 15);  // first column of the lane's chunk
     const __amdgpu_buffer_rsrc_t sc_rsrc = make_rsrc(P.scales, (size_t)n_groups * N * 2);
     const __amdgpu_buffer_rsrc_t nz_rsrc = make_rsrc(P.nsz, (size_t)n_groups * N * 4);
-    const int grp = (8 * k8) / gs;
-    const uint32_t dead = row_ok ? 0u : 0x80000000u;  // rows past K: out of range, read as zeros
-    const uint32_t q_voff = (uint32_t)((k8 * N + 8 * half) * 4) | dead;
-    const uint32_t sc_voff = (uint32_t)((grp * N + 8 * half) * 2) | dead;
-    const uint32_t nz_voff = (uint32_t)((grp * N + 8 * half) * 4) | dead;
+    const __amdgpu_buffer_rsrc_t tb_rsrc = (wave == 0) ? sc_rsrc : nz_rsrc;
+    const bool tb_live = (wave < 3) && (g0 + tb_g) < n_groups;
+    const uint32_t tb_off = (uint32_t)(((g0 + tb_g) * N + tb_col) * tb_elem) | (tb_live ? 0u : 0x80000000u);
+    // this lane's group inside the tile, and its table read offsets
+    const int gl = row_ok ? ((8 * k8) / gs - g0) : 0;
+    const uint32_t sc_r = (uint32_t)(gl * (BK * 2) + 8 * half * 2);
+    const uint32_t nz_r = (uint32_t)(1024 + gl * (BK * 4) + 8 * half * 4);
 
-    u32x4 a_st[4];  // the dY tile is staged in two halves of 128 rows
-    BSet bs[2];
     u32x4 xf[2][MT], wf[2][NT];
 
-    // global loads of one half (128 rows) of the dY tile of stage `st` (clamped: the surplus loads
-    // of the last iteration re-read the final stage and are never used)
-    auto load_A = [&](int st, int hf) {
-      const int stc = min(st, n_stages - 1);
-      const uint32_t soff = (uint32_t)stc * (BK * 2) + (uint32_t)(4 * hf) * a_blk;
-      uint32_t poison = 0;
-      if constexpr (NTAIL) poison = ((stc * BK + 8 * oct) < N) ? 0u : 0x80000000u;  // N % 64 == 32
+    // direct loads of stage `st` into buffer SB
+    auto load_stage = [&](int st, auto sb_c) {
+      const uint32_t n0 = (uint32_t)st * BK;
+      uint32_t dy_poison[2] = {0u, 0u}, wq_poison[2] = {0u, 0u}, tb_poison = 0u;
+      if constexpr (NTAIL) {  // N % 64 == 32: the upper half of the last stage lies past N
+        dy_poison[0] = ((int)n0 + 8 * dy_chunk_even < N) ? 0u : 0x80000000u;
+        dy_poison[1] = ((int)n0 + 8 * (dy_chunk_even ^ 4) < N) ? 0u : 0x80000000u;
+        wq_poison[0] = ((int)n0 + 4 * wq_chunk[0] < N) ? 0u : 0x80000000u;
+        wq_poison[1] = ((int)n0 + 4 * wq_chunk[1] < N) ? 0u : 0x80000000u;
+        tb_poison = ((int)n0 + tb_col < N) ? 0u : 0x80000000u;
+      }
+      char* ldy = dy_buf(sb_c) + wave * (64 * BK * 2);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) a_st[i] = __builtin_amdgcn_raw_buffer_load_b128(dy_rsrc, a_off | poison, soff + i * a_blk, 0);
-    };
-    auto commit_A = [&](int buf, int hf) {
-      char* lw = reinterpret_cast<char*>(lds[buf]) + lds_w_off + hf * (4 * 32 * LDS_STRIDE * 2);
+      for (int i = 0; i < 8; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(dy_rsrc, (__attribute__((address_space(3))) void*)(ldy + i * (8 * BK * 2)), 16,
+                                                 dy_off[i] | dy_poison[i & 1], n0 * 2, 0, 0);
+      char* lwq = wq_buf(sb_c) + wave * 2048;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lw + i * 32 * LDS_STRIDE * 2) = a_st[i];
+      for (int i = 0; i < 2; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(q_rsrc, (__attribute__((address_space(3))) void*)(lwq + i * 1024), 16,
+                                                 wq_off[i] | wq_poison[i], n0 * 4, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(tb_rsrc, (__attribute__((address_space(3))) void*)(tb_buf(sb_c) + wave * 1024), 16,
+                                               tb_off | tb_poison, n0 * (uint32_t)tb_elem, 0, 0);
     };
-    // weight operands of K step (st, t): columns n = 64*st + 16*t + 8*half .. +7 of the lane's row
-    auto load_B = [&](BSet& b, int st, int t) {
-      const int stc = min(st, n_stages - 1);
-      const uint32_t n = (uint32_t)(stc * BK + 16 * t);
-      uint32_t poison = 0;
-      if constexpr (NTAIL) poison = ((int)n + 8 * half < N) ? 0u : 0x80000000u;
-      b.q0 = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, q_voff | poison, n * 4, 0);
-      b.q1 = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (q_voff | poison) + 16, n * 4, 0);
-      b.sc = __builtin_amdgcn_raw_buffer_load_b128(sc_rsrc, sc_voff | poison, n * 2, 0);
-      b.nz0 = __builtin_amdgcn_raw_buffer_load_b128(nz_rsrc, nz_voff | poison, n * 4, 0);
-      b.nz1 = __builtin_amdgcn_raw_buffer_load_b128(nz_rsrc, (nz_voff | poison) + 16, n * 4, 0);
-    };
-    // LDS fragments of step t and the two unpacked weight fragments, into parity `par`
-    auto prefetch = [&](int buf, int t, const BSet& b, auto par_c) {
+    // LDS -> registers for step t of buffer SB: the 8 dY fragments and the two unpacked weight
+    // fragments, into parity `par`
+    auto prep = [&](auto sb_c, auto t_c, auto par_c) {
+      constexpr int t = decltype(t_c)::value;
       constexpr int par = decltype(par_c)::value;
-      const char* lr = reinterpret_cast<const char*>(lds[buf]) + lds_r_off + t * 32;
+      const char* lq = wq_buf(sb_c);
+      const char* lt = tb_buf(sb_c);
+      const u32x4 q0 = *reinterpret_cast<const u32x4*>(lq + wq_r[t][0]);
+      const u32x4 q1 = *reinterpret_cast<const u32x4*>(lq + wq_r[t][1]);
+      const u32x4 sc = *reinterpret_cast<const u32x4*>(lt + sc_r + t * 32);
+      const u32x4 nz0 = *reinterpret_cast<const u32x4*>(lt + nz_r + t * 64);
+      const u32x4 nz1 = *reinterpret_cast<const u32x4*>(lt + nz_r + t * 64 + 16);
+      const char* lr = dy_buf(sb_c) + dy_r[t];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * LDS_STRIDE * 2);
+      for (int mt = 0; mt < MT; ++mt) xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2);
       // this wave's byte of the 8 words: low nibble = column tile 0 (k = 8*k8 + 2*wave), high = tile 1
-      const uint32_t p01 = __builtin_amdgcn_perm(b.q0[1], b.q0[0], sel_pair);
-      const uint32_t p23 = __builtin_amdgcn_perm(b.q0[3], b.q0[2], sel_pair);
-      const uint32_t p45 = __builtin_amdgcn_perm(b.q1[1], b.q1[0], sel_pair);
-      const uint32_t p67 = __builtin_amdgcn_perm(b.q1[3], b.q1[2], sel_pair);
+      const uint32_t p01 = __builtin_amdgcn_perm(q0[1], q0[0], sel_pair);
+      const uint32_t p23 = __builtin_amdgcn_perm(q0[3], q0[2], sel_pair);
+      const uint32_t p45 = __builtin_amdgcn_perm(q1[1], q1[0], sel_pair);
+      const uint32_t p67 = __builtin_amdgcn_perm(q1[3], q1[2], sel_pair);
       const uint32_t x0 = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
       const uint32_t x1 = __builtin_amdgcn_perm(p67, p45, 0x05040100u);
       const uint32_t lo0 = opaque(x0 & 0x0F0F0F0Fu), hi0 = opaque((x0 >> 4) & 0x0F0F0F0Fu);
@@ -176,10 +229,10 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       float sfv[8], nzv[8];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        sfv[2 * i] = fp16_bits_to_f32((uint16_t)(b.sc[i] & 0xffffu));
-        sfv[2 * i + 1] = fp16_bits_to_f32((uint16_t)(b.sc[i] >> 16));
-        nzv[i] = __uint_as_float(b.nz0[i]);
-        nzv[4 + i] = __uint_as_float(b.nz1[i]);
+        sfv[2 * i] = fp16_bits_to_f32((uint16_t)(sc[i] & 0xffffu));
+        sfv[2 * i + 1] = fp16_bits_to_f32((uint16_t)(sc[i] >> 16));
+        nzv[i] = __uint_as_float(nz0[i]);
+        nzv[4 + i] = __uint_as_float(nz1[i]);
       }
       // element i of a fragment <-> column n + i; value = scale * nibble + (-scale * zero), exact in fp32
       wf[par][0][0] = pack2<T>(__builtin_fmaf(sfv[0], ubyte0(lo0), nzv[0]), __builtin_fmaf(sfv[1], ubyte1(lo0), nzv[1]));
@@ -198,69 +251,70 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[par][j], xf[par][mt], acc[mt][j]);
     };
-    // Everything else of a step sits between its 16 MFMAs (in-order issue, one wave per SIMD):
-    // per MFMA 3 VALU, an LDS read after every second one, and the step's buffer loads.
-    auto interleave = [&](auto n_vmem_c) {
-      constexpr int n_vmem = decltype(n_vmem_c)::value;
+    // Everything else of a step sits between its 16 MFMAs (in-order issue, one wave per SIMD).  The
+    // 13 LDS reads go first (one per MFMA; the 5 weight-operand reads lead, the unpack depends on
+    // them), the ~60 unpack instructions follow from the fourth MFMA on, and in the last step of a
+    // stage the 11 direct loads of a later stage are spread over the first MFMAs as well.
+    auto interleave = [&](auto with_vmem_c) {
+      constexpr bool with_vmem = decltype(with_vmem_c)::value;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
-        if ((i & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if (i < n_vmem) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if (i < 13) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (i >= 3) __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+        if (with_vmem && i < 11) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     };
-    using V9 = std::integral_constant<int, 9>;
-    using V5 = std::integral_constant<int, 5>;
+    using WithVmem = std::integral_constant<bool, true>;
+    using NoVmem = std::integral_constant<bool, false>;
 
-    // Pipeline: the weights of MFMA step u are loaded during step u-2 and unpacked during step u-1
-    // (two register sets, by parity of u); the dY tile of the next stage is loaded in two halves
-    // during steps 0 and 1 and written to the idle LDS buffer during steps 1 and 2.
-    __syncthreads();  // the previous projection's last LDS reads are done
-    load_A(0, 0);
-    commit_A(0, 0);
-    load_A(0, 1);
-    commit_A(0, 1);
-    load_B(bs[0], 0, 0);
-    load_B(bs[1], 0, 1);
-    __syncthreads();
-    prefetch(0, 0, bs[0], P0{});
-
-    for (int s = 0; s < n_stages; ++s) {
-      const int buf = s & 1;
-      // step 0
-      load_A(s + 1, 0);
-      load_B(bs[0], s, 2);
-      prefetch(buf, 1, bs[1], P1{});
-      mfma_step(P0{});
-      interleave(V9{});
-      // step 1
-      commit_A(buf ^ 1, 0);
-      load_A(s + 1, 1);
-      load_B(bs[1], s, 3);
-      prefetch(buf, 2, bs[0], P0{});
-      mfma_step(P1{});
-      interleave(V9{});
-      // step 2, then hand the next dY tile over
-      load_B(bs[0], s + 1, 0);
-      prefetch(buf, 3, bs[1], P1{});
-      mfma_step(P0{});
-      interleave(V5{});
-      commit_A(buf ^ 1, 1);
+    // One stage out of buffer SB = s % 2: steps 0-2 prepare steps 1-3 of the same buffer; then the
+    // wave waits for its own direct loads of stage s+1 (issued one stage earlier) and the barrier
+    // makes all four waves' parts visible and closes the reads of buffer SB, so step 3 can issue
+    // the loads of stage s+2 into it while preparing step 0 of stage s+1 from the other buffer.
+    // The last two stages re-load the final stage (no branch); that data is never used.
+    auto stage = [&](int s, auto sb_c) {
+      constexpr int SB = decltype(sb_c)::value;
+      using S1 = std::integral_constant<int, SB ^ 1>;
+      prep(sb_c, I1{}, I1{});
+      mfma_step(I0{});
+      interleave(NoVmem{});
+      prep(sb_c, I2{}, I0{});
+      mfma_step(I1{});
+      interleave(NoVmem{});
+      prep(sb_c, I3{}, I1{});
+      mfma_step(I0{});
+      interleave(NoVmem{});
+      __builtin_amdgcn_s_waitcnt(WAIT_VM0);
       __syncthreads();
-      // step 3
-      load_B(bs[1], s + 1, 1);
-      prefetch(buf ^ 1, 0, bs[0], P0{});
-      mfma_step(P1{});
-      interleave(V5{});
+      load_stage(min(s + 2, n_stages - 1), sb_c);
+      prep(S1{}, I0{}, I0{});
+      mfma_step(I1{});
+      interleave(WithVmem{});
+    };
+
+    __syncthreads();  // the previous projection's last LDS reads are done
+    load_stage(0, I0{});
+    __builtin_amdgcn_s_waitcnt(WAIT_VM0);
+    __syncthreads();
+    load_stage(min(1, n_stages - 1), I1{});
+    prep(I0{}, I0{}, I0{});
+
+    const int n_full = n_stages & ~1;
+    int s = 0;
+    for (; s < n_full; s += 2) {
+      stage(s, I0{});
+      stage(s + 1, I1{});
     }
+    if (s < n_stages) stage(s, I0{});
   }
 
   // ---- epilogue ---------------------------------------------------------------------------
   // register 4*i0+i1 of acc[mt][j] is dX[m0 + 32*mt + l32][8*(k8base + 8*i0 + 4*half + i1) + 2*wave + j]
+  __builtin_amdgcn_s_waitcnt(WAIT_VM0);  // the surplus direct loads of the last stage have landed
   __syncthreads();
-  uint16_t* base_plane = &lds[0][0];
+  uint16_t* base_plane = ep_planes;
   uint16_t* lora_plane = base_plane + EP_ROWS * EP_STRIDE;
   bool any_lora = false;
   for (int p = 0; p < a.n_proj; ++p) any_lora = any_lora || (select_proj(a, p).r > 0);
