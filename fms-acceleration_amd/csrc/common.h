@@ -132,7 +132,9 @@ FMSA_DEVI int xcd_remap(int pid, int total) {
 }
 
 // SiLU pieces with the reference's rounding points (UL/swiglu.py:26-33, 65-83).
-FMSA_DEVI float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// 1 / (1 + 2^(-x log2 e)) with the hardware exp2 and reciprocal (1 ulp each): four instructions
+// instead of the ~14 of an IEEE division; the result is rounded to the storage type right after.
+FMSA_DEVI float sigmoidf_(float x) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896341f)); }
 
 // Host-side launch helpers (api.hip)
 #define FMSA_CHECK_LAUNCH()                                   \

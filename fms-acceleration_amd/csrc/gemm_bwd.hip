@@ -320,6 +320,41 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
   for (int p = 0; p < a.n_proj; ++p) any_lora = any_lora || (select_proj(a, p).r > 0);
   const int kcol_lane = 8 * (k8base + l32) + 2 * wave;  // column whose A^T row this lane feeds to the LoRA MFMA
   const int k_tile0 = 8 * k8base;
+  // Coalesced side of the epilogue: lane = (row tid/32 of each group of 8 rows, 8-column chunk
+  // tid%32).  All global accesses go through buffer resources over the tile's rows, so rows past M
+  // and columns past K need no branches (loads return zero, stores are dropped), and the loads of a
+  // whole 64-row pass (e and g, or the mask source) are in flight one pass ahead of their use.
+  const bool swiglu = a.mode == FMSA_BWD_SWIGLU;
+  const int chunk = tid & 31;
+  const uint32_t col_dead = (k_tile0 + 8 * chunk) < K ? 0u : 0x80000000u;
+  const uint32_t eg_row_bytes = __builtin_amdgcn_readfirstlane((uint32_t)(a.ldeg * 2));
+  const uint32_t dx_row_bytes = __builtin_amdgcn_readfirstlane((uint32_t)(a.lddx * 2));
+  const uint32_t mk_row_bytes = __builtin_amdgcn_readfirstlane((uint32_t)(a.ldmask * 2));
+  const __amdgpu_buffer_rsrc_t e_rsrc = make_rsrc(a.e + (size_t)m0 * a.ldeg, swiglu ? (size_t)rows_valid * a.ldeg * 2 : 0);
+  const __amdgpu_buffer_rsrc_t g_rsrc = make_rsrc(a.g + (size_t)m0 * a.ldeg, swiglu ? (size_t)rows_valid * a.ldeg * 2 : 0);
+  const __amdgpu_buffer_rsrc_t h_rsrc = make_rsrc(a.h + (size_t)m0 * a.ldeg, swiglu ? (size_t)rows_valid * a.ldeg * 2 : 0);
+  const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(a.dX + (size_t)m0 * a.lddx, swiglu ? 0 : (size_t)rows_valid * a.lddx * 2);
+  const __amdgpu_buffer_rsrc_t mk_rsrc =
+      make_rsrc(a.mask_src + (size_t)m0 * a.ldmask, a.mask_src ? (size_t)rows_valid * a.ldmask * 2 : 0);
+  const uint32_t eg_voff = (uint32_t)(((tid >> 5) * a.ldeg + k_tile0 + 8 * chunk) * 2) | col_dead;
+  const uint32_t dx_voff = (uint32_t)(((tid >> 5) * a.lddx + k_tile0 + 8 * chunk) * 2) | col_dead;
+  const uint32_t mk_voff = (uint32_t)(((tid >> 5) * a.ldmask + k_tile0 + 8 * chunk) * 2) | col_dead;
+  u32x4 pre_a[2][EP_ROWS / 8], pre_b[2][EP_ROWS / 8];
+  auto issue_loads = [&](auto q_c) {
+    constexpr int q = decltype(q_c)::value;
+    if (swiglu) {
+#pragma unroll
+      for (int it = 0; it < EP_ROWS / 8; ++it) {
+        pre_a[q & 1][it] = __builtin_amdgcn_raw_buffer_load_b128(e_rsrc, eg_voff, (uint32_t)(EP_ROWS * q + 8 * it) * eg_row_bytes, 0);
+        pre_b[q & 1][it] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, eg_voff, (uint32_t)(EP_ROWS * q + 8 * it) * eg_row_bytes, 0);
+      }
+    } else if (a.mask_src && any_lora) {
+#pragma unroll
+      for (int it = 0; it < EP_ROWS / 8; ++it)
+        pre_a[q & 1][it] = __builtin_amdgcn_raw_buffer_load_b128(mk_rsrc, mk_voff, (uint32_t)(EP_ROWS * q + 8 * it) * mk_row_bytes, 0);
+    }
+  };
+  issue_loads(std::integral_constant<int, 0>{});
 
   static_for<0, MT / 2>([&](auto q_c) {
     constexpr int q = decltype(q_c)::value;
@@ -372,68 +407,64 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       }
     });
     __syncthreads();
-    // coalesced pass: 64 rows x 32 chunks of 8 columns
+      // coalesced pass: 64 rows x 32 chunks of 8 columns; iteration `it` handles row 8*it + tid/32
+    if (q + 1 < MT / 2) issue_loads(std::integral_constant<int, (q + 1 < MT / 2) ? q + 1 : q>{});
 #pragma unroll
     for (int it = 0; it < EP_ROWS * 32 / 256; ++it) {
-      const int idx = tid + 256 * it;
-      const int row = idx >> 5, chunk = idx & 31;
-      const int m = m0 + EP_ROWS * q + row;
-      const int k = k_tile0 + 8 * chunk;
-      if (m < a.M && k < K) {
-        const u32x4 bv = *reinterpret_cast<const u32x4*>(base_plane + row * EP_STRIDE + 8 * chunk);
-        u32x4 lv = {0u, 0u, 0u, 0u};
-        if (any_lora) lv = *reinterpret_cast<const u32x4*>(lora_plane + row * EP_STRIDE + 8 * chunk);
-        if (a.mode == FMSA_BWD_SWIGLU) {
-          const size_t off = (size_t)m * a.ldeg + k;
-          const u32x4 ev = *reinterpret_cast<const u32x4*>(a.e + off);
-          const u32x4 gv = *reinterpret_cast<const u32x4*>(a.g + off);
+      const int row = (tid >> 5) + 8 * it;
+      const uint32_t soff_rows = (uint32_t)(EP_ROWS * q + 8 * it);
+      const u32x4 bv = *reinterpret_cast<const u32x4*>(base_plane + row * EP_STRIDE + 8 * chunk);
+      u32x4 lv = {0u, 0u, 0u, 0u};
+      if (any_lora) lv = *reinterpret_cast<const u32x4*>(lora_plane + row * EP_STRIDE + 8 * chunk);
+      if (swiglu) {
+        const u32x4 ev = pre_a[q & 1][it];
+        const u32x4 gv = pre_b[q & 1][it];
+        u32x4 mv = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+        if (a.mask_src) mv = __builtin_amdgcn_raw_buffer_load_b128(mk_rsrc, mk_voff, soff_rows * mk_row_bytes, 0);
+        u32x4 hv, dgv, dev;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          float hh[2], dg[2], de[2];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const float e32 = j ? unpack_hi<T>(ev[w]) : unpack_lo<T>(ev[w]);
+            const float g32 = j ? unpack_hi<T>(gv[w]) : unpack_lo<T>(gv[w]);
+            const float b32 = j ? unpack_hi<T>(bv[w]) : unpack_lo<T>(bv[w]);
+            const float l32f = j ? unpack_hi<T>(lv[w]) : unpack_lo<T>(lv[w]);
+            const uint32_t mbits = (j ? (mv[w] >> 16) : mv[w]) & 0x7fffu;
+            const float se = sigmoidf_(e32);
+            const float f = unpack1<T>(pack1<T>(se * e32));
+            const float h = unpack1<T>(pack1<T>(f * g32));
+            // LoRA part of dh is masked by (dropout(h) != 0): mask_src holds dropout(h) when a
+            // dropout was applied, otherwise h itself (recomputed here) decides
+            const bool keep = a.mask_src ? (mbits != 0) : (h != 0.f);
+            const float DW = unpack1<T>(pack1<T>(keep ? b32 + l32f : b32));
+            hh[j] = h;
+            dg[j] = DW * f;                                    // d_g ("df", UL/swiglu.py:77)
+            const float dgt = unpack1<T>(pack1<T>(DW * g32));  // dg = DW * g in storage dtype (:79)
+            de[j] = dgt * se * (1.0f + e32 * (1.0f - se));     // d_e (:81-83)
+          }
+          hv[w] = pack2<T>(hh[0], hh[1]);
+          dgv[w] = pack2<T>(dg[0], dg[1]);
+          dev[w] = pack2<T>(de[0], de[1]);
+        }
+        __builtin_amdgcn_raw_buffer_store_b128(hv, h_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(dgv, e_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(dev, g_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
+      } else {
+        u32x4 ov = bv;
+        if (any_lora) {
           u32x4 mv = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-          if (a.mask_src) mv = *reinterpret_cast<const u32x4*>(a.mask_src + (size_t)m * a.ldmask + k);
-          u32x4 hv, dgv, dev;
+          if (a.mask_src) mv = pre_a[q & 1][it];
 #pragma unroll
           for (int w = 0; w < 4; ++w) {
-            float hh[2], dg[2], de[2];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const float e32 = j ? unpack_hi<T>(ev[w]) : unpack_lo<T>(ev[w]);
-              const float g32 = j ? unpack_hi<T>(gv[w]) : unpack_lo<T>(gv[w]);
-              const float b32 = j ? unpack_hi<T>(bv[w]) : unpack_lo<T>(bv[w]);
-              const float l32f = j ? unpack_hi<T>(lv[w]) : unpack_lo<T>(lv[w]);
-              const uint32_t mbits = (j ? (mv[w] >> 16) : mv[w]) & 0x7fffu;
-              const float se = sigmoidf_(e32);
-              const float f = unpack1<T>(pack1<T>(se * e32));
-              const float h = unpack1<T>(pack1<T>(f * g32));
-              // LoRA part of dh is masked by (dropout(h) != 0): mask_src holds dropout(h) when a
-              // dropout was applied, otherwise h itself (recomputed here) decides
-              const bool keep = a.mask_src ? (mbits != 0) : (h != 0.f);
-              const float DW = unpack1<T>(pack1<T>(keep ? b32 + l32f : b32));
-              hh[j] = h;
-              dg[j] = DW * f;                                    // d_g ("df", UL/swiglu.py:77)
-              const float dgt = unpack1<T>(pack1<T>(DW * g32));  // dg = DW * g in storage dtype (:79)
-              de[j] = dgt * se * (1.0f + e32 * (1.0f - se));     // d_e (:81-83)
-            }
-            hv[w] = pack2<T>(hh[0], hh[1]);
-            dgv[w] = pack2<T>(dg[0], dg[1]);
-            dev[w] = pack2<T>(de[0], de[1]);
+            // +-0 in the mask source count as zero
+            const float l0 = (mv[w] & 0x7fffu) ? unpack_lo<T>(lv[w]) : 0.f;
+            const float l1 = ((mv[w] >> 16) & 0x7fffu) ? unpack_hi<T>(lv[w]) : 0.f;
+            ov[w] = pack2<T>(unpack_lo<T>(bv[w]) + l0, unpack_hi<T>(bv[w]) + l1);
           }
-          *reinterpret_cast<u32x4*>(a.h + off) = hv;
-          *reinterpret_cast<u32x4*>(a.e + off) = dgv;
-          *reinterpret_cast<u32x4*>(a.g + off) = dev;
-        } else {
-          u32x4 ov = bv;
-          if (any_lora) {
-            u32x4 mv = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-            if (a.mask_src) mv = *reinterpret_cast<const u32x4*>(a.mask_src + (size_t)m * a.ldmask + k);
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-              // +-0 in the mask source count as zero
-              const float l0 = (mv[w] & 0x7fffu) ? unpack_lo<T>(lv[w]) : 0.f;
-              const float l1 = ((mv[w] >> 16) & 0x7fffu) ? unpack_hi<T>(lv[w]) : 0.f;
-              ov[w] = pack2<T>(unpack_lo<T>(bv[w]) + l0, unpack_hi<T>(bv[w]) + l1);
-            }
-          }
-          *reinterpret_cast<u32x4*>(a.dX + (size_t)m * a.lddx + k) = ov;
         }
+        __builtin_amdgcn_raw_buffer_store_b128(ov, dx_rsrc, dx_voff, soff_rows * dx_row_bytes, 0);
       }
     }
     __syncthreads();
