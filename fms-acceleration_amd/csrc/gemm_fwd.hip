@@ -23,6 +23,9 @@ namespace {
 
 constexpr int BM = 256;
 constexpr int BK = 64;
+constexpr int EP_ROWS = 64;          // tokens per epilogue pass
+constexpr int EP_STRIDE_L = 256 + 8;  // plane row stride (elements), linear: one plane of 256 columns
+constexpr int EP_STRIDE_S = 128 + 8;  // SwiGLU: three planes (e, g, h) of 128 columns
 constexpr int NBUF = 2;  // LDS stage buffers / register slots for the weight words
 constexpr int MT = 8;
 constexpr int NT = 2;
@@ -62,6 +65,8 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // in flight into the other
   __shared__ __attribute__((aligned(1024))) uint16_t lds0[BM * BK];
   __shared__ __attribute__((aligned(1024))) uint16_t lds1[BM * BK];
+  __shared__ __attribute__((aligned(16))) uint16_t ep_planes[3 * EP_ROWS * EP_STRIDE_S];  // >= EP_ROWS * EP_STRIDE_L
+  static_assert(3 * EP_STRIDE_S >= EP_STRIDE_L, "the linear plane must fit");
   auto lds_buf = [&](auto b_c) -> char* {
     constexpr int b = decltype(b_c)::value;
     return reinterpret_cast<char*>(b == 0 ? lds0 : lds1);
@@ -339,83 +344,167 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   }
   if (s < n_stages) stage(s, I0{});
 
-  // ---- epilogue ---------------------------------------------------------------------------
-  // accumulator register 4*i0+i1 of acc[mt][j] is Y[m0 + 32*mt + l32][col0[j] + 8*i0 + 4*half + i1]
-  static_for<0, MT>([&](auto mt_c) {
-    constexpr int mt = decltype(mt_c)::value;
-    const int m = m0 + 32 * mt + l32;
-    const bool m_ok = m < a.M;
+  // ---- LoRA term as extra contraction steps: acc += U[:, j0..j0+15] x (s * B[:, j0..j0+15])^T -------
+  // s * B is rounded to the storage type, the rounding point of the reference's
+  // `(X @ A.t()) @ (s * B.t())` (UL/gptq/fast_lora.py:167-169).  Rows past M read zeros through the
+  // buffer resource.
+  // One loop for both modes (no mode branch around the accumulators): tile j takes U and B of its
+  // own projection -- gate / up in SwiGLU mode, twice the same projection otherwise.
+  {
+    const uint16_t* Uj[NT];
+    const uint16_t* Bj[NT];
+    int rj[NT];
+    float sj[NT];
+    __amdgpu_buffer_rsrc_t u_rsrc[NT];
+    int r_max = 0;
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       const FwdProjDev P = select_proj(a, pj[j]);
-      if (P.r > 0) {
-        f32x16 tmp;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) tmp[i] = 0.f;
-        for (int j0 = 0; j0 < P.r; j0 += 16) {
-          const int ko = j0 + 8 * half;
-          u32x4 uf = {0u, 0u, 0u, 0u}, bf = {0u, 0u, 0u, 0u};
-          if (ko < P.r) {
-            if (m_ok) uf = *reinterpret_cast<const u32x4*>(P.U + (size_t)m * P.r + ko);
-            bf = *reinterpret_cast<const u32x4*>(P.B + (size_t)(col0[j] + l32) * P.r + ko);
-          }
-          tmp = mfma32<T>(bf, uf, tmp);
-        }
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[mt][j][i] += P.s * tmp[i];
-      }
-      if (P.bias) {
-#pragma unroll
-        for (int i0 = 0; i0 < 4; ++i0) {
-          const u32x2 bv = *reinterpret_cast<const u32x2*>(P.bias + col0[j] + 8 * i0 + 4 * half);
-          acc[mt][j][4 * i0 + 0] += unpack_lo<T>(bv[0]);
-          acc[mt][j][4 * i0 + 1] += unpack_hi<T>(bv[0]);
-          acc[mt][j][4 * i0 + 2] += unpack_lo<T>(bv[1]);
-          acc[mt][j][4 * i0 + 3] += unpack_hi<T>(bv[1]);
-        }
-      }
+      rj[j] = __builtin_amdgcn_readfirstlane(P.r);
+      sj[j] = P.s;
+      Uj[j] = P.U;
+      Bj[j] = P.B;
+      u_rsrc[j] = make_rsrc(P.U + (size_t)m0 * rj[j], rj[j] > 0 ? (size_t)rows_valid * rj[j] * 2 : 0);
+      r_max = max(r_max, rj[j]);
     }
-    if (!m_ok) return;
-    if (a.mode == FMSA_FWD_SWIGLU) {
-      if (!active[0]) return;
-      const FwdProjDev& Pe = a.p[0];
-      const FwdProjDev& Pg = a.p[1];
+    for (int j0 = 0; j0 < r_max; j0 += 16) {
+      const int ko = j0 + 8 * half;
+      u32x4 uf[NT][MT], bw[NT];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const bool live = ko < rj[j];
+        const uint32_t dead = live ? 0u : 0x80000000u;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          uf[j][mt] = __builtin_amdgcn_raw_buffer_load_b128(u_rsrc[j], (uint32_t)(((32 * mt + l32) * rj[j] + ko) * 2) | dead, 0, 0);
+        u32x4 bf = {0u, 0u, 0u, 0u};
+        if (live) bf = *reinterpret_cast<const u32x4*>(Bj[j] + (size_t)(col0[j] + l32) * rj[j] + ko);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) bw[j][w] = pack2<T>(sj[j] * unpack_lo<T>(bf[w]), sj[j] * unpack_hi<T>(bf[w]));
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(bw[j], uf[j][mt], acc[mt][j]);
+    }
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------
+  // accumulator register 4*i0+i1 of acc[mt][j] is Y[m0 + 32*mt + l32][col0[j] + 8*i0 + 4*half + i1].
+  // 64 tokens at a time the rounded outputs go through LDS planes (8-byte writes per lane) and
+  // leave as 16-byte row segments through buffer stores: rows past M and columns past N are
+  // dropped by the range check, so there are no branches.
+  const bool swiglu = a.mode == FMSA_FWD_SWIGLU;
+  const FwdProjDev PL = select_proj(a, pj[0]);
+  const int cb = swiglu ? bn * 128 : (bn - a.nblk_start[pj[0]]) * 256;  // first output column of the tile
+  const int lcol = swiglu ? wave * 32 : wave * 64;                      // wave's first column inside the tile
+  const int estride = swiglu ? EP_STRIDE_S : EP_STRIDE_L;              // plane row stride, elements
+  uint16_t* plane0 = ep_planes;
+  uint16_t* plane1 = ep_planes + EP_ROWS * EP_STRIDE_S;
+  uint16_t* plane2 = ep_planes + 2 * EP_ROWS * EP_STRIDE_S;
+  // coalesced side: linear 32 chunks per row (8 rows per sweep), SwiGLU 16 chunks per row (16 rows)
+  const int cchunk = swiglu ? (tid & 15) : (tid & 31);
+  const int crow = swiglu ? (tid >> 4) : (tid >> 5);
+  const int crows_per_it = swiglu ? 16 : 8;
+  const int n_out = swiglu ? a.p[0].N : PL.N;
+  const uint32_t col_dead = (cb + 8 * cchunk) < n_out ? 0u : 0x80000000u;
+  const int64_t ld0 = swiglu ? a.p[0].ldy : PL.ldy;
+  const __amdgpu_buffer_rsrc_t y0_rsrc = make_rsrc((swiglu ? a.p[0].Y : PL.Y) + (size_t)m0 * ld0, (size_t)rows_valid * ld0 * 2);
+  const __amdgpu_buffer_rsrc_t y1_rsrc = make_rsrc(a.p[1].Y + (size_t)m0 * a.p[1].ldy, swiglu ? (size_t)rows_valid * a.p[1].ldy * 2 : 0);
+  const __amdgpu_buffer_rsrc_t h_rsrc = make_rsrc(a.H + (size_t)m0 * a.ldh, swiglu ? (size_t)rows_valid * a.ldh * 2 : 0);
+  const uint32_t y0_voff = (uint32_t)((crow * ld0 + cb + 8 * cchunk) * 2) | col_dead;
+  const uint32_t y1_voff = (uint32_t)((crow * a.p[1].ldy + cb + 8 * cchunk) * 2) | col_dead;
+  const uint32_t h_voff = (uint32_t)((crow * a.ldh + cb + 8 * cchunk) * 2) | col_dead;
+  const uint32_t y0_row = __builtin_amdgcn_readfirstlane((uint32_t)(ld0 * 2));
+  const uint32_t y1_row = __builtin_amdgcn_readfirstlane((uint32_t)(a.p[1].ldy * 2));
+  const uint32_t h_row = __builtin_amdgcn_readfirstlane((uint32_t)(a.ldh * 2));
+  // bias of the lane's 4 x 4 columns per tile
+  float bias_v[NT][16];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const FwdProjDev P = select_proj(a, pj[j]);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) bias_v[j][i] = 0.f;
+    if (P.bias) {
 #pragma unroll
       for (int i0 = 0; i0 < 4; ++i0) {
-        const int n = col0[0] + 8 * i0 + 4 * half;
-        u32x2 ev, gv, hv;
-        float hf[4];
+        const u32x2 bv = *reinterpret_cast<const u32x2*>(P.bias + col0[j] + 8 * i0 + 4 * half);
+        bias_v[j][4 * i0 + 0] = unpack_lo<T>(bv[0]);
+        bias_v[j][4 * i0 + 1] = unpack_hi<T>(bv[0]);
+        bias_v[j][4 * i0 + 2] = unpack_lo<T>(bv[1]);
+        bias_v[j][4 * i0 + 3] = unpack_hi<T>(bv[1]);
+      }
+    }
+  }
+  __syncthreads();  // (the stage buffers are not reused, but all waves are past the main loop)
+
+  static_for<0, MT / 2>([&](auto q_c) {
+    constexpr int q = decltype(q_c)::value;
+    static_for<0, 2>([&](auto ml_c) {
+      constexpr int ml = decltype(ml_c)::value;
+      constexpr int mt = 2 * q + ml;
+      const int prow = 32 * ml + l32;
+      if (swiglu) {
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
-          ev[q] = pack2<T>(acc[mt][0][4 * i0 + 2 * q], acc[mt][0][4 * i0 + 2 * q + 1]);
-          gv[q] = pack2<T>(acc[mt][1][4 * i0 + 2 * q], acc[mt][1][4 * i0 + 2 * q + 1]);
-          // f = RNE(e32 * sigmoid(e32)) on the rounded e; h = RNE(f * g) on the rounded g
-          const float e0 = unpack_lo<T>(ev[q]), e1 = unpack_hi<T>(ev[q]);
-          const uint32_t fv = pack2<T>(e0 * sigmoidf_(e0), e1 * sigmoidf_(e1));
-          hf[2 * q] = unpack_lo<T>(fv) * unpack_lo<T>(gv[q]);
-          hf[2 * q + 1] = unpack_hi<T>(fv) * unpack_hi<T>(gv[q]);
+        for (int i0 = 0; i0 < 4; ++i0) {
+          u32x2 ev, gv, hv;
+          float hf[4];
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            ev[w] = pack2<T>(acc[mt][0][4 * i0 + 2 * w] + bias_v[0][4 * i0 + 2 * w],
+                             acc[mt][0][4 * i0 + 2 * w + 1] + bias_v[0][4 * i0 + 2 * w + 1]);
+            gv[w] = pack2<T>(acc[mt][1][4 * i0 + 2 * w] + bias_v[1][4 * i0 + 2 * w],
+                             acc[mt][1][4 * i0 + 2 * w + 1] + bias_v[1][4 * i0 + 2 * w + 1]);
+            // f = RNE(e32 * sigmoid(e32)) on the rounded e; h = RNE(f * g) on the rounded g
+            const float e0 = unpack_lo<T>(ev[w]), e1 = unpack_hi<T>(ev[w]);
+            const uint32_t fv = pack2<T>(e0 * sigmoidf_(e0), e1 * sigmoidf_(e1));
+            hf[2 * w] = unpack_lo<T>(fv) * unpack_lo<T>(gv[w]);
+            hf[2 * w + 1] = unpack_hi<T>(fv) * unpack_hi<T>(gv[w]);
+          }
+          hv[0] = pack2<T>(hf[0], hf[1]);
+          hv[1] = pack2<T>(hf[2], hf[3]);
+          const int o = prow * EP_STRIDE_S + lcol + 8 * i0 + 4 * half;
+          *reinterpret_cast<u32x2*>(plane0 + o) = ev;
+          *reinterpret_cast<u32x2*>(plane1 + o) = gv;
+          *reinterpret_cast<u32x2*>(plane2 + o) = hv;
         }
-        hv[0] = pack2<T>(hf[0], hf[1]);
-        hv[1] = pack2<T>(hf[2], hf[3]);
-        *reinterpret_cast<u32x2*>(Pe.Y + (size_t)m * Pe.ldy + n) = ev;
-        *reinterpret_cast<u32x2*>(Pg.Y + (size_t)m * Pg.ldy + n) = gv;
-        *reinterpret_cast<u32x2*>(a.H + (size_t)m * a.ldh + n) = hv;
+      } else {
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int i0 = 0; i0 < 4; ++i0) {
+            u32x2 yv;
+            yv[0] = pack2<T>(acc[mt][j][4 * i0 + 0] + bias_v[j][4 * i0 + 0], acc[mt][j][4 * i0 + 1] + bias_v[j][4 * i0 + 1]);
+            yv[1] = pack2<T>(acc[mt][j][4 * i0 + 2] + bias_v[j][4 * i0 + 2], acc[mt][j][4 * i0 + 3] + bias_v[j][4 * i0 + 3]);
+            *reinterpret_cast<u32x2*>(plane0 + prow * EP_STRIDE_L + lcol + 32 * j + 8 * i0 + 4 * half) = yv;
+          }
+      }
+    });
+    __syncthreads();
+    if (swiglu) {
+#pragma unroll
+      for (int it = 0; it < EP_ROWS / 16; ++it) {
+        const int row = crow + 16 * it;
+        const uint32_t srow = (uint32_t)(EP_ROWS * q + 16 * it);
+        const int o = row * EP_STRIDE_S + 8 * cchunk;
+        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane0 + o), y0_rsrc, y0_voff, srow * y0_row, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane1 + o), y1_rsrc, y1_voff, srow * y1_row, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane2 + o), h_rsrc, h_voff, srow * h_row, 0);
       }
     } else {
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        if (!active[j]) continue;
-        const FwdProjDev P = select_proj(a, pj[j]);
-#pragma unroll
-        for (int i0 = 0; i0 < 4; ++i0) {
-          u32x2 yv;
-          yv[0] = pack2<T>(acc[mt][j][4 * i0 + 0], acc[mt][j][4 * i0 + 1]);
-          yv[1] = pack2<T>(acc[mt][j][4 * i0 + 2], acc[mt][j][4 * i0 + 3]);
-          *reinterpret_cast<u32x2*>(P.Y + (size_t)m * P.ldy + col0[j] + 8 * i0 + 4 * half) = yv;
-        }
+      for (int it = 0; it < EP_ROWS / 8; ++it) {
+        const int row = crow + 8 * it;
+        const uint32_t srow = (uint32_t)(EP_ROWS * q + 8 * it);
+        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane0 + row * EP_STRIDE_L + 8 * cchunk), y0_rsrc,
+                                               y0_voff, srow * y0_row, 0);
       }
     }
+    __syncthreads();
   });
+  (void)estride;
+  (void)crows_per_it;
+  (void)active;
 }
 
 }  // namespace
