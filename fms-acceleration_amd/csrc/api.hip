@@ -6,10 +6,10 @@ int launch_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, hip
 int launch_gptq_permute_rows(const int32_t* qweight, const int32_t* perm, int K, int N, int32_t* out, hipStream_t st);
 int launch_permute_cols(const void* in, int64_t ld_in, const int32_t* perm, int M, int C, int gather, void* out,
                         int64_t ld_out, hipStream_t st);
-int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out,
+int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out, int64_t ldo,
                      hipStream_t st);
 int lora_grad_splits(int M, int C);
-int launch_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
+int launch_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
                      int act_dtype, int out_dtype, void* out, void* workspace, hipStream_t st);
 int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,
                          int64_t ldh, int act_dtype, hipStream_t st);
@@ -17,6 +17,8 @@ int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int m
                             void* g, void* h_out, int64_t ldeg, int act_dtype, hipStream_t st);
 
 int launch_gptq_nsz(const fmsa_gptq_weight* w, float* out, hipStream_t st);
+int launch_lora_pack(const void* A, const void* B, int r, int K, int N, int param_dtype, int act_dtype, void* A16, void* At16,
+                     void* B16, void* Bt16, hipStream_t st);
 int launch_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, hipStream_t st);
 int launch_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype, hipStream_t st);
 int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, int M, int I, int64_t ld, int act_dtype,
@@ -68,7 +70,7 @@ const char* fmsa_strerror(int code) {
   }
 }
 
-int fmsa_abi_version(void) { return 1; }
+int fmsa_abi_version(void) { return 2; }
 
 int fmsa_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, void* stream) {
   if (!w || !out) return FMSA_ERR_NULL;
@@ -96,14 +98,14 @@ int fmsa_permute_cols(const void* in, int64_t ld_in, const int32_t* perm, int M,
 }
 
 int fmsa_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out,
-                   void* stream) {
+                   int64_t ldout, void* stream) {
   if (!X || !Wd || !out) return FMSA_ERR_NULL;
-  if (M <= 0 || C <= 0 || r <= 0 || ldx < C) return FMSA_ERR_SHAPE;
+  if (M <= 0 || C <= 0 || r <= 0 || ldx < C || ldout < r) return FMSA_ERR_SHAPE;
   if (int rc = check_rank(r)) return rc;
   if (C % 8 != 0) return FMSA_ERR_SHAPE;
   if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
   if (!aligned16(X) || !aligned16(Wd) || ldx % 8 != 0) return FMSA_ERR_ALIGN;
-  return launch_lora_down(X, ldx, Wd, M, C, r, act_dtype, out, (hipStream_t)stream);
+  return launch_lora_down(X, ldx, Wd, M, C, r, act_dtype, out, ldout, (hipStream_t)stream);
 }
 
 size_t fmsa_lora_grad_workspace(int M, int C, int r) {
@@ -111,16 +113,16 @@ size_t fmsa_lora_grad_workspace(int M, int C, int r) {
   return (size_t)lora_grad_splits(M, C) * (size_t)r * (size_t)C * sizeof(float);
 }
 
-int fmsa_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
+int fmsa_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
                    int act_dtype, int out_dtype, void* out, void* workspace, size_t workspace_bytes, void* stream) {
   if (!L || !R || !out) return FMSA_ERR_NULL;
-  if (M <= 0 || C <= 0 || r <= 0 || ldr < C) return FMSA_ERR_SHAPE;
-  if (C % 8 != 0 || ldr % 8 != 0 || r % 8 != 0 || r > 128) return FMSA_ERR_SHAPE;
+  if (M <= 0 || C <= 0 || r <= 0 || ldr < C || ldl < r) return FMSA_ERR_SHAPE;
+  if (C % 8 != 0 || ldr % 8 != 0 || ldl % 8 != 0 || r % 8 != 0 || r > 128) return FMSA_ERR_SHAPE;
   if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
   if (out_dtype != FMSA_F16 && out_dtype != FMSA_BF16 && out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
   if (!workspace || workspace_bytes < fmsa_lora_grad_workspace(M, C, r)) return FMSA_ERR_WORKSPACE;
   if (!aligned16(R) || !aligned16(L) || !aligned16(workspace)) return FMSA_ERR_ALIGN;
-  return launch_lora_grad(L, R, ldr, M, C, r, scale, transpose_out, act_dtype, out_dtype, out, workspace,
+  return launch_lora_grad(L, ldl, R, ldr, M, C, r, scale, transpose_out, act_dtype, out_dtype, out, workspace,
                           (hipStream_t)stream);
 }
 
@@ -143,7 +145,8 @@ int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, in
     if (int rc = check_rank(s.r)) return rc;
     if (s.r > 0) {
       if (!s.U || !s.B) return FMSA_ERR_NULL;
-      if (!aligned16(s.U) || !aligned16(s.B)) return FMSA_ERR_ALIGN;
+      if (!aligned16(s.U) || !aligned16(s.B) || s.ldu % 8 != 0) return FMSA_ERR_ALIGN;
+      if (s.ldu < s.r) return FMSA_ERR_SHAPE;
     }
     if (s.bias && !aligned16(s.bias)) return FMSA_ERR_ALIGN;
   }
@@ -176,7 +179,8 @@ int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mod
     if (int rc = check_rank(s.r)) return rc;
     if (s.r > 0) {
       if (!s.T || !s.At) return FMSA_ERR_NULL;
-      if (!aligned16(s.T) || !aligned16(s.At)) return FMSA_ERR_ALIGN;
+      if (!aligned16(s.T) || !aligned16(s.At) || s.ldt % 8 != 0) return FMSA_ERR_ALIGN;
+      if (s.ldt < s.r) return FMSA_ERR_SHAPE;
     }
     if (s.mask_src && s.r > 0) {
       if (s.ldmask < K) return FMSA_ERR_SHAPE;
@@ -223,6 +227,15 @@ int fmsa_gptq_make_nsz(const fmsa_gptq_weight* w, float* out, void* stream) {
   if (int rc = check_weight(w, 0)) return rc;
   if (!aligned16(out)) return FMSA_ERR_ALIGN;
   return launch_gptq_nsz(w, out, (hipStream_t)stream);
+}
+
+int fmsa_lora_pack(const void* A, const void* B, int r, int K, int N, int param_dtype, int act_dtype, void* A16, void* At16,
+                   void* B16, void* Bt16, void* stream) {
+  if (!A || !B) return FMSA_ERR_NULL;
+  if (r <= 0 || K <= 0 || N <= 0) return FMSA_ERR_SHAPE;
+  if (param_dtype != FMSA_F32 && param_dtype != FMSA_BF16 && param_dtype != FMSA_F16) return FMSA_ERR_DTYPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  return launch_lora_pack(A, B, r, K, N, param_dtype, act_dtype, A16, At16, B16, Bt16, (hipStream_t)stream);
 }
 
 int fmsa_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, void* stream) {

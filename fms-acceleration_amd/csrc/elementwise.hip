@@ -63,6 +63,34 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* __restr
   *reinterpret_cast<u32x4*>(g + off) = dev;
 }
 
+// ---- adapter pack ------------------------------------------------------------------------------
+// One launch turns the two LoRA parameters (any float type) into the four activation-type copies
+// the GEMM kernels read: A [r, K], A^T [K, r], B [N, r], B^T [r, N].  Each conversion is one RNE
+// rounding of the parameter value (the `.to(dtype)` of UL/gptq/fast_lora.py:167).
+template <typename TIN> FMSA_DEVI float load_param(const void* p, int64_t i);
+template <> FMSA_DEVI float load_param<float>(const void* p, int64_t i) { return reinterpret_cast<const float*>(p)[i]; }
+template <> FMSA_DEVI float load_param<bf16_t>(const void* p, int64_t i) { return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]); }
+template <> FMSA_DEVI float load_param<f16_t>(const void* p, int64_t i) { return fp16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]); }
+
+template <typename TIN, typename T>
+__global__ __launch_bounds__(256) void lora_pack_kernel(const void* __restrict__ A, const void* __restrict__ B, int r, int K, int N,
+                                                        uint16_t* __restrict__ A16, uint16_t* __restrict__ At16,
+                                                        uint16_t* __restrict__ B16, uint16_t* __restrict__ Bt16) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < (int64_t)r * K) {
+    const int j = (int)(idx / K), k = (int)(idx % K);
+    const uint16_t v = pack1<T>(load_param<TIN>(A, idx));
+    if (A16) A16[idx] = v;
+    if (At16) At16[(int64_t)k * r + j] = v;
+  }
+  if (idx < (int64_t)N * r) {
+    const int n = (int)(idx / r), j = (int)(idx % r);
+    const uint16_t v = pack1<T>(load_param<TIN>(B, idx));
+    if (B16) B16[idx] = v;
+    if (Bt16) Bt16[(int64_t)j * N + n] = v;
+  }
+}
+
 }  // namespace
 
 int launch_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype, hipStream_t st) {
@@ -88,6 +116,29 @@ int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, i
   else
     hipLaunchKernelGGL(swiglu_bwd_kernel<f16_t>, grid, block, 0, st, (const uint16_t*)dh, lddh, (uint16_t*)e,
                        (uint16_t*)g, (uint16_t*)h, M, I, ld);
+  FMSA_CHECK_LAUNCH();
+  return FMSA_OK;
+}
+
+int launch_lora_pack(const void* A, const void* B, int r, int K, int N, int param_dtype, int act_dtype, void* A16, void* At16,
+                     void* B16, void* Bt16, hipStream_t st) {
+  const int64_t n = (int64_t)r * (K > N ? K : N);
+  dim3 grid((unsigned)((n + 255) / 256)), block(256);
+#define LAUNCH(TIN, TT)                                                                                          \
+  hipLaunchKernelGGL((lora_pack_kernel<TIN, TT>), grid, block, 0, st, A, B, r, K, N, (uint16_t*)A16, (uint16_t*)At16, \
+                     (uint16_t*)B16, (uint16_t*)Bt16)
+#define DISPATCH(TT)                                      \
+  do {                                                    \
+    if (param_dtype == FMSA_F32) LAUNCH(float, TT);       \
+    else if (param_dtype == FMSA_BF16) LAUNCH(bf16_t, TT); \
+    else LAUNCH(f16_t, TT);                               \
+  } while (0)
+  if (act_dtype == FMSA_BF16)
+    DISPATCH(bf16_t);
+  else
+    DISPATCH(f16_t);
+#undef DISPATCH
+#undef LAUNCH
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }

@@ -45,6 +45,7 @@ struct BwdProjDev {
   const uint16_t* dY;
   int64_t lddy;
   const uint16_t* T;
+  int64_t ldt;
   const uint16_t* At;  // [K, r]
   int N, group_size, r;
   float s;
@@ -381,7 +382,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
             const int ko = j0 + 8 * half;
             u32x4 tf = {0u, 0u, 0u, 0u}, af[NT] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
             if (ko < P.r) {
-              if (m_ok) tf = *reinterpret_cast<const u32x4*>(P.T + (size_t)m * P.r + ko);
+              if (m_ok) tf = *reinterpret_cast<const u32x4*>(P.T + (size_t)m * P.ldt + ko);
               if (row_ok) {
 #pragma unroll
                 for (int j = 0; j < NT; ++j)
@@ -516,6 +517,7 @@ int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int m
     d.dY = (const uint16_t*)s.dY;
     d.lddy = s.lddy;
     d.T = (const uint16_t*)s.T;
+    d.ldt = s.ldt;
     d.At = (const uint16_t*)s.At;
     d.N = s.w.N;
     d.group_size = s.w.group_size;

@@ -35,6 +35,7 @@ struct FwdProjDev {
   const uint16_t* scales;
   const int32_t* qzeros;
   const uint16_t* U;
+  int64_t ldu;
   const uint16_t* B;
   const uint16_t* bias;
   uint16_t* Y;
@@ -354,6 +355,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     const uint16_t* Uj[NT];
     const uint16_t* Bj[NT];
     int rj[NT];
+    int64_t lduj[NT];
     float sj[NT];
     __amdgpu_buffer_rsrc_t u_rsrc[NT];
     int r_max = 0;
@@ -364,7 +366,8 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
       sj[j] = P.s;
       Uj[j] = P.U;
       Bj[j] = P.B;
-      u_rsrc[j] = make_rsrc(P.U + (size_t)m0 * rj[j], rj[j] > 0 ? (size_t)rows_valid * rj[j] * 2 : 0);
+      lduj[j] = P.ldu;
+      u_rsrc[j] = make_rsrc(P.U + (size_t)m0 * P.ldu, rj[j] > 0 ? (size_t)rows_valid * P.ldu * 2 : 0);
       r_max = max(r_max, rj[j]);
     }
     for (int j0 = 0; j0 < r_max; j0 += 16) {
@@ -376,7 +379,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
         const uint32_t dead = live ? 0u : 0x80000000u;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          uf[j][mt] = __builtin_amdgcn_raw_buffer_load_b128(u_rsrc[j], (uint32_t)(((32 * mt + l32) * rj[j] + ko) * 2) | dead, 0, 0);
+          uf[j][mt] = __builtin_amdgcn_raw_buffer_load_b128(u_rsrc[j], (uint32_t)(((32 * mt + l32) * lduj[j] + ko) * 2) | dead, 0, 0);
         u32x4 bf = {0u, 0u, 0u, 0u};
         if (live) bf = *reinterpret_cast<const u32x4*>(Bj[j] + (size_t)(col0[j] + l32) * rj[j] + ko);
 #pragma unroll
@@ -529,6 +532,7 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
     d.scales = s.w.scales;
     d.qzeros = s.w.qzeros;
     d.U = (const uint16_t*)s.U;
+    d.ldu = s.ldu;
     d.B = (const uint16_t*)s.B;
     d.bias = (const uint16_t*)s.bias;
     d.Y = (uint16_t*)s.Y;

@@ -13,7 +13,7 @@ namespace {
 template <typename T, int RT>
 __global__ __launch_bounds__(256) void lora_down_kernel(const uint16_t* __restrict__ X, int64_t ldx,
                                                         const uint16_t* __restrict__ Wd, int M, int C, int r,
-                                                        uint16_t* __restrict__ out) {
+                                                        uint16_t* __restrict__ out, int64_t ldo) {
   __shared__ float red[4][RT][64][4];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -31,7 +31,7 @@ __global__ __launch_bounds__(256) void lora_down_kernel(const uint16_t* __restri
   for (int t = 0; t < RT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const uint16_t* xrow = X + (size_t)(m_ok ? m : 0) * ldx + 8 * q;
-#pragma unroll 2
+#pragma unroll 8
   for (int c0 = c_begin; c0 < c_end; c0 += 32) {
     const bool c_ok = (c0 + 8 * q) < c_end;
     u32x4 xf = {0u, 0u, 0u, 0u};
@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void lora_down_kernel(const uint16_t* __restri
     const float v = (red[0][t][ln][i] + red[1][t][ln][i]) + (red[2][t][ln][i] + red[3][t][ln][i]);
     const int row = blockIdx.x * 16 + 4 * (ln >> 4) + i;
     const int j = 16 * t + (ln & 15);
-    if (row < M && j < r) out[(size_t)row * r + j] = pack1<T>(v);
+    if (row < M && j < r) out[(size_t)row * ldo + j] = pack1<T>(v);
   }
 }
 
@@ -74,7 +74,7 @@ constexpr int LG_TC = 128;              // columns of R per workgroup
 constexpr int LG_RSTRIDE = LG_TC + 16;  // elements: 256 B + 32 B pad
 
 template <typename T, int RT>
-__global__ __launch_bounds__(256) void lora_grad_partial_kernel(const uint16_t* __restrict__ L,
+__global__ __launch_bounds__(256) void lora_grad_partial_kernel(const uint16_t* __restrict__ L, int64_t ldl,
                                                                 const uint16_t* __restrict__ R, int64_t ldr, int M,
                                                                 int C, int r, int rows_per_split,
                                                                 float* __restrict__ partial) {
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void lora_grad_partial_kernel(const uint16_t* 
     lst = u32x4{0u, 0u, 0u, 0u};
     if (l_thread) {
       const int m = m0 + l_row;
-      if (m < m_end && l_col_ok) lst = *reinterpret_cast<const u32x4*>(L + (size_t)m * r + 8 * l_chunk);
+      if (m < m_end && l_col_ok) lst = *reinterpret_cast<const u32x4*>(L + (size_t)m * ldl + 8 * l_chunk);
     }
   };
   auto commit_tile = [&](int buf) {
@@ -198,20 +198,22 @@ __global__ __launch_bounds__(256) void lora_grad_reduce_kernel(const float* __re
 
 int lora_grad_splits(int M, int C) {
   const int ncb = (C + LG_TC - 1) / LG_TC;
-  int splits = 2048 / ncb;
-  const int max_splits = (M + 63) / 64;  // at least two 32-token tiles per split
+  // about four workgroups per CU, but at least 512 tokens (16 tiles) per split: shorter splits spend
+  // their time in the prologue and in writing / re-reading partial sums
+  int splits = 1024 / ncb;
+  const int max_splits = (M + 511) / 512;
   if (splits > max_splits) splits = max_splits;
   if (splits < 1) splits = 1;
   return splits;
 }
 
 int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out,
-                     hipStream_t st) {
+                     int64_t ldo, hipStream_t st) {
   dim3 grid((M + 15) / 16), block(256);
   const int rt = (r + 15) / 16;
 #define LAUNCH(TT, RT)                                                                                           \
   hipLaunchKernelGGL((lora_down_kernel<TT, RT>), grid, block, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, \
-                     M, C, r, (uint16_t*)out)
+                     M, C, r, (uint16_t*)out, ldo)
 #define DISPATCH(TT)            \
   switch (rt) {                 \
     case 1: LAUNCH(TT, 1); break; \
@@ -230,7 +232,7 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
   return FMSA_OK;
 }
 
-int launch_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
+int launch_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
                      int act_dtype, int out_dtype, void* out, void* workspace, hipStream_t st) {
   const int splits = lora_grad_splits(M, C);
   int rows_per_split = (M + splits - 1) / splits;
@@ -238,8 +240,8 @@ int launch_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, in
   dim3 grid1((C + LG_TC - 1) / LG_TC, splits), block(256);
   const int rt = (r + 15) / 16;
 #define LAUNCH(TT, RT)                                                                                            \
-  hipLaunchKernelGGL((lora_grad_partial_kernel<TT, RT>), grid1, block, 0, st, (const uint16_t*)L, (const uint16_t*)R, \
-                     ldr, M, C, r, rows_per_split, (float*)workspace)
+  hipLaunchKernelGGL((lora_grad_partial_kernel<TT, RT>), grid1, block, 0, st, (const uint16_t*)L, ldl,               \
+                     (const uint16_t*)R, ldr, M, C, r, rows_per_split, (float*)workspace)
 #define DISPATCH(TT)                      \
   switch (rt) {                           \
     case 1: LAUNCH(TT, 1); break;         \

@@ -54,8 +54,9 @@ class _Proj:
         self.A_param, self.B_param = A, B
         self.r = 0 if A is None else A.shape[0]
         self.s = 0.0 if S is None else float(S)
-        self.A = None if A is None else A.detach().to(dtype).contiguous()  # [r, K]
-        self.B = None if B is None else B.detach().to(dtype).contiguous()  # [N, r]
+        self.A = self.At = self.B = self.Bt = None  # [r, K], [K, r], [N, r], [r, N] in the activation dtype
+        if A is not None:
+            self.A, self.At, self.B, self.Bt = fmsa_hip.lora_pack(A, B, dtype)
         self.dtype = dtype
 
     def dense(self):
@@ -68,7 +69,7 @@ class _Proj:
         U = None
         if self.r:
             U = fmsa_hip.lora_down(Xd, self.A)
-            Y.addmm_(U, self.B.t(), alpha=self.s)
+            Y.addmm_(U, self.Bt, alpha=self.s)
         if self.bias is not None:
             Y += self.bias
         return Y, U
@@ -89,7 +90,7 @@ class _Proj:
         return dA, dB
 
     def T(self, dY2):
-        return fmsa_hip.lora_down(dY2, self.B.t().contiguous()) if self.r else None
+        return fmsa_hip.lora_down(dY2, self.Bt) if self.r else None
 
 
 class LoRA_W(torch.autograd.Function):

@@ -37,6 +37,7 @@ EXPORTED_SYMBOLS = (
     "fmsa_swiglu_bwd",
     "fmsa_gptq_make_nsz",
     "fmsa_nf4_dequant",
+    "fmsa_lora_pack",
 )
 
 
@@ -72,6 +73,7 @@ class FwdProj(Structure):
     _fields_ = [
         ("w", GptqWeight),
         ("U", c_void_p),
+        ("ldu", c_int64),
         ("B", c_void_p),
         ("bias", c_void_p),
         ("Y", c_void_p),
@@ -88,6 +90,7 @@ class BwdProj(Structure):
         ("dY", c_void_p),
         ("lddy", c_int64),
         ("T", c_void_p),
+        ("ldt", c_int64),
         ("At", c_void_p),
         ("mask_src", c_void_p),
         ("ldmask", c_int64),
@@ -116,10 +119,10 @@ def lib() -> ctypes.CDLL:
     L.fmsa_gptq_dequant.argtypes = [POINTER(GptqWeight), c_int, c_void_p, c_void_p]
     L.fmsa_gptq_permute_rows.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]
     L.fmsa_permute_cols.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int64, c_void_p]
-    L.fmsa_lora_down.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]
+    L.fmsa_lora_down.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int64, c_void_p]
     L.fmsa_lora_grad_workspace.restype = c_size_t
     L.fmsa_lora_grad_workspace.argtypes = [c_int, c_int, c_int]
-    L.fmsa_lora_grad.argtypes = [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+    L.fmsa_lora_grad.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
                                  c_void_p, c_void_p, c_size_t, c_void_p]
     L.fmsa_gptq_lora_fwd.argtypes = [POINTER(FwdProj), c_int, c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                                      c_int, c_void_p]
@@ -129,6 +132,8 @@ def lib() -> ctypes.CDLL:
     L.fmsa_swiglu_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
     L.fmsa_gptq_make_nsz.argtypes = [POINTER(GptqWeight), c_void_p, c_void_p]
     L.fmsa_nf4_dequant.argtypes = [POINTER(Nf4Weight), c_int, c_void_p, c_void_p]
+    L.fmsa_lora_pack.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_void_p]
     for name in EXPORTED_SYMBOLS:
         getattr(L, name)  # AttributeError here means the library is stale: rebuild it
     _lib = L
@@ -209,14 +214,16 @@ def permute_cols(x2d, perm, gather: bool):
     return out
 
 
-def lora_down(x2d, wd):
-    """out [M, r] = x2d [M, C] @ wd [r, C]^T."""
+def lora_down(x2d, wd, out=None):
+    """out [M, r] = x2d [M, C] @ wd [r, C]^T.  `out` may be a column slice of a wider buffer."""
     M, C = x2d.shape
     r = wd.shape[0]
     assert wd.shape[1] == C and wd.is_contiguous() and wd.dtype == x2d.dtype and x2d.stride(1) == 1
-    out = torch.empty((M, r), dtype=x2d.dtype, device=x2d.device)
-    _check("fmsa_lora_down",
-           lib().fmsa_lora_down(_ptr(x2d), x2d.stride(0), _ptr(wd), M, C, r, act_enum(x2d.dtype), _ptr(out), _stream(out)))
+    if out is None:
+        out = torch.empty((M, r), dtype=x2d.dtype, device=x2d.device)
+    assert out.shape == (M, r) and out.stride(1) == 1 and out.dtype == x2d.dtype
+    _check("fmsa_lora_down", lib().fmsa_lora_down(_ptr(x2d), x2d.stride(0), _ptr(wd), M, C, r, act_enum(x2d.dtype), _ptr(out),
+                                                  out.stride(0), _stream(out)))
     return out
 
 
@@ -236,12 +243,12 @@ def lora_grad(L, R, scale: float, transpose_out: bool, out_dtype=torch.float32):
     """scale * L[M, r]^T @ R[M, C] -> [r, C] (or [C, r] when transpose_out)."""
     M, r = L.shape
     C = R.shape[1]
-    assert R.shape[0] == M and L.is_contiguous() and R.stride(1) == 1 and L.dtype == R.dtype
+    assert R.shape[0] == M and L.stride(1) == 1 and R.stride(1) == 1 and L.dtype == R.dtype
     out = torch.empty((C, r) if transpose_out else (r, C), dtype=out_dtype, device=R.device)
     nbytes = lib().fmsa_lora_grad_workspace(M, C, r)
     ws = _workspace(nbytes, R.device)
     _check("fmsa_lora_grad",
-           lib().fmsa_lora_grad(_ptr(L), _ptr(R), R.stride(0), M, C, r, float(scale), int(transpose_out),
+           lib().fmsa_lora_grad(_ptr(L), L.stride(0), _ptr(R), R.stride(0), M, C, r, float(scale), int(transpose_out),
                                 act_enum(R.dtype), _DTYPE_ENUM[out_dtype], _ptr(out), _ptr(ws), ws.numel(), _stream(out)))
     return out
 
@@ -256,7 +263,9 @@ def gptq_lora_fwd(x2d, projs: Sequence[dict], mode: int = FWD_LINEAR):
         w = p["w"]
         y = torch.empty((M, w.N), dtype=x2d.dtype, device=x2d.device)
         outs.append(y)
-        arr[i] = FwdProj(w, _ptr(p.get("U")) if p["r"] else None, _ptr(p.get("B")) if p["r"] else None,
+        U = p.get("U") if p["r"] else None
+        assert U is None or U.stride(1) == 1
+        arr[i] = FwdProj(w, _ptr(U), 0 if U is None else U.stride(0), _ptr(p.get("B")) if p["r"] else None,
                          _ptr(p.get("bias")), _ptr(y), y.stride(0), int(p["r"]), float(p["s"] or 0.0))
     h = None
     if mode == FWD_SWIGLU:
@@ -278,7 +287,9 @@ def gptq_lora_bwd_dx(projs: Sequence[dict], M: int, K: int, mode: int = BWD_LINE
         dy = p["dY"]
         assert dy.stride(1) == 1
         ms = p.get("mask_src")
-        arr[i] = BwdProj(p["w"], _ptr(p["nsz"]), _ptr(dy), dy.stride(0), _ptr(p.get("T")) if p["r"] else None,
+        T = p.get("T") if p["r"] else None
+        assert T is None or T.stride(1) == 1
+        arr[i] = BwdProj(p["w"], _ptr(p["nsz"]), _ptr(dy), dy.stride(0), _ptr(T), 0 if T is None else T.stride(0),
                          _ptr(p.get("At")) if p["r"] else None, _ptr(ms), 0 if ms is None else ms.stride(0),
                          int(p["r"]), float(p["s"] or 0.0))
     if mode == BWD_SWIGLU:
@@ -322,3 +333,30 @@ def nf4_dequant(packed, absmax_q, absmax2, code2, code, offset: float, shape, bl
     out = torch.empty((N, K), dtype=out_dtype, device=packed.device)
     _check("fmsa_nf4_dequant", lib().fmsa_nf4_dequant(ctypes.byref(w), _DTYPE_ENUM[out_dtype], _ptr(out), _stream(out)))
     return out
+
+
+def lora_pack(A, B, act_dtype, A16_out=None):
+    """(A16 [r, K], At16 [K, r], B16 [N, r], Bt16 [r, N]) in `act_dtype` from lora_A.weight [r, K] and
+    lora_B.weight [N, r] (fp32 / bf16 / fp16), one launch.  `A16_out` (contiguous [r, K]) lets the
+    caller place A16 inside a larger stacked matrix."""
+    if not (A.is_cuda and B.is_cuda):
+        raise RuntimeError("fmsa_hip needs GPU tensors")
+    A, B = A.detach(), B.detach()
+    if A.dtype != B.dtype:
+        B = B.to(A.dtype)
+    A = A if A.is_contiguous() else A.contiguous()
+    B = B if B.is_contiguous() else B.contiguous()
+    r, K = A.shape
+    N = B.shape[0]
+    own_a = A16_out is None
+    buf = torch.empty(r * K * (2 if own_a else 1) + 2 * r * N, dtype=act_dtype, device=A.device)
+    o = 0
+    if own_a:
+        A16_out, o = buf[: r * K].view(r, K), r * K
+    assert A16_out.shape == (r, K) and A16_out.is_contiguous() and A16_out.dtype == act_dtype
+    At16 = buf[o : o + r * K].view(K, r)
+    B16 = buf[o + r * K : o + r * K + N * r].view(N, r)
+    Bt16 = buf[o + r * K + N * r :].view(r, N)
+    _check("fmsa_lora_pack", lib().fmsa_lora_pack(_ptr(A), _ptr(B), r, K, N, _DTYPE_ENUM[A.dtype], act_enum(act_dtype),
+                                                  _ptr(A16_out), _ptr(At16), _ptr(B16), _ptr(Bt16), _stream(A)))
+    return A16_out, At16, B16, Bt16

@@ -87,23 +87,33 @@ int fmsa_permute_cols(const void* in, int64_t ld_in, const int32_t* perm, int M,
  * Skinny LoRA GEMMs.
  * ------------------------------------------------------------------------------------------ */
 
-/* out[M, r] = X[M, C] * Wd[r, C]^T, fp32 accumulate, one rounding to act_dtype.
+/* out[M, r] (row stride ldout >= r) = X[M, C] * Wd[r, C]^T, fp32 accumulate, one rounding to act_dtype.
  * Covers `X @ A.t()` of matmul_lora (UL/gptq/fast_lora.py:166-167) with Wd = lora_A.weight
  * [r, K], and `dY @ B` of the backward (:822) with Wd = lora_B.weight^T [r, N].
- * r % 8 == 0, r <= 128, C % 8 == 0. */
+ * r % 8 == 0, r <= 128, C % 8 == 0.  Adapters that share X can be stacked: Wd = [A_q; A_k; A_v]
+ * gives their U's side by side in one pass over X, and ldout lets several calls write side by side
+ * into one [M, sum r] buffer. */
 int fmsa_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype,
-                   void* out, void* stream);
+                   void* out, int64_t ldout, void* stream);
 
-/* out = scale * L[M, r]^T * R[M, C]   (a reduction over the M tokens), written as
+/* out = scale * L[M, r]^T * R[M, C]   (a reduction over the M tokens; L has row stride ldl >= r), written as
  *   [r, C] when transpose_out == 0   (dA = s * (dY B)^T Xd,  UL/gptq/fast_lora.py:822,824,842)
  *   [C, r] when transpose_out == 1   (dB = s * dY^T (Xd A^T), :823,825,843)
  * Deterministic two-pass reduction: partial sums over fixed M-chunks go to `workspace`
  * (fp32, fmsa_lora_grad_workspace() bytes) and are summed in a fixed order.
  * out_dtype: FMSA_F32, FMSA_BF16 or FMSA_F16. */
 size_t fmsa_lora_grad_workspace(int M, int C, int r);
-int fmsa_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, int r, float scale,
+int fmsa_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale,
                    int transpose_out, int act_dtype, int out_dtype, void* out, void* workspace,
                    size_t workspace_bytes, void* stream);
+
+/* The four activation-type copies of one adapter that the kernels above and below read, in one
+ * launch: A16 [r, K], At16 [K, r] from A = lora_A.weight [r, K]; B16 [N, r], Bt16 [r, N] from
+ * B = lora_B.weight [N, r].  Each value is the parameter rounded once (RNE) to act_dtype -- the
+ * `A.to(dtype)`, `B.to(dtype)` of matmul_lora (UL/gptq/fast_lora.py:167) plus the transposes its
+ * backward takes (:822-831).  param_dtype: FMSA_F32, FMSA_BF16 or FMSA_F16.  Outputs may be NULL. */
+int fmsa_lora_pack(const void* A, const void* B, int r, int K, int N, int param_dtype, int act_dtype,
+                   void* A16, void* At16, void* B16, void* Bt16, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Fused forward:  Y_p = X * deq(W_p) + s_p * U_p * B_p^T (+ bias_p)   for 1..3 projections
@@ -115,6 +125,7 @@ int fmsa_lora_grad(const void* L, const void* R, int64_t ldr, int M, int C, int 
 typedef struct fmsa_fwd_proj {
   fmsa_gptq_weight w;
   const void* U;    /* [M, r] act_dtype = Xd * A^T (fmsa_lora_down); NULL when r == 0 */
+  int64_t ldu;      /* row stride of U, >= r, % 8 == 0                                 */
   const void* B;    /* [N, r] act_dtype = lora_B.weight                               */
   const void* bias; /* [N] act_dtype or NULL                                           */
   void* Y;          /* [M, N] act_dtype                                                */
@@ -144,6 +155,7 @@ typedef struct fmsa_bwd_proj {
   const void* dY;    /* [M, N] act_dtype */
   int64_t lddy;
   const void* T;     /* [M, r] act_dtype = dY * B; NULL when r == 0 */
+  int64_t ldt;       /* row stride of T, >= r, % 8 == 0 */
   const void* At;    /* [K, r] act_dtype = lora_A.weight^T (contiguous) */
   const void* mask_src; /* [M, K] act_dtype or NULL; every non-NULL entry of one call must be the same */
   int64_t ldmask;

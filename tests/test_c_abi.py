@@ -29,8 +29,8 @@ def test_header_and_library_agree():
 
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(fmsa_hip.GptqWeight) == 48
-    assert ctypes.sizeof(fmsa_hip.FwdProj) == 96
-    assert ctypes.sizeof(fmsa_hip.BwdProj) == 112
+    assert ctypes.sizeof(fmsa_hip.FwdProj) == 104
+    assert ctypes.sizeof(fmsa_hip.BwdProj) == 120
 
 
 def _w(K=64, N=64, gs=64, q=0x1000, s=0x2000, z=0x3000, g=None, zo=0):
@@ -55,9 +55,9 @@ def test_fused_forward_validation():
     f = lib.fmsa_gptq_lora_fwd
 
     def proj(**kw):
-        d = dict(w=_w(), U=0x4000, B=0x5000, bias=None, Y=0x6000, ldy=64, r=16, s=1.0)
+        d = dict(w=_w(), U=0x4000, ldu=16, B=0x5000, bias=None, Y=0x6000, ldy=64, r=16, s=1.0)
         d.update(kw)
-        return fmsa_hip.FwdProj(d["w"], d["U"], d["B"], d["bias"], d["Y"], d["ldy"], d["r"], d["s"])
+        return fmsa_hip.FwdProj(d["w"], d["U"], d["ldu"], d["B"], d["bias"], d["Y"], d["ldy"], d["r"], d["s"])
 
     def call(p, n=1, X=0x7000, ldx=64, M=8, mode=0, H=None, ldh=0, dt=1):
         arr = (fmsa_hip.FwdProj * 3)(*([p] * 3))
@@ -72,6 +72,8 @@ def test_fused_forward_validation():
     assert call(proj(w=_w(gs=24, K=96)), ldx=96) == -5            # group size not a multiple of 16
     assert call(proj(r=12)) == -5
     assert call(proj(U=None)) == -1
+    assert call(proj(ldu=8)) == -2                        # U rows shorter than the rank
+    assert call(proj(ldu=20)) == -3                       # U rows not 16-byte aligned
     assert call(proj(Y=None)) == -1
     assert call(proj(ldy=32)) == -2
     assert call(proj(), n=1, mode=1) == -2                # SwiGLU needs exactly gate + up
@@ -80,21 +82,24 @@ def test_fused_forward_validation():
 
 def test_bwd_and_skinny_validation():
     lib = fmsa_hip.lib()
-    p = fmsa_hip.BwdProj(_w(), 0x9000, 0xA000, 64, 0xB000, 0xC000, None, 0, 16, 1.0)
+    p = fmsa_hip.BwdProj(_w(), 0x9000, 0xA000, 64, 0xB000, 16, 0xC000, None, 0, 16, 1.0)
     arr = (fmsa_hip.BwdProj * 3)(p, p, p)
     f = lib.fmsa_gptq_lora_bwd_dx
     assert f(arr, 1, 8, 0, None, 0, None, None, None, 0, 1, None) == -1       # dX missing
     assert f(arr, 1, 8, 1, None, 0, None, None, None, 0, 1, None) == -1       # e/g/h missing
     assert f(arr, 2, 8, 1, None, 0, 0x1000, 0x2000, 0x3000, 64, 1, None) == -2  # SwiGLU takes one projection
-    p2 = fmsa_hip.BwdProj(_w(), None, 0xA000, 64, 0xB000, 0xC000, None, 0, 16, 1.0)
+    p2 = fmsa_hip.BwdProj(_w(), None, 0xA000, 64, 0xB000, 16, 0xC000, None, 0, 16, 1.0)
     assert f((fmsa_hip.BwdProj * 1)(p2), 1, 8, 0, 0xD000, 64, None, None, None, 0, 1, None) == -1  # nsz missing
-    m1 = fmsa_hip.BwdProj(_w(), 0x9000, 0xA000, 64, 0xB000, 0xC000, 0xE000, 64, 16, 1.0)
-    m2 = fmsa_hip.BwdProj(_w(), 0x9000, 0xA000, 64, 0xB000, 0xC000, 0xF000, 64, 16, 1.0)
+    m1 = fmsa_hip.BwdProj(_w(), 0x9000, 0xA000, 64, 0xB000, 16, 0xC000, 0xE000, 64, 16, 1.0)
+    m2 = fmsa_hip.BwdProj(_w(), 0x9000, 0xA000, 64, 0xB000, 16, 0xC000, 0xF000, 64, 16, 1.0)
     assert f((fmsa_hip.BwdProj * 2)(m1, m2), 2, 8, 0, 0xD000, 64, None, None, None, 0, 1, None) == -5  # two masks
-    assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 64, 12, 1, 0x3000, None) == -5
-    assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 60, 16, 1, 0x3000, None) == -2
+    assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 64, 12, 1, 0x3000, 16, None) == -5
+    assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 60, 16, 1, 0x3000, 16, None) == -2
+    assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 64, 16, 1, 0x3000, 8, None) == -2   # ldout < r
     assert lib.fmsa_lora_grad_workspace(8192, 4096, 16) > 0
-    assert lib.fmsa_lora_grad(0x1000, 0x2000, 64, 8, 64, 16, 1.0, 0, 1, 2, 0x3000, None, 0, None) == -6
+    assert lib.fmsa_lora_grad(0x1000, 16, 0x2000, 64, 8, 64, 16, 1.0, 0, 1, 2, 0x3000, None, 0, None) == -6
+    assert lib.fmsa_lora_pack(None, 0x1000, 16, 64, 64, 2, 1, None, None, None, None, None) == -1
+    assert lib.fmsa_lora_pack(0x1000, 0x2000, 16, 64, 64, 2, 2, None, None, None, None, None) == -4
     assert lib.fmsa_swiglu_fwd(0x1000, 0x2000, 0x3000, 8, 60, 64, 1, None) == -2
     assert lib.fmsa_gptq_permute_rows(0x1000, 0x2000, 64, 64, 0x1000, None) == -5  # in place
 
