@@ -171,6 +171,7 @@ int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mod
   for (int p = 0; p < n_proj; ++p) {
     const fmsa_bwd_proj& s = projs[p];
     if (int rc = check_weight(&s.w, 8)) return rc;
+    if (s.w.group_size < 32) return FMSA_ERR_UNSUPPORTED;  // at most 8 groups per 256 output columns
     if (s.w.K != K) return FMSA_ERR_SHAPE;
     if (!s.dY || !s.nsz) return FMSA_ERR_NULL;
     if (s.lddy < s.w.N) return FMSA_ERR_SHAPE;

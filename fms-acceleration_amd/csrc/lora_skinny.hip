@@ -7,53 +7,69 @@
 namespace {
 
 // ---- lora_down ----------------------------------------------------------------------------------
-// One workgroup = 16 tokens; its 4 waves split C into 4 contiguous quarters and each runs
-// MFMA 16x16x32 over its quarter (X fragment straight from global: 16 rows x 64 B per load), then
-// the four partial [16 x r] tiles are summed through LDS in a fixed order.
-template <typename T, int RT>
+// One workgroup = 16 * MTL tokens; its 4 waves split C into 4 contiguous quarters and each runs
+// MFMA 16x16x32 over its quarter (X fragments straight from global: 16 rows x 64 B per load; a Wd
+// fragment is loaded once per step and used for all MTL token tiles), then the four partial
+// [16 * MTL x r] tiles are summed through LDS in a fixed order.
+template <typename T, int RT, int MTL>
 __global__ __launch_bounds__(256) void lora_down_kernel(const uint16_t* __restrict__ X, int64_t ldx,
                                                         const uint16_t* __restrict__ Wd, int M, int C, int r,
                                                         uint16_t* __restrict__ out, int64_t ldo) {
-  __shared__ float red[4][RT][64][4];
+  __shared__ float red[4][MTL][RT][64][4];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int l16 = lane & 15, q = lane >> 4;
-  const int m = blockIdx.x * 16 + l16;
-  const bool m_ok = m < M;
+  const int m_base = blockIdx.x * (16 * MTL);
   // quarter boundaries in units of 32 columns
   const int n32 = (C + 31) / 32;
   const int per = (n32 + 3) / 4;
   const int c_begin = wave * per * 32;
   const int c_end = min(C, (wave + 1) * per * 32);
 
-  f32x4 acc[RT];
+  f32x4 acc[MTL][RT];
 #pragma unroll
-  for (int t = 0; t < RT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int u = 0; u < MTL; ++u)
+#pragma unroll
+    for (int t = 0; t < RT; ++t) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const uint16_t* xrow = X + (size_t)(m_ok ? m : 0) * ldx + 8 * q;
-#pragma unroll 8
+  const uint16_t* xrow[MTL];
+  bool m_ok[MTL];
+#pragma unroll
+  for (int u = 0; u < MTL; ++u) {
+    const int m = m_base + 16 * u + l16;
+    m_ok[u] = m < M;
+    xrow[u] = X + (size_t)(m_ok[u] ? m : 0) * ldx + 8 * q;
+  }
+#pragma unroll 4
   for (int c0 = c_begin; c0 < c_end; c0 += 32) {
     const bool c_ok = (c0 + 8 * q) < c_end;
-    u32x4 xf = {0u, 0u, 0u, 0u};
-    if (m_ok && c_ok) xf = *reinterpret_cast<const u32x4*>(xrow + c0);
+    u32x4 xf[MTL];
+#pragma unroll
+    for (int u = 0; u < MTL; ++u) {
+      xf[u] = u32x4{0u, 0u, 0u, 0u};
+      if (m_ok[u] && c_ok) xf[u] = *reinterpret_cast<const u32x4*>(xrow[u] + c0);
+    }
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
       const int j = 16 * t + l16;
       u32x4 wf = {0u, 0u, 0u, 0u};
       if (j < r && c_ok) wf = *reinterpret_cast<const u32x4*>(Wd + (size_t)j * C + c0 + 8 * q);
-      acc[t] = mfma16<T>(xf, wf, acc[t]);  // D[i = token][j = rank]
+#pragma unroll
+      for (int u = 0; u < MTL; ++u) acc[u][t] = mfma16<T>(xf[u], wf, acc[u][t]);  // D[i = token][j = rank]
     }
   }
 #pragma unroll
-  for (int t = 0; t < RT; ++t)
+  for (int u = 0; u < MTL; ++u)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][t][lane][i] = acc[t][i];
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][u][t][lane][i] = acc[u][t][i];
   __syncthreads();
-  // lane l of the tile holds D[4*(l>>4) + i][l & 15]; 256 threads sum RT*256 outputs
-  for (int o = tid; o < RT * 256; o += 256) {
-    const int t = o >> 8, ln = (o >> 2) & 63, i = o & 3;
-    const float v = (red[0][t][ln][i] + red[1][t][ln][i]) + (red[2][t][ln][i] + red[3][t][ln][i]);
-    const int row = blockIdx.x * 16 + 4 * (ln >> 4) + i;
+  // lane l of a tile holds D[4*(l>>4) + i][l & 15]; 256 threads sum MTL*RT*256 outputs
+  for (int o = tid; o < MTL * RT * 256; o += 256) {
+    const int u = o / (RT * 256), t = (o >> 8) % RT, ln = (o >> 2) & 63, i = o & 3;
+    const float v = (red[0][u][t][ln][i] + red[1][u][t][ln][i]) + (red[2][u][t][ln][i] + red[3][u][t][ln][i]);
+    const int row = m_base + 16 * u + 4 * (ln >> 4) + i;
     const int j = 16 * t + (ln & 15);
     if (row < M && j < r) out[(size_t)row * ldo + j] = pack1<T>(v);
   }
@@ -209,11 +225,19 @@ int lora_grad_splits(int M, int C) {
 
 int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out,
                      int64_t ldo, hipStream_t st) {
-  dim3 grid((M + 15) / 16), block(256);
+  // 32 tokens per workgroup once that still leaves a workgroup per CU (halves the re-reads of Wd)
+  const int mtl = (M >= 32 * 256 && r <= 64) ? 2 : 1;
+  dim3 grid((M + 16 * mtl - 1) / (16 * mtl)), block(256);
   const int rt = (r + 15) / 16;
-#define LAUNCH(TT, RT)                                                                                           \
-  hipLaunchKernelGGL((lora_down_kernel<TT, RT>), grid, block, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, \
-                     M, C, r, (uint16_t*)out, ldo)
+#define LAUNCH(TT, RT)                                                                                                   \
+  do {                                                                                                                   \
+    if (mtl == 2)                                                                                                        \
+      hipLaunchKernelGGL((lora_down_kernel<TT, RT, 2>), grid, block, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, \
+                         M, C, r, (uint16_t*)out, ldo);                                                                  \
+    else                                                                                                                 \
+      hipLaunchKernelGGL((lora_down_kernel<TT, RT, 1>), grid, block, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, \
+                         M, C, r, (uint16_t*)out, ldo);                                                                  \
+  } while (0)
 #define DISPATCH(TT)            \
   switch (rt) {                 \
     case 1: LAUNCH(TT, 1); break; \

@@ -203,6 +203,7 @@ def test_bwd_dx_three_projections(dtype):
     M, K, r, s = 320, 1024, 16, 2.0
     Ns = [1024, 256, 288]
     x = randn((M, K), 2, dtype)
+    x[::5, ::3] = 0  # masked entries: no LoRA contribution from any projection
     ws = [make_gptq(K, N, 128, seed=10 + i) for i, N in enumerate(Ns)]
     ABs = [olora.make_lora(K, N, r, 20 + i) for i, N in enumerate(Ns)]
     dys = [randn((M, N), 30 + i, dtype) for i, N in enumerate(Ns)]
@@ -224,11 +225,13 @@ def test_bwd_swiglu(M, H, I, dtype):
     wd = make_gptq(I, H, 128 if I % 128 == 0 else 32 * 11, seed=5)  # down: I -> H, so K = I, N = H
     Ad, Bd = olora.make_lora(I, H, r, 6)
     e = randn((M, I), 7, dtype)
+    e[::9, ::4] = 0  # h = silu(0) * g = 0 there: the LoRA part of dh is masked
     g = randn((M, I), 8, dtype)
     dy = randn((M, H), 9, dtype)
     e_d, g_d = dev(e).clone(), dev(g).clone()
     h = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(wd, dev(dy), Ad, Bd, s, dtype)], M, I, fmsa_hip.BWD_SWIGLU, e=e_d, g=g_d)
-    dh_ref = dy.float() @ wd["dense"].t() + (dy.float() @ Bd.to(dtype).float()) @ (s * Ad.to(dtype).float())
+    h_mask = (olora.swiglu_fwd(e, g) != 0).float()
+    dh_ref = dy.float() @ wd["dense"].t() + h_mask * ((dy.float() @ Bd.to(dtype).float()) @ (s * Ad.to(dtype).float()))
     # h does not depend on the GEMM: it must match the reference's rounding points closely
     h_ref, _, _ = olora.swiglu_bwd(dh_ref.to(dtype), e, g)
     assert olora.max_rel_err(h.cpu(), h_ref.float()) < 4e-3
