@@ -29,6 +29,25 @@ M_TOKENS, HIDDEN, INTER, N_HEADS, N_KV, HEAD_DIM = 8192, 4096, 14336, 32, 8, 128
 RANK, GROUP = 16, 128
 ALPHA_MLP, ALPHA_ATTN = 16.0, 32.0
 
+# Bytes per launch that cross between L2 and the fabric (MALL / HBM) for the two launches that can
+# be the dominant one: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, each scaled by what the
+# same counter reads for the 1 GiB device copy of --calibration-copy (factors 2.000 and 1.000);
+# profiles/gptq_lora_gemms_llama3_8b_hbm_traffic_pmc.txt holds the runs.
+ROOFLINE_TRAFFIC_BYTES = {
+    "gptq_lora_fwd<swiglu> K=4096 N=14336+14336": 1451.3e6 + 723.0e6,
+    "gptq_lora_bwd_dx<linear> K=4096 N=14336+14336": 1541.5e6 + 74.5e6,
+}
+_W_BYTES = HIDDEN * INTER // 2 + (HIDDEN // GROUP) * INTER * 2 + (HIDDEN // GROUP) * INTER // 2  # packed + scales + zeros
+# algorithmic bytes of the same launches
+ALGORITHMIC_BYTES = {
+    # X once, gate and up weights once, U and B, the three outputs e, g, h
+    "gptq_lora_fwd<swiglu> K=4096 N=14336+14336":
+        M_TOKENS * HIDDEN * 2 + 2 * _W_BYTES + 2 * (M_TOKENS * RANK * 2 + INTER * RANK * 2) + 3 * M_TOKENS * INTER * 2,
+    # d_g and d_e once, up and gate weights + fp32 offset tables once, T and A^T, the mask source X, dX
+    "gptq_lora_bwd_dx<linear> K=4096 N=14336+14336":
+        2 * M_TOKENS * INTER * 2 + 2 * (_W_BYTES + (HIDDEN // GROUP) * INTER * 4) + 2 * (M_TOKENS * RANK * 2 + HIDDEN * RANK * 2)
+        + 2 * M_TOKENS * HIDDEN * 2,
+}
 
 def proj_flops(M, K, N, r):
     """Algorithmic FLOPs of one projection, forward + backward: base fwd + base dX (frozen W has no
@@ -99,61 +118,55 @@ def make_step(attn, mlp, M, device, dtype):
     return step
 
 
-def time_kernels(M, device, dtype):
-    """Average duration of each GEMM launch of the step, measured with events recorded on the
-    stream the kernels are launched on (torch's current stream)."""
-    import torch
+class LaunchTimer:
+    """Brackets every fused-GEMM launch of the step with a pair of events recorded on the stream the
+    kernel is launched on (torch's current stream), by wrapping the two ctypes entry points."""
 
-    import fmsa_hip
+    def __init__(self, M):
+        import fmsa_hip
 
-    torch.manual_seed(0)
+        self.mod, self.M, self.records = fmsa_hip, M, []
+        self._fwd, self._bwd = fmsa_hip.gptq_lora_fwd, fmsa_hip.gptq_lora_bwd_dx
 
-    def rand_weight(K, N):
-        qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 8, N), dtype=torch.int32, device=device)
-        qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // GROUP, N // 8), dtype=torch.int32, device=device)
-        sc = (torch.rand(K // GROUP, N, device=device) * 0.004 + 0.001).half()
-        return (qw, sc, qz), fmsa_hip.make_weight(qw, sc, qz, None, GROUP)
+    def _timed(self, label, flop, fn, *args, **kw):
+        import torch
 
-    def timeit(fn, n=10, warm=3):
-        for _ in range(warm):
-            fn()
         s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
         s.record()
-        for _ in range(n):
-            fn()
+        out = fn(*args, **kw)
         e.record()
-        torch.cuda.synchronize()
-        return s.elapsed_time(e) / n
+        self.records.append((label, flop, s, e))
+        return out
 
-    r, H, I = RANK, HIDDEN, INTER
-    rn = lambda *s: (torch.randn(*s, device=device) * 0.5).to(dtype)  # noqa: E731
-    x, dy, dgi = rn(M, H), rn(M, H), rn(M, I)
-    keep_g, Wg = rand_weight(H, I)
-    keep_u, Wu = rand_weight(H, I)
-    keep_d, Wd = rand_weight(I, H)
-    A_h, B_i, A_i, B_h = rn(r, H), rn(I, r), rn(r, I), rn(H, r)
-    U = fmsa_hip.lora_down(x, A_h)
-    pg = {"w": Wg, "U": U, "B": B_i, "bias": None, "r": r, "s": 1.0}
-    pu = {"w": Wu, "U": U, "B": B_i, "bias": None, "r": r, "s": 1.0}
-    e, g, h = fmsa_hip.gptq_lora_fwd(x, [pg, pu], fmsa_hip.FWD_SWIGLU)
-    Ud = fmsa_hip.lora_down(h, A_i)
-    pd = {"w": Wd, "U": Ud, "B": B_h, "bias": None, "r": r, "s": 1.0}
-    Td = fmsa_hip.lora_down(dy, B_h.t().contiguous())
-    bd = {"w": Wd, "nsz": fmsa_hip.gptq_make_nsz(Wd, dy.device), "dY": dy, "T": Td, "At": A_i.t().contiguous(), "mask_src": None, "r": r, "s": 1.0}
-    Tu = fmsa_hip.lora_down(dgi, B_i.t().contiguous())
-    bu = {"w": Wu, "nsz": fmsa_hip.gptq_make_nsz(Wu, dgi.device), "dY": dgi, "T": Tu, "At": A_h.t().contiguous(), "mask_src": x, "r": r, "s": 1.0}
-    bg = dict(bu, w=Wg, nsz=fmsa_hip.gptq_make_nsz(Wg, x.device))
-    e2, g2 = e.clone(), g.clone()
-    out = {}
-    f1 = 2.0 * M * H * I
-    out["gptq_lora_fwd<swiglu> gate+up"] = (timeit(lambda: fmsa_hip.gptq_lora_fwd(x, [pg, pu], fmsa_hip.FWD_SWIGLU)), 2 * f1)
-    out["gptq_lora_fwd<linear> down"] = (timeit(lambda: fmsa_hip.gptq_lora_fwd(h, [pd])), f1)
-    out["gptq_lora_bwd_dx<swiglu> down"] = (
-        timeit(lambda: fmsa_hip.gptq_lora_bwd_dx([bd], M, I, fmsa_hip.BWD_SWIGLU, e=e2, g=g2)), f1)
-    out["gptq_lora_bwd_dx<linear> up+gate"] = (timeit(lambda: fmsa_hip.gptq_lora_bwd_dx([bu, bg], M, H)), 2 * f1)
-    del keep_g, keep_u, keep_d
-    return out
+    def __enter__(self):
+        mod, M = self.mod, self.M
+
+        def fwd(x2d, projs, mode=mod.FWD_LINEAR):
+            K, Ns = projs[0]["w"].K, [p["w"].N for p in projs]
+            flop = sum(2.0 * M * K * n + 2.0 * M * p["r"] * n for n, p in zip(Ns, projs))
+            kind = "swiglu" if mode == mod.FWD_SWIGLU else "linear"
+            return self._timed(f"gptq_lora_fwd<{kind}> K={K} N={'+'.join(map(str, Ns))}", flop, self._fwd, x2d, projs, mode)
+
+        def bwd(projs, M_, K, mode=mod.BWD_LINEAR, e=None, g=None):
+            Ns = [p["w"].N for p in projs]
+            flop = sum(2.0 * M * K * n + 2.0 * M * p["r"] * K for n, p in zip(Ns, projs))
+            kind = "swiglu" if mode == mod.BWD_SWIGLU else "linear"
+            return self._timed(f"gptq_lora_bwd_dx<{kind}> K={K} N={'+'.join(map(str, Ns))}", flop, self._bwd, projs, M_, K, mode, e=e, g=g)
+
+        mod.gptq_lora_fwd, mod.gptq_lora_bwd_dx = fwd, bwd
+        return self
+
+    def __exit__(self, *exc):
+        self.mod.gptq_lora_fwd, self.mod.gptq_lora_bwd_dx = self._fwd, self._bwd
+
+    def summary(self):
+        """label -> (average ms per launch, algorithmic FLOP per launch, launches)."""
+        acc = {}
+        for label, flop, s, e in self.records:
+            t = acc.setdefault(label, [0.0, flop, 0])
+            t[0] += s.elapsed_time(e)
+            t[2] += 1
+        return {k: (v[0] / v[2], v[1], v[2]) for k, v in acc.items()}
 
 
 def cpu_baseline(sample_tokens: int):
@@ -219,6 +232,9 @@ def main():
     ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one device copy of 1 GiB (a kernel of known traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the fused-LoRA path is data parallel over tokens and this build "
@@ -234,6 +250,12 @@ def main():
 
     attn, mlp = build_layer(device)
     step = make_step(attn, mlp, M, device, dtype)
+    if args.calibration_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -268,15 +290,24 @@ def main():
         "algorithmic_tflop_per_step": flops / 1e12,
     }
     if not args.no_kernel_timing:
-        kt = time_kernels(M, device, dtype)
-        dominant = max(kt, key=lambda k: kt[k][0])
-        ms, fl = kt[dominant]
+        # the same K steps once more, every fused-GEMM launch bracketed by events on its stream (kept
+        # out of the pass that produced `value`: the event packets serialise the queue a little)
+        with LaunchTimer(M) as timer:
+            for _ in range(args.steps):
+                step()
+            torch.cuda.synchronize()
+        kt = timer.summary()
+        per_step = {k: v[0] * v[2] / args.steps for k, v in kt.items()}
+        dominant = max(per_step, key=per_step.get)
+        ms, fl, _ = kt[dominant]
         result["roofline"] = {
             "kernel": dominant, "bound": "mfma", "achieved": fl / ms / 1e9, "peak": PEAK_BF16_TFLOPS,
-            "unit": "TFLOP/s", "frac": fl / ms / 1e9 / PEAK_BF16_TFLOPS, "traffic": None,
+            "unit": "TFLOP/s", "frac": fl / ms / 1e9 / PEAK_BF16_TFLOPS, "traffic": ROOFLINE_TRAFFIC_BYTES.get(dominant),
             "avg_launch_ms": ms, "algorithmic_flop_per_launch": fl,
+            "algorithmic_bytes_per_launch": ALGORITHMIC_BYTES.get(dominant),
         }
-        result["kernels"] = {k: {"ms": v[0], "tflops": v[1] / v[0] / 1e9} for k, v in kt.items()}
+        result["kernels"] = {k: {"ms": v[0], "tflops": v[1] / v[0] / 1e9, "launches_per_step": v[2] / args.steps}
+                             for k, v in kt.items()}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.cpu_sample_tokens)
     print(json.dumps(result))

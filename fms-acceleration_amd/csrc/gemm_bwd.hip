@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
   const int half = lane >> 5;
 
   int pid = xcd_remap(blockIdx.x, a.nbm * a.nbk);
-  constexpr int GROUP_M = 8;
+  constexpr int GROUP_M = 4;  // token blocks per group: 4 x 8 tiles in flight per XCD share X and W tiles in its L2
   const int width = GROUP_M * a.nbk;
   const int first_m = (pid / width) * GROUP_M;
   const int gsz = min(a.nbm - first_m, GROUP_M);

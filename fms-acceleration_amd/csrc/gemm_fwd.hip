@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 
   // ---- tile assignment: XCD-contiguous ranges, then grouped-M order inside the range --------
   int pid = xcd_remap(blockIdx.x, a.nbm * a.nbn);
-  constexpr int GROUP_M = 8;
+  constexpr int GROUP_M = 4;  // token blocks per group: 4 x 8 tiles in flight per XCD share X and W tiles in its L2
   const int width = GROUP_M * a.nbn;
   const int first_m = (pid / width) * GROUP_M;
   const int gsz = min(a.nbm - first_m, GROUP_M);
