@@ -355,6 +355,35 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
         pre_a[q & 1][it] = __builtin_amdgcn_raw_buffer_load_b128(mk_rsrc, mk_voff, (uint32_t)(EP_ROWS * q + 8 * it) * mk_row_bytes, 0);
     }
   };
+  // LoRA operands of the first 16 ranks of every projection: the A^T fragments of the lane's two
+  // columns are the same for all token tiles (loaded once), the T fragments of the two token tiles
+  // of a pass are fetched one pass ahead, so their latency hides behind the coalesced stores.
+  u32x4 af0[3][NT], tf0[3][2];
+  bool lora_live[3];
+  static_for<0, 3>([&](auto p_c) {
+    constexpr int p = decltype(p_c)::value;
+    const BwdProjDev& P = a.p[p];
+    lora_live[p] = p < a.n_proj && P.r > 0;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      af0[p][j] = u32x4{0u, 0u, 0u, 0u};
+      if (lora_live[p] && row_ok && 8 * half < P.r) af0[p][j] = *reinterpret_cast<const u32x4*>(P.At + (size_t)(kcol_lane + j) * P.r + 8 * half);
+    }
+  });
+  auto load_tf = [&](auto q_c) {
+    constexpr int q = decltype(q_c)::value;
+    static_for<0, 3>([&](auto p_c) {
+      constexpr int p = decltype(p_c)::value;
+      const BwdProjDev& P = a.p[p];
+#pragma unroll
+      for (int ml = 0; ml < 2; ++ml) {
+        const int m = m0 + 32 * (2 * q + ml) + l32;
+        tf0[p][ml] = u32x4{0u, 0u, 0u, 0u};
+        if (lora_live[p] && m < a.M && 8 * half < P.r) tf0[p][ml] = *reinterpret_cast<const u32x4*>(P.T + (size_t)m * P.ldt + 8 * half);
+      }
+    });
+  };
+  load_tf(std::integral_constant<int, 0>{});
   issue_loads(std::integral_constant<int, 0>{});
 
   static_for<0, MT / 2>([&](auto q_c) {
@@ -370,33 +399,37 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
 #pragma unroll
         for (int i = 0; i < 16; ++i) lora[j][i] = 0.f;
       if (any_lora) {
-        for (int p = 0; p < a.n_proj; ++p) {
-          const BwdProjDev P = select_proj(a, p);
-          if (P.r <= 0) continue;
-          f32x16 tmp[NT];
+        static_for<0, 3>([&](auto p_c) {
+          constexpr int p = decltype(p_c)::value;
+          if (lora_live[p]) {
+            const BwdProjDev& P = a.p[p];
+            f32x16 tmp[NT];
 #pragma unroll
-          for (int j = 0; j < NT; ++j)
+            for (int j = 0; j < NT; ++j) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) tmp[j][i] = 0.f;
-          for (int j0 = 0; j0 < P.r; j0 += 16) {
-            const int ko = j0 + 8 * half;
-            u32x4 tf = {0u, 0u, 0u, 0u}, af[NT] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-            if (ko < P.r) {
-              if (m_ok) tf = *reinterpret_cast<const u32x4*>(P.T + (size_t)m * P.ldt + ko);
-              if (row_ok) {
+              for (int i = 0; i < 16; ++i) tmp[j][i] = 0.f;
+              tmp[j] = mfma32<T>(af0[p][j], tf0[p][ml], tmp[j]);
+            }
+            for (int j0 = 16; j0 < P.r; j0 += 16) {  // ranks beyond the prefetched 16
+              const int ko = j0 + 8 * half;
+              u32x4 tf = {0u, 0u, 0u, 0u}, af[NT] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+              if (ko < P.r) {
+                if (m_ok) tf = *reinterpret_cast<const u32x4*>(P.T + (size_t)m * P.ldt + ko);
+                if (row_ok) {
 #pragma unroll
-                for (int j = 0; j < NT; ++j)
-                  af[j] = *reinterpret_cast<const u32x4*>(P.At + (size_t)(kcol_lane + j) * P.r + ko);
+                  for (int j = 0; j < NT; ++j)
+                    af[j] = *reinterpret_cast<const u32x4*>(P.At + (size_t)(kcol_lane + j) * P.r + ko);
+                }
               }
+#pragma unroll
+              for (int j = 0; j < NT; ++j) tmp[j] = mfma32<T>(af[j], tf, tmp[j]);
             }
 #pragma unroll
-            for (int j = 0; j < NT; ++j) tmp[j] = mfma32<T>(af[j], tf, tmp[j]);
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+              for (int i = 0; i < 16; ++i) lora[j][i] += P.s * tmp[j][i];
           }
-#pragma unroll
-          for (int j = 0; j < NT; ++j)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) lora[j][i] += P.s * tmp[j][i];
-        }
+        });
       }
       // rounded pairs (tile 0, tile 1) = adjacent output columns -> one 4-byte LDS write
 #pragma unroll
@@ -409,7 +442,10 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     });
     __syncthreads();
       // coalesced pass: 64 rows x 32 chunks of 8 columns; iteration `it` handles row 8*it + tid/32
-    if (q + 1 < MT / 2) issue_loads(std::integral_constant<int, (q + 1 < MT / 2) ? q + 1 : q>{});
+    if (q + 1 < MT / 2) {
+      load_tf(std::integral_constant<int, (q + 1 < MT / 2) ? q + 1 : q>{});
+      issue_loads(std::integral_constant<int, (q + 1 < MT / 2) ? q + 1 : q>{});
+    }
 #pragma unroll
     for (int it = 0; it < EP_ROWS * 32 / 256; ++it) {
       const int row = (tid >> 5) + 8 * it;
