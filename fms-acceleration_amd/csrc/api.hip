@@ -19,6 +19,12 @@ int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int m
 int launch_gptq_nsz(const fmsa_gptq_weight* w, float* out, hipStream_t st);
 int launch_lora_pack(const void* A, const void* B, int r, int K, int N, int param_dtype, int act_dtype, void* A16, void* At16,
                      void* B16, void* Bt16, hipStream_t st);
+int launch_rms_fwd(const void* X, int64_t ldx, const void* W, int M, int C, float eps, int gemma, int x_dtype, int w_dtype, void* Y,
+                   int64_t ldy, float* r, hipStream_t st);
+int launch_rms_bwd(void* dY, int64_t lddy, const void* X, int64_t ldx, const void* W, const float* r, int M, int C, int gemma,
+                   int x_dtype, int w_dtype, hipStream_t st);
+int launch_rope(void* Q, int64_t ldq, const void* cosp, const void* sinp, int64_t ldcs, int M, int n_heads, int head_dim, int cs_rows,
+                int backward, int q_dtype, int cs_dtype, hipStream_t st);
 int launch_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, hipStream_t st);
 int launch_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype, hipStream_t st);
 int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, int M, int I, int64_t ld, int act_dtype,
@@ -247,6 +253,43 @@ int fmsa_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, void* s
   if (out_dtype != FMSA_F16 && out_dtype != FMSA_BF16 && out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
   if (!aligned16(out) || (reinterpret_cast<uintptr_t>(w->packed) & 7u)) return FMSA_ERR_ALIGN;
   return launch_nf4_dequant(w, out_dtype, out, (hipStream_t)stream);
+}
+
+namespace {
+inline bool is_float_dtype(int d) { return d == FMSA_F16 || d == FMSA_BF16 || d == FMSA_F32; }
+inline bool aligned_rows(const void* p, int64_t ld, int d) {
+  const int esz = d == FMSA_F32 ? 4 : 2;
+  return aligned16(p) && (ld * esz) % 16 == 0;
+}
+}  // namespace
+
+int fmsa_rms_layernorm_fwd(const void* X, int64_t ldx, const void* W, int M, int C, float eps, int gemma, int x_dtype,
+                           int w_dtype, void* Y, int64_t ldy, float* r, void* stream) {
+  if (!X || !W || !Y || !r) return FMSA_ERR_NULL;
+  if (M <= 0 || C <= 0 || C % 8 != 0 || ldx < C || ldy < C) return FMSA_ERR_SHAPE;
+  if (!is_float_dtype(x_dtype) || !is_float_dtype(w_dtype)) return FMSA_ERR_DTYPE;
+  if (!aligned_rows(X, ldx, x_dtype) || !aligned_rows(Y, ldy, x_dtype) || !aligned16(W)) return FMSA_ERR_ALIGN;
+  return launch_rms_fwd(X, ldx, W, M, C, eps, gemma, x_dtype, w_dtype, Y, ldy, r, (hipStream_t)stream);
+}
+
+int fmsa_rms_layernorm_bwd(void* dY, int64_t lddy, const void* X, int64_t ldx, const void* W, const float* r, int M, int C,
+                           int gemma, int x_dtype, int w_dtype, void* stream) {
+  if (!dY || !X || !W || !r) return FMSA_ERR_NULL;
+  if (M <= 0 || C <= 0 || C % 8 != 0 || ldx < C || lddy < C) return FMSA_ERR_SHAPE;
+  if (!is_float_dtype(x_dtype) || !is_float_dtype(w_dtype)) return FMSA_ERR_DTYPE;
+  if (!aligned_rows(X, ldx, x_dtype) || !aligned_rows(dY, lddy, x_dtype) || !aligned16(W)) return FMSA_ERR_ALIGN;
+  return launch_rms_bwd(dY, lddy, X, ldx, W, r, M, C, gemma, x_dtype, w_dtype, (hipStream_t)stream);
+}
+
+int fmsa_rope_embedding(void* Q, int64_t ldq, const void* cos, const void* sin, int64_t ldcs, int M, int n_heads,
+                        int head_dim, int cs_rows, int backward, int q_dtype, int cs_dtype, void* stream) {
+  if (!Q || !cos || !sin) return FMSA_ERR_NULL;
+  if (M <= 0 || n_heads <= 0 || head_dim <= 0 || head_dim % 16 != 0 || cs_rows <= 0) return FMSA_ERR_SHAPE;
+  if (ldq < (int64_t)n_heads * head_dim || ldcs < head_dim / 2) return FMSA_ERR_SHAPE;
+  if (!is_float_dtype(q_dtype) || !is_float_dtype(cs_dtype)) return FMSA_ERR_DTYPE;
+  if (!aligned_rows(Q, ldq, q_dtype) || !aligned_rows(cos, ldcs, cs_dtype) || !aligned_rows(sin, ldcs, cs_dtype))
+    return FMSA_ERR_ALIGN;
+  return launch_rope(Q, ldq, cos, sin, ldcs, M, n_heads, head_dim, cs_rows, backward, q_dtype, cs_dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

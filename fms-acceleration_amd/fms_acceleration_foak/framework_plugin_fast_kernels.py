@@ -1,9 +1,9 @@
 """FastKernelsAccelerationPlugin: turns the `fused_ops_and_kernels` configuration into registered
 ModelPatcher rules (reference: fms_acceleration_foak/framework_plugin_fast_kernels.py:31-222).
 
-Only the `fused_lora` switch has kernels behind it in this build (rule suffixes "qkvo" and "mlp").
-The other switches of the reference (`fast_loss`, `fast_rms_layernorm`, `fast_rope_embeddings`) are
-accepted and validated so that existing YAML files load unchanged, but they select no rule here.
+Switches with kernels behind them in this build: `fused_lora` (rule suffixes "qkvo", "mlp"),
+`fast_rms_layernorm` ("rms") and `fast_rope_embeddings` ("rope").  `fast_loss` is accepted and
+validated so that existing YAML files load unchanged, but it selects no rule here.
 """
 from __future__ import annotations
 

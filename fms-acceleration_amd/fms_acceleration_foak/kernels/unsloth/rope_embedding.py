@@ -1,0 +1,48 @@
+"""Rotary position embedding on the gfx950 kernel of libfmsa_hip (drop-in for
+kernels/unsloth/rope_embedding.py of the reference: `Fast_RoPE_Embedding` :68-128 and
+`fast_rope_embedding(Q, K, cos, sin, position_ids=None)` :132-135).
+
+Like the reference the rotation is applied in place on the [batch, seq, heads, head_dim] view of the
+projection output and ignores `position_ids` (:131): row m of the flattened tokens takes position
+m % seq_len of a 2-D cos / sin; a 3-D cos / sin [batch, seq, head_dim] (what recent transformers
+pass) is used row by row, which is the same thing for the default positions."""
+import torch
+
+import fmsa_hip
+
+
+def _rows(t):
+    """cos / sin as [rows, head_dim]: [seq, d], [1, seq, d] -> [seq, d]; [batch, seq, d] -> [batch*seq, d]."""
+    t = t.squeeze()
+    if t.dim() == 3:
+        t = t.reshape(-1, t.shape[-1])
+    if t.dim() != 2:
+        raise ValueError(f"cos / sin must be [seq, head_dim] or [batch, seq, head_dim], got {tuple(t.shape)}")
+    return t if t.stride(1) == 1 else t.contiguous()
+
+
+class Fast_RoPE_Embedding(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, Q, cos, sin):
+        cos, sin = _rows(cos), _rows(sin)
+        batch, seq_len, n_heads, head_dim = Q.shape
+        if seq_len > cos.shape[0]:
+            raise ValueError("cos / sin cover fewer positions than the sequence")
+        Q2 = Q.view(batch * seq_len, n_heads * head_dim)
+        fmsa_hip.rope_embedding_(Q2, cos, sin, n_heads, head_dim, backward=False)
+        ctx.cos, ctx.sin = cos, sin
+        return Q2.view(batch, seq_len, n_heads, head_dim)
+
+    @staticmethod
+    def backward(ctx, dY):
+        batch, seq_len, n_heads, head_dim = dY.shape
+        dY2 = dY.reshape(batch * seq_len, n_heads * head_dim)  # reshape: dY may be non-contiguous (:111-112)
+        dY2 = dY2 if dY2.stride(1) == 1 else dY2.contiguous()
+        fmsa_hip.rope_embedding_(dY2, ctx.cos, ctx.sin, n_heads, head_dim, backward=True)
+        return dY2.view(batch, seq_len, n_heads, head_dim), None, None
+
+
+def fast_rope_embedding(Q, K, cos, sin, position_ids=None, unsqueeze_dim=1):
+    Q = Fast_RoPE_Embedding.apply(Q.transpose(1, 2), cos, sin).transpose(1, 2)
+    K = Fast_RoPE_Embedding.apply(K.transpose(1, 2), cos, sin).transpose(1, 2)
+    return Q, K

@@ -1,6 +1,7 @@
-"""Shared construction of the `<arch>-qkvo` / `<arch>-mlp` rules: the three dense architectures
-differ only in their attention / MLP classes (reference: models/llama.py:73-123, mistral.py:70-119,
-granite.py:78-128)."""
+"""Shared construction of the patch rules: `<arch>-qkvo` / `<arch>-mlp` (fused LoRA; the
+architectures differ only in their attention / MLP classes, reference models/llama.py:73-123,
+mistral.py:70-119, granite.py:78-128), `<arch>-rms` (RMS layer norm forward replaced, llama.py:65-69)
+and `<arch>-rope` (the modelling module's apply_rotary_pos_emb replaced, llama.py:154-161)."""
 from __future__ import annotations
 
 import warnings
@@ -55,3 +56,16 @@ def fused_lora_rules(arch: str, attn_cls, mlp_cls, base_type: str, config=None, 
             )
             rules = filter_mp_rules(rules, {"mlp"}, drop=True)
     return rules
+
+
+def norm_rope_rules(arch: str, rms_cls, modeling_module: str):
+    """`<arch>-rms` and `<arch>-rope` on the libfmsa_hip kernels."""
+    from ..kernels.unsloth import fast_rms_layernorm, fast_rope_embedding  # pylint: disable=import-outside-toplevel
+
+    return [
+        ModelPatcherRule(rule_id=f"{arch}-rms", trigger=ModelPatcherTrigger(check=rms_cls), forward=fast_rms_layernorm),
+        ModelPatcherRule(
+            rule_id=f"{arch}-rope",
+            import_and_maybe_reload=(f"{modeling_module}.apply_rotary_pos_emb", fast_rope_embedding, None),
+        ),
+    ]

@@ -1,11 +1,14 @@
-"""Patch rule `granitemoe-qkvo` (reference: fms_acceleration_foak/models/granitemoe.py): the attention
-projections of this mixture-of-experts architecture take the fused LoRA operators; its expert MLPs
-have no fused-LoRA rule in the reference either, and its RMSNorm / RoPE / loss rules belong to
-other kernels and are not built."""
-from transformers.models.granitemoe.modeling_granitemoe import GraniteMoeAttention
+"""Patch rules `granitemoe-rms`, `granitemoe-qkvo`, `granitemoe-rope` (reference: fms_acceleration_foak/models/granitemoe.py):
+the attention projections of this mixture-of-experts architecture take the fused LoRA operators; its
+expert MLPs have no fused-LoRA rule in the reference either, and its loss rules belong to other
+kernels and are not built."""
+from transformers.models.granitemoe.modeling_granitemoe import GraniteMoeAttention, GraniteMoeRMSNorm
 
-from ._rules import fused_lora_rules
+from ._rules import fused_lora_rules, norm_rope_rules
 
 
 def get_mp_rules(base_type: str, config=None):
-    return fused_lora_rules("granitemoe", GraniteMoeAttention, None, base_type, config, label="GraniteMoe")
+    return [
+        *fused_lora_rules("granitemoe", GraniteMoeAttention, None, base_type, config, label="GraniteMoe"),
+        *norm_rope_rules("granitemoe", GraniteMoeRMSNorm, "transformers.models.granitemoe.modeling_granitemoe"),
+    ]

@@ -38,6 +38,9 @@ EXPORTED_SYMBOLS = (
     "fmsa_gptq_make_nsz",
     "fmsa_nf4_dequant",
     "fmsa_lora_pack",
+    "fmsa_rms_layernorm_fwd",
+    "fmsa_rms_layernorm_bwd",
+    "fmsa_rope_embedding",
 )
 
 
@@ -134,6 +137,12 @@ def lib() -> ctypes.CDLL:
     L.fmsa_nf4_dequant.argtypes = [POINTER(Nf4Weight), c_int, c_void_p, c_void_p]
     L.fmsa_lora_pack.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p]
+    L.fmsa_rms_layernorm_fwd.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p,
+                                         c_int64, c_void_p, c_void_p]
+    L.fmsa_rms_layernorm_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                         c_int, c_void_p]
+    L.fmsa_rope_embedding.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int,
+                                      c_int, c_void_p]
     for name in EXPORTED_SYMBOLS:
         getattr(L, name)  # AttributeError here means the library is stale: rebuild it
     _lib = L
@@ -360,3 +369,39 @@ def lora_pack(A, B, act_dtype, A16_out=None):
     _check("fmsa_lora_pack", lib().fmsa_lora_pack(_ptr(A), _ptr(B), r, K, N, _DTYPE_ENUM[A.dtype], act_enum(act_dtype),
                                                   _ptr(A16_out), _ptr(At16), _ptr(B16), _ptr(Bt16), _stream(A)))
     return A16_out, At16, B16, Bt16
+
+
+def rms_layernorm_fwd(x2d, weight, eps: float, gemma: bool = False):
+    """(Y [M, C] in x2d's dtype, r [M] fp32 = 1 / rms) of an RMS layer norm over the rows of x2d."""
+    if not (x2d.is_cuda and weight.is_cuda):
+        raise RuntimeError("fmsa_hip needs GPU tensors")
+    M, C = x2d.shape
+    assert x2d.stride(1) == 1 and weight.is_contiguous() and weight.numel() == C
+    y = torch.empty((M, C), dtype=x2d.dtype, device=x2d.device)
+    r = torch.empty(M, dtype=torch.float32, device=x2d.device)
+    _check("fmsa_rms_layernorm_fwd",
+           lib().fmsa_rms_layernorm_fwd(_ptr(x2d), x2d.stride(0), _ptr(weight), M, C, float(eps), int(gemma), _DTYPE_ENUM[x2d.dtype],
+                                        _DTYPE_ENUM[weight.dtype], _ptr(y), y.stride(0), _ptr(r), _stream(x2d)))
+    return y, r
+
+
+def rms_layernorm_bwd(dy2d, x2d, weight, r, gemma: bool = False):
+    """Overwrites dy2d with dX and returns it."""
+    M, C = x2d.shape
+    assert dy2d.shape == (M, C) and dy2d.stride(1) == 1 and x2d.stride(1) == 1 and dy2d.dtype == x2d.dtype
+    _check("fmsa_rms_layernorm_bwd",
+           lib().fmsa_rms_layernorm_bwd(_ptr(dy2d), dy2d.stride(0), _ptr(x2d), x2d.stride(0), _ptr(weight), _ptr(r), M, C, int(gemma),
+                                        _DTYPE_ENUM[x2d.dtype], _DTYPE_ENUM[weight.dtype], _stream(x2d)))
+    return dy2d
+
+
+def rope_embedding_(q2d, cos2d, sin2d, n_heads: int, head_dim: int, backward: bool = False):
+    """In place on q2d [M, n_heads * head_dim]; row m uses row m % cos2d.shape[0] of cos / sin."""
+    if not (q2d.is_cuda and cos2d.is_cuda and sin2d.is_cuda):
+        raise RuntimeError("fmsa_hip needs GPU tensors")
+    assert q2d.stride(1) == 1 and cos2d.stride(1) == 1 and cos2d.stride() == sin2d.stride() and cos2d.dtype == sin2d.dtype
+    _check("fmsa_rope_embedding",
+           lib().fmsa_rope_embedding(_ptr(q2d), q2d.stride(0), _ptr(cos2d), _ptr(sin2d), cos2d.stride(0), q2d.shape[0], n_heads,
+                                     head_dim, cos2d.shape[0], int(backward), _DTYPE_ENUM[q2d.dtype], _DTYPE_ENUM[cos2d.dtype],
+                                     _stream(q2d)))
+    return q2d

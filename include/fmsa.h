@@ -207,6 +207,27 @@ typedef struct fmsa_nf4_weight {
 
 int fmsa_nf4_dequant(const fmsa_nf4_weight* w /*host*/, int out_dtype, void* out, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * The two bandwidth-bound operators next to the q/k/v projections.  x_dtype / w_dtype / q_dtype /
+ * cs_dtype: FMSA_F16, FMSA_BF16 or FMSA_F32; rows 16-byte aligned, C % 8 == 0, head_dim % 16 == 0.
+ *
+ * RMS layer norm (kernels/unsloth/rms_layernorm.py:21-47, 99-109 forward; :50-86 backward):
+ *   fwd: r[m] = rsqrt(mean(x^2) + eps); Y = round_w(x * r) * W, in w_dtype arithmetic, stored in
+ *        x_dtype.  gemma != 0: fp32 throughout, r = 1 / sqrt(.), weight W + 1.
+ *   bwd: dX = r/C * (C * dY_W - (x r) * sum(dY_W * x r)), dY_W = dY * W (gemma: W + 1), fp32,
+ *        written over dY (the weight is frozen: no dW, as in the reference).
+ * Rotary embedding (kernels/unsloth/rope_embedding.py:22-65), in place on Q [M, n_heads*head_dim]:
+ *   (q1, q2) <- (q1 cos - q2 sin, q2 cos + q1 sin) on the halves of every head; row m uses row
+ *   m % cs_rows of cos / sin [cs_rows, >= head_dim/2]; backward != 0 negates sin.
+ * ------------------------------------------------------------------------------------------ */
+int fmsa_rms_layernorm_fwd(const void* X, int64_t ldx, const void* W, int M, int C, float eps, int gemma,
+                           int x_dtype, int w_dtype, void* Y, int64_t ldy, float* r, void* stream);
+int fmsa_rms_layernorm_bwd(void* dY, int64_t lddy, const void* X, int64_t ldx, const void* W, const float* r,
+                           int M, int C, int gemma, int x_dtype, int w_dtype, void* stream);
+int fmsa_rope_embedding(void* Q, int64_t ldq, const void* cos, const void* sin, int64_t ldcs, int M,
+                        int n_heads, int head_dim, int cs_rows, int backward, int q_dtype, int cs_dtype,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -115,3 +115,21 @@ def test_product_path_refuses_cpu_tensors():
     ql = QuantLinear(4, 64, 64, 64, False)
     with pytest.raises(RuntimeError):
         ql(torch.zeros(2, 64, dtype=torch.float16))
+
+
+def test_norm_rope_validation():
+    lib = fmsa_hip.lib()
+    f = lib.fmsa_rms_layernorm_fwd
+    assert f(None, 64, 0x2000, 8, 64, 1e-5, 0, 1, 1, 0x3000, 64, 0x4000, None) == -1
+    assert f(0x1000, 64, 0x2000, 8, 60, 1e-5, 0, 1, 1, 0x3000, 64, 0x4000, None) == -2   # C % 8
+    assert f(0x1000, 32, 0x2000, 8, 64, 1e-5, 0, 1, 1, 0x3000, 64, 0x4000, None) == -2   # ldx < C
+    assert f(0x1000, 64, 0x2000, 8, 64, 1e-5, 0, 5, 1, 0x3000, 64, 0x4000, None) == -4   # dtype
+    assert f(0x1004, 64, 0x2000, 8, 64, 1e-5, 0, 1, 1, 0x3000, 64, 0x4000, None) == -3   # alignment
+    b = lib.fmsa_rms_layernorm_bwd
+    assert b(0x1000, 64, 0x2000, 64, 0x3000, None, 8, 64, 0, 1, 1, None) == -1           # r missing
+    assert b(0x1000, 64, 0x2000, 64, 0x3000, 0x4000, 0, 64, 0, 1, 1, None) == -2
+    rp = lib.fmsa_rope_embedding
+    assert rp(0x1000, 256, 0x2000, None, 64, 8, 4, 64, 8, 0, 1, 1, None) == -1
+    assert rp(0x1000, 256, 0x2000, 0x3000, 64, 8, 4, 24, 8, 0, 1, 1, None) == -2          # head_dim % 16
+    assert rp(0x1000, 128, 0x2000, 0x3000, 64, 8, 4, 64, 8, 0, 1, 1, None) == -2          # ldq < heads * head_dim
+    assert rp(0x1000, 256, 0x2000, 0x3000, 64, 8, 4, 64, 0, 0, 1, 1, None) == -2          # no cos rows

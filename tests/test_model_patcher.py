@@ -178,7 +178,7 @@ def test_mlp_rule_dropped_for_non_silu_activation():
     with warnings.catch_warnings(record=True):
         warnings.simplefilter("always")
         ids = [r.rule_id for r in llama.get_mp_rules("auto_gptq", cfg)]
-    assert ids == ["llama-qkvo"]
+    assert ids == ["llama-qkvo", "llama-rms", "llama-rope"]
 
 
 def test_partial_lora_follows_the_reference_rule_logic():
@@ -223,3 +223,35 @@ def test_filter_mp_rules():
     rules = [ModelPatcherRule(rule_id=i) for i in ("a-qkvo", "a-mlp", "a-rms")]
     assert [r.rule_id for r in filter_mp_rules(rules, {"qkvo", "mlp"})] == ["a-qkvo", "a-mlp"]
     assert [r.rule_id for r in filter_mp_rules(rules, {"mlp"}, drop=True)] == ["a-qkvo", "a-rms"]
+
+
+def test_rms_and_rope_rules_registered_and_applied():
+    """fast_rms_layernorm / fast_rope_embeddings select the `<arch>-rms` / `<arch>-rope` rules: the
+    norm modules get the new forward, the modelling module's apply_rotary_pos_emb is replaced."""
+    import transformers.models.llama.modeling_llama as ml
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaRMSNorm
+
+    from fms_acceleration_foak import FastKernelsAccelerationPlugin
+    from fms_acceleration_foak.kernels.unsloth import fast_rms_layernorm, fast_rope_embedding
+
+    cfg = LlamaConfig(hidden_size=64, intermediate_size=128, num_attention_heads=4, num_hidden_layers=1, vocab_size=32)
+    cfg.architectures = ["LlamaForCausalLM"]
+    from transformers import LlamaForCausalLM
+
+    model = LlamaForCausalLM(cfg)  # the import rule only applies to models defined under the patched module path
+    plugin = FastKernelsAccelerationPlugin(
+        {"training": {"fused_ops_and_kernels": {"fast_rms_layernorm": True, "fast_rope_embeddings": True}}})
+    original = ml.apply_rotary_pos_emb
+    try:
+        with instantiate_model_patcher():
+            plugin.augmentation(model, type("T", (), {"bf16": True, "fp16": False})(), ())
+            ids = set(ModelPatcher.rules)
+            assert {"llama-rms", "llama-rope", "mistral-rms", "granite-rope", "mixtral-rms", "granitemoe-rope"} <= ids
+            assert not any(i.endswith(("qkvo", "mlp")) for i in ids)
+            patch_model(model)
+            norms = [m for m in model.modules() if isinstance(m, LlamaRMSNorm)]
+            assert len(norms) == 3 and all(m.forward.__func__ is fast_rms_layernorm for m in norms)
+            assert ml.apply_rotary_pos_emb is fast_rope_embedding
+    finally:
+        ml.apply_rotary_pos_emb = original
