@@ -107,54 +107,7 @@ def get_lora_parameters(proj):
     return qstate, bias, A, B, s, dropout
 
 
-# ----------------------------------------------------------------------------------------------
-# per-weight preparation, cached on the qweight tensor
-# ----------------------------------------------------------------------------------------------
-class _PreparedWeight:
-    """The C-ABI view of one QuantLinear.  For an act-order g_idx the packed rows are re-ordered
-    once (fmsa_gptq_permute_rows) so that the group of row k' is k' // group_size; `perm` then
-    maps the kernels' row order back to the model's: row k' of the repacked weight is row
-    perm[k'] of the original."""
-
-    __slots__ = ("struct", "K", "N", "group_size", "perm", "nsz", "_keep")
-
-    def __init__(self, qweight, scales, qzeros, g_idx, bits):
-        if bits != 4:
-            raise NotImplementedError(f"the gfx950 fused kernels cover 4-bit GPTQ only (got bits={bits})")
-        if not qweight.is_cuda:
-            raise RuntimeError("fused GPTQ-LoRA ops need the quantised weight on the GPU")
-        K, N, G = qweight.shape[0] * 8, qweight.shape[1], scales.shape[0]
-        if K % G != 0:
-            raise NotImplementedError(f"in_features {K} is not a multiple of the number of groups {G}")
-        gs = K // G
-        zero_offset = int(getattr(qzeros, "offset", 0) or 0)
-        qweight, scales, qzeros = qweight.contiguous(), scales.contiguous(), qzeros.contiguous()
-        ident = torch.arange(K, device=g_idx.device, dtype=torch.int64) // gs
-        g64 = g_idx.to(torch.int64)
-        g64 = torch.where(g64 < 0, g64 + G, g64)
-        perm = None
-        if not torch.equal(g64, ident):
-            perm64 = torch.argsort(g64, stable=True)
-            if not torch.equal(g64[perm64], ident):
-                raise NotImplementedError("act-order g_idx with groups of unequal size is not supported")
-            perm = perm64.to(torch.int32).contiguous()
-            qweight = fmsa_hip.gptq_permute_rows(qweight, perm)
-        self.K, self.N, self.group_size, self.perm = K, N, gs, perm
-        self._keep = (qweight, scales, qzeros)
-        self.struct = fmsa_hip.make_weight(qweight, scales, qzeros, None, gs, zero_offset)
-        # -scale * zero per (group, column), fp32: read by the input-gradient kernel (frozen weight,
-        # so it is built once)
-        self.nsz = fmsa_hip.gptq_make_nsz(self.struct, qweight.device)
-
-
-def _prepare(qweight, scales, qzeros, g_idx, bits) -> _PreparedWeight:
-    key = (qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(), g_idx.data_ptr(), g_idx._version,
-           qweight._version, int(getattr(qzeros, "offset", 0) or 0))
-    cached = getattr(qweight, "_fmsa_prepared", None)
-    if cached is None or cached[0] != key:
-        cached = (key, _PreparedWeight(qweight, scales, qzeros, g_idx, bits))
-        qweight._fmsa_prepared = cached
-    return cached[1]
+from fmsa_hip.gptq_prepared import prepare as _prepare  # per-weight C-ABI view, cached on the qweight tensor
 
 
 # ----------------------------------------------------------------------------------------------

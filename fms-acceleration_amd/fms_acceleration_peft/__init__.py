@@ -5,3 +5,4 @@ from .framework_plugin_bnb import BNBAccelerationPlugin
 from .lora import LoraLinear
 from .qlinear import QuantLinear, QuantLinearFunction
 from .nf4 import Linear4bit, Params4bit, QuantState, quantize_nf4
+from .gptq_checkpoint import QuantizeConfig, convert_gptq_v1_to_v2_format, convert_gptq_v2_to_v1_format, load_quantized, save_quantized

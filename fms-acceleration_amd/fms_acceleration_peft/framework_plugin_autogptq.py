@@ -1,10 +1,10 @@
 """Configuration shell of the GPTQ-LoRA plugin (reference:
 accelerated-peft/src/fms_acceleration_peft/framework_plugin_autogptq.py:44-395).
 
-Only the boundary is built: registration under `peft.quantization.auto_gptq`, validation of the
-configuration keys, and the `quantization_method` marker that the fast-kernels plugin keys on.
-Loading a quantised checkpoint and installing PEFT adapters need the gptqmodel loader, peft and
-hub checkpoints; callers of this build construct `QuantLinear` + `LoraLinear` modules directly.
+Built: registration under `peft.quantization.auto_gptq`, validation of the configuration keys, a
+loader for LOCAL GPTQ checkpoint directories (gptq_checkpoint.py) and the `quantization_method`
+marker that the fast-kernels plugin keys on.  Installing PEFT adapters needs peft, which is not
+available here: callers wrap the QuantLinear modules in `LoraLinear` themselves.
 """
 from fms_acceleration import AccelerationPlugin
 
@@ -29,11 +29,33 @@ class AutoGPTQAccelerationPlugin(AccelerationPlugin):
         return True
 
     def model_loader(self, model_name: str, **kwargs):
-        raise NotImplementedError(
-            "GPTQ checkpoint loading is outside the fused-LoRA hot path of this build: wrap the "
-            "model's linears in fms_acceleration_peft.QuantLinear / LoraLinear and set "
-            "model.quantization_method = 'gptq'"
-        )
+        """Load a GPTQ checkpoint from a LOCAL directory (config.json + quantize_config.json +
+        safetensors): the architecture is built from its config with empty weights, the packed
+        linears become QuantLinear modules and the tensors are read from the file (reference:
+        :108-222, which goes through the hub and accelerate; there is no network here)."""
+        import os  # pylint: disable=import-outside-toplevel
+
+        import torch  # pylint: disable=import-outside-toplevel
+        from transformers import AutoConfig, AutoModelForCausalLM  # pylint: disable=import-outside-toplevel
+
+        from .gptq_checkpoint import load_quantized  # pylint: disable=import-outside-toplevel
+
+        if not os.path.isdir(model_name):
+            raise NotImplementedError(
+                f"'{model_name}' is not a local directory: this build loads GPTQ checkpoints from disk only "
+                "(no hub access)"
+            )
+        torch_dtype = kwargs.get("torch_dtype", torch.float16)
+        config = AutoConfig.from_pretrained(model_name)
+        prev = torch.get_default_dtype()
+        torch.set_default_dtype(torch_dtype)
+        try:
+            model = AutoModelForCausalLM.from_config(config)
+        finally:
+            torch.set_default_dtype(prev)
+        device = kwargs.get("device", "cuda" if torch.cuda.is_available() else "cpu")
+        model, _ = load_quantized(model, model_name, device=device)
+        return model
 
     def augmentation(self, model, train_args, modifiable_args):
         # the marker FastKernelsAccelerationPlugin.augmentation looks for (:235-236 of the reference)

@@ -2,10 +2,9 @@
 
 Buffer names, shapes and dtypes are those of the reference's tritonv2 QuantLinear
 (gptqmodel/nn_modules/qlinear/qlinear_tritonv2.py:67-99), so a state_dict of one loads into the
-other.  `forward` is the reference's unfused path (`QuantLinearFunction`,
-gptqmodel/nn_modules/triton_utils/dequant.py:132-161): materialise the dense weight with the
-dequant kernel, matmul, no gradient for the frozen base.  It exists as the baseline the fused
-operators are compared with; the fused path never calls it.
+other.  `forward` is the module-level path without LoRA fusion (`QuantLinearFunction`,
+gptqmodel/nn_modules/triton_utils/dequant.py:132-161: base projection only, no gradient for the
+frozen weight): what a PEFT LoRA layer calls when the fused-LoRA rules are not installed.
 """
 from __future__ import annotations
 
@@ -17,8 +16,12 @@ from torch import nn
 
 
 class QuantLinearFunction(torch.autograd.Function):
-    """y = x @ deq(W); dx = dy @ deq(W)^T (dequant.py:141-161).  The dense weight is produced in the
-    activation dtype by libfmsa_hip (one rounding) instead of fp16 followed by an autocast re-cast."""
+    """y = x @ deq(W); dx = dy @ deq(W)^T (dequant.py:141-161).
+
+    bf16 / fp16 activations go through the fused dequant-GEMM kernels with the adapter disabled
+    (r = 0): the 4-bit weight is unpacked in registers on its way into the MFMA and no dense matrix
+    is ever written.  Other activation types (fp32) take the dequantise-then-matmul route, with the
+    dense weight produced in the activation dtype by one rounding."""
 
     @staticmethod
     def forward(ctx, x, qweight, scales, qzeros, g_idx, bits, group_size, zero_offset):
@@ -26,19 +29,39 @@ class QuantLinearFunction(torch.autograd.Function):
 
         if bits != 4:
             raise NotImplementedError("the gfx950 kernels cover 4-bit GPTQ only")
-        W = fmsa_hip.gptq_dequant(qweight, scales, qzeros, g_idx, group_size, zero_offset, x.dtype)
         ctx.save_for_backward(qweight, scales, qzeros, g_idx)
-        ctx.meta = (group_size, zero_offset)
-        return x @ W
+        ctx.meta = (bits, group_size, zero_offset)
+        ctx.fused = x.dtype in (torch.float16, torch.bfloat16) and group_size % 16 == 0
+        if not ctx.fused:
+            W = fmsa_hip.gptq_dequant(qweight, scales, qzeros, g_idx, group_size, zero_offset, x.dtype)
+            return x @ W
+        from fmsa_hip.gptq_prepared import prepare
+
+        w = prepare(qweight, scales, qzeros, g_idx, bits)
+        x2 = x if x.is_contiguous() else x.contiguous()
+        if w.perm is not None:  # act-order: the repacked weight walks K in sorted-group order
+            x2 = fmsa_hip.permute_cols(x2, w.perm, gather=True)
+        (y,) = fmsa_hip.gptq_lora_fwd(x2, [{"w": w.struct, "U": None, "B": None, "bias": None, "r": 0, "s": 0.0}])
+        return y
 
     @staticmethod
     def backward(ctx, dy):
         import fmsa_hip
 
         qweight, scales, qzeros, g_idx = ctx.saved_tensors
-        group_size, zero_offset = ctx.meta
-        W = fmsa_hip.gptq_dequant(qweight, scales, qzeros, g_idx, group_size, zero_offset, dy.dtype)
-        return dy @ W.t(), None, None, None, None, None, None, None
+        bits, group_size, zero_offset = ctx.meta
+        if not ctx.fused or group_size < 32:
+            W = fmsa_hip.gptq_dequant(qweight, scales, qzeros, g_idx, group_size, zero_offset, dy.dtype)
+            return dy @ W.t(), None, None, None, None, None, None, None
+        from fmsa_hip.gptq_prepared import prepare
+
+        w = prepare(qweight, scales, qzeros, g_idx, bits)
+        dy2 = dy if dy.is_contiguous() else dy.contiguous()
+        dx = fmsa_hip.gptq_lora_bwd_dx(
+            [{"w": w.struct, "nsz": w.nsz, "dY": dy2, "T": None, "At": None, "mask_src": None, "r": 0, "s": 0.0}], dy2.shape[0], w.K)
+        if w.perm is not None:
+            dx = fmsa_hip.permute_cols(dx, w.perm, gather=False)
+        return dx, None, None, None, None, None, None, None
 
 
 class QuantLinear(nn.Module):
