@@ -25,6 +25,12 @@ int launch_rms_bwd(void* dY, int64_t lddy, const void* X, int64_t ldx, const voi
                    int x_dtype, int w_dtype, hipStream_t st);
 int launch_rope(void* Q, int64_t ldq, const void* cosp, const void* sinp, int64_t ldcs, int M, int n_heads, int head_dim, int cs_rows,
                 int backward, int q_dtype, int cs_dtype, hipStream_t st);
+int launch_ce_fwd(const void* logits, int64_t ld, const int64_t* labels, int M, int V, int dtype, int vec, float* losses, float* lse,
+                  hipStream_t st);
+int launch_ce_bwd(void* logits, int64_t ld, const float* dloss, int64_t dloss_stride, const float* lse, const int64_t* labels, int M,
+                  int V, int dtype, int vec, hipStream_t st);
+int launch_ce_fused(void* logits, int64_t ld, const int64_t* labels, int M, int V, int dtype, int vec, int64_t ignore_index,
+                    const float* scale, float smoothing, float* losses, hipStream_t st);
 int launch_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, hipStream_t st);
 int launch_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype, hipStream_t st);
 int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, int M, int I, int64_t ld, int act_dtype,
@@ -290,6 +296,34 @@ int fmsa_rope_embedding(void* Q, int64_t ldq, const void* cos, const void* sin, 
   if (!aligned_rows(Q, ldq, q_dtype) || !aligned_rows(cos, ldcs, cs_dtype) || !aligned_rows(sin, ldcs, cs_dtype))
     return FMSA_ERR_ALIGN;
   return launch_rope(Q, ldq, cos, sin, ldcs, M, n_heads, head_dim, cs_rows, backward, q_dtype, cs_dtype, (hipStream_t)stream);
+}
+
+int fmsa_cross_entropy_fwd(const void* logits, int64_t ld, const int64_t* labels, int M, int V, int dtype, float* losses,
+                           float* logsumexp, void* stream) {
+  if (!logits || !labels || !losses || !logsumexp) return FMSA_ERR_NULL;
+  if (M <= 0 || V <= 0 || ld < V) return FMSA_ERR_SHAPE;
+  if (!is_float_dtype(dtype)) return FMSA_ERR_DTYPE;
+  const int vec = (V % 8 == 0) && aligned_rows(logits, ld, dtype);
+  return launch_ce_fwd(logits, ld, labels, M, V, dtype, vec, losses, logsumexp, (hipStream_t)stream);
+}
+
+int fmsa_cross_entropy_bwd(void* logits, int64_t ld, const float* dloss, int64_t dloss_stride, const float* logsumexp,
+                           const int64_t* labels, int M, int V, int dtype, void* stream) {
+  if (!logits || !labels || !dloss || !logsumexp) return FMSA_ERR_NULL;
+  if (M <= 0 || V <= 0 || ld < V || dloss_stride < 0) return FMSA_ERR_SHAPE;
+  if (!is_float_dtype(dtype)) return FMSA_ERR_DTYPE;
+  const int vec = (V % 8 == 0) && aligned_rows(logits, ld, dtype);
+  return launch_ce_bwd(logits, ld, dloss, dloss_stride, logsumexp, labels, M, V, dtype, vec, (hipStream_t)stream);
+}
+
+int fmsa_cross_entropy_fused(void* logits, int64_t ld, const int64_t* labels, int M, int V, int dtype, int64_t ignore_index,
+                             const float* scale, float label_smoothing, float* losses, void* stream) {
+  if (!logits || !labels || !losses) return FMSA_ERR_NULL;
+  if (M <= 0 || V <= 0 || ld < V) return FMSA_ERR_SHAPE;
+  if (!(label_smoothing >= 0.0f && label_smoothing <= 1.0f)) return FMSA_ERR_SHAPE;
+  if (!is_float_dtype(dtype)) return FMSA_ERR_DTYPE;
+  const int vec = (V % 8 == 0) && aligned_rows(logits, ld, dtype);
+  return launch_ce_fused(logits, ld, labels, M, V, dtype, vec, ignore_index, scale, label_smoothing, losses, (hipStream_t)stream);
 }
 
 }  // extern "C"

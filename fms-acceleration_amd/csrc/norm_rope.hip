@@ -345,3 +345,242 @@ int launch_rope(void* Q, int64_t ldq, const void* cosp, const void* sinp, int64_
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }
+
+// ---- cross entropy over the vocabulary (reference: kernels/unsloth/cross_entropy_loss.py:22-190) --------
+// forward: one workgroup per row streams the logits once with an online (max, sum exp) pair per
+// thread, combines the 256 pairs through LDS, and writes logsumexp and loss = logsumexp - x[label]
+// (0 for label == -100).  backward, in place: logits <- dloss * (exp(x - logsumexp) - [col == label]).
+namespace {
+
+template <int D> FMSA_DEVI float load1(const void* p, int64_t i);
+template <> FMSA_DEVI float load1<FMSA_F32>(const void* p, int64_t i) { return reinterpret_cast<const float*>(p)[i]; }
+template <> FMSA_DEVI float load1<FMSA_BF16>(const void* p, int64_t i) { return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]); }
+template <> FMSA_DEVI float load1<FMSA_F16>(const void* p, int64_t i) { return fp16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]); }
+template <int D> FMSA_DEVI void store1(void* p, int64_t i, float v);
+template <> FMSA_DEVI void store1<FMSA_F32>(void* p, int64_t i, float v) { reinterpret_cast<float*>(p)[i] = v; }
+template <> FMSA_DEVI void store1<FMSA_BF16>(void* p, int64_t i, float v) { reinterpret_cast<uint16_t*>(p)[i] = pack1<bf16_t>(v); }
+template <> FMSA_DEVI void store1<FMSA_F16>(void* p, int64_t i, float v) { reinterpret_cast<uint16_t*>(p)[i] = pack1<f16_t>(v); }
+
+constexpr float kLog2e = 1.44269504088896341f;
+constexpr float kLn2 = 0.69314718055994531f;
+
+// (m, s) <- (m, s) (+) (x): running maximum and sum of exp(. - m)
+FMSA_DEVI void online_add(float& m, float& s, float x) {
+  const float mn = fmaxf(m, x);
+  s = s * __builtin_amdgcn_exp2f((m - mn) * kLog2e) + __builtin_amdgcn_exp2f((x - mn) * kLog2e);
+  m = mn;
+}
+
+template <int D, bool VEC>
+__global__ __launch_bounds__(256) void ce_fwd_kernel(const void* __restrict__ logits, int64_t ld, const int64_t* __restrict__ labels,
+                                                     int V, float* __restrict__ losses, float* __restrict__ lse_out) {
+  __shared__ float red_m[256], red_s[256];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int64_t base = (int64_t)row * ld;
+  float m = -INFINITY, s = 0.f;
+  if (VEC) {
+    for (int c = 8 * tid; c < V; c += 2048) {  // V % 8 == 0
+      float x[8];
+      Vec8<D>::load(logits, base + c, x);
+      float mx = x[0];
+#pragma unroll
+      for (int k = 1; k < 8; ++k) mx = fmaxf(mx, x[k]);
+      const float mn = fmaxf(m, mx);
+      float acc = 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) acc += __builtin_amdgcn_exp2f((x[k] - mn) * kLog2e);
+      s = s * __builtin_amdgcn_exp2f((m - mn) * kLog2e) + acc;
+      m = mn;
+    }
+  } else {
+    for (int c = tid; c < V; c += 256) online_add(m, s, load1<D>(logits, base + c));
+  }
+  red_m[tid] = m;
+  red_s[tid] = s;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (tid < o) {
+      const float m2 = red_m[tid + o], s2 = red_s[tid + o];
+      const float mn = fmaxf(red_m[tid], m2);
+      // a thread that saw no element holds (-inf, 0): its term must not turn into NaN
+      const float a = red_m[tid] == -INFINITY ? 0.f : red_s[tid] * __builtin_amdgcn_exp2f((red_m[tid] - mn) * kLog2e);
+      const float b = m2 == -INFINITY ? 0.f : s2 * __builtin_amdgcn_exp2f((m2 - mn) * kLog2e);
+      red_m[tid] = mn;
+      red_s[tid] = a + b;
+    }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    const float lse = red_m[0] + __builtin_amdgcn_logf(red_s[0]) * kLn2;
+    const int64_t label = labels[row];
+    lse_out[row] = lse;
+    // a label outside [0, V) that is not -100 is a caller error: it is treated as ignored rather than read out of bounds
+    losses[row] = (label < 0 || label >= V) ? 0.f : lse - load1<D>(logits, base + label);
+  }
+}
+
+template <int D, bool VEC>
+__global__ __launch_bounds__(256) void ce_bwd_kernel(void* __restrict__ logits, int64_t ld, const float* __restrict__ dloss,
+                                                     int64_t dloss_stride, const float* __restrict__ lse,
+                                                     const int64_t* __restrict__ labels, int V) {
+  const int row = blockIdx.x;
+  const int64_t base = (int64_t)row * ld;
+  const int64_t label = labels[row];
+  const float dl = label == -100 ? 0.f : dloss[(int64_t)row * dloss_stride];
+  const float l = lse[row];
+  if (VEC) {
+    const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+    if (c >= V) return;
+    float x[8], y[8];
+    Vec8<D>::load(logits, base + c, x);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      float p = __builtin_amdgcn_exp2f((x[k] - l) * kLog2e);
+      if (c + k == label) p -= 1.0f;
+      y[k] = dl * p;
+    }
+    Vec8<D>::store(logits, base + c, y);
+  } else {
+    for (int c = blockIdx.y * 2048 + threadIdx.x; c < min(V, (int)(blockIdx.y + 1) * 2048); c += 256) {
+      float p = __builtin_amdgcn_exp2f((load1<D>(logits, base + c) - l) * kLog2e);
+      if (c == label) p -= 1.0f;
+      store1<D>(logits, base + c, dl * p);
+    }
+  }
+}
+
+
+// Loss and logits gradient in one launch (reference: fused_ops/liger_ce/cross_entropy.py:33-186): the
+// loss head calls this on each freshly computed chunk of logits, so nothing is saved for a backward
+// pass.  One workgroup per row: pass 1 streams the row (online max / sum exp, and sum x for label
+// smoothing), pass 2 re-reads it (the row was just fetched, so mostly from cache) and overwrites it
+// with  scale * (softmax - eps - [col == label] (1 - smoothing)),  eps = smoothing / V.
+// loss = scale * ((1 - smoothing) (lse - x[label]) + smoothing * lse - eps * sum x).  Rows whose label
+// equals ignore_index get loss 0 and an all-zero gradient.  `scale` is read from device memory so the
+// caller never has to wait for the count of valid labels.
+template <int D, bool VEC>
+__global__ __launch_bounds__(256) void ce_fused_kernel(void* __restrict__ logits, int64_t ld, const int64_t* __restrict__ labels,
+                                                       int V, int64_t ignore_index, const float* __restrict__ scale_ptr,
+                                                       float smoothing, float* __restrict__ losses) {
+  __shared__ float red_m[256], red_s[256], red_x[256];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int64_t base = (int64_t)row * ld;
+  const int64_t label = labels[row];
+  if (label == ignore_index || label < 0 || label >= V) {  // uniform over the workgroup; out-of-range labels count as ignored
+    if (VEC) {
+      float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (int c = 8 * tid; c < V; c += 2048) Vec8<D>::store(logits, base + c, z);
+    } else {
+      for (int c = tid; c < V; c += 256) store1<D>(logits, base + c, 0.f);
+    }
+    if (tid == 0) losses[row] = 0.f;
+    return;
+  }
+  const float scale = scale_ptr ? scale_ptr[0] : 1.0f;
+  const float x_label = load1<D>(logits, base + label);  // read by every thread before any store of pass 2
+  float m = -INFINITY, s = 0.f, sx = 0.f;
+  if (VEC) {
+    for (int c = 8 * tid; c < V; c += 2048) {
+      float x[8];
+      Vec8<D>::load(logits, base + c, x);
+      float mx = x[0];
+#pragma unroll
+      for (int k = 1; k < 8; ++k) mx = fmaxf(mx, x[k]);
+      const float mn = fmaxf(m, mx);
+      float acc = 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        acc += __builtin_amdgcn_exp2f((x[k] - mn) * kLog2e);
+        sx += x[k];
+      }
+      s = s * __builtin_amdgcn_exp2f((m - mn) * kLog2e) + acc;
+      m = mn;
+    }
+  } else {
+    for (int c = tid; c < V; c += 256) {
+      const float x = load1<D>(logits, base + c);
+      online_add(m, s, x);
+      sx += x;
+    }
+  }
+  red_m[tid] = m;
+  red_s[tid] = s;
+  red_x[tid] = sx;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (tid < o) {
+      const float m2 = red_m[tid + o], s2 = red_s[tid + o];
+      const float mn = fmaxf(red_m[tid], m2);
+      const float a = red_m[tid] == -INFINITY ? 0.f : red_s[tid] * __builtin_amdgcn_exp2f((red_m[tid] - mn) * kLog2e);
+      const float b = m2 == -INFINITY ? 0.f : s2 * __builtin_amdgcn_exp2f((m2 - mn) * kLog2e);
+      red_m[tid] = mn;
+      red_s[tid] = a + b;
+      red_x[tid] += red_x[tid + o];
+    }
+    __syncthreads();
+  }
+  const float lse = red_m[0] + __builtin_amdgcn_logf(red_s[0]) * kLn2;
+  const float eps = smoothing / (float)V;
+  if (tid == 0) losses[row] = scale * ((1.0f - smoothing) * (lse - x_label) + (smoothing * lse - eps * red_x[0]));
+  const float hit = 1.0f - smoothing;
+  if (VEC) {
+    for (int c = 8 * tid; c < V; c += 2048) {
+      float x[8], y[8];
+      Vec8<D>::load(logits, base + c, x);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        float p = __builtin_amdgcn_exp2f((x[k] - lse) * kLog2e) - eps;
+        if (c + k == label) p -= hit;
+        y[k] = scale * p;
+      }
+      Vec8<D>::store(logits, base + c, y);
+    }
+  } else {
+    for (int c = tid; c < V; c += 256) {
+      float p = __builtin_amdgcn_exp2f((load1<D>(logits, base + c) - lse) * kLog2e) - eps;
+      if (c == label) p -= hit;
+      store1<D>(logits, base + c, scale * p);
+    }
+  }
+}
+
+}  // namespace
+
+int launch_ce_fwd(const void* logits, int64_t ld, const int64_t* labels, int M, int V, int dtype, int vec, float* losses, float* lse,
+                  hipStream_t st) {
+  dim3 grid(M), block(256);
+  FMSA_DISPATCH_DTYPE(dtype, D, {
+    if (vec)
+      hipLaunchKernelGGL((ce_fwd_kernel<D, true>), grid, block, 0, st, logits, ld, labels, V, losses, lse);
+    else
+      hipLaunchKernelGGL((ce_fwd_kernel<D, false>), grid, block, 0, st, logits, ld, labels, V, losses, lse);
+  })
+  FMSA_CHECK_LAUNCH();
+  return FMSA_OK;
+}
+
+int launch_ce_bwd(void* logits, int64_t ld, const float* dloss, int64_t dloss_stride, const float* lse, const int64_t* labels, int M,
+                  int V, int dtype, int vec, hipStream_t st) {
+  dim3 grid(M, (V + 2047) / 2048), block(256);
+  FMSA_DISPATCH_DTYPE(dtype, D, {
+    if (vec)
+      hipLaunchKernelGGL((ce_bwd_kernel<D, true>), grid, block, 0, st, logits, ld, dloss, dloss_stride, lse, labels, V);
+    else
+      hipLaunchKernelGGL((ce_bwd_kernel<D, false>), grid, block, 0, st, logits, ld, dloss, dloss_stride, lse, labels, V);
+  })
+  FMSA_CHECK_LAUNCH();
+  return FMSA_OK;
+}
+
+int launch_ce_fused(void* logits, int64_t ld, const int64_t* labels, int M, int V, int dtype, int vec, int64_t ignore_index,
+                    const float* scale, float smoothing, float* losses, hipStream_t st) {
+  dim3 grid(M), block(256);
+  FMSA_DISPATCH_DTYPE(dtype, D, {
+    if (vec)
+      hipLaunchKernelGGL((ce_fused_kernel<D, true>), grid, block, 0, st, logits, ld, labels, V, ignore_index, scale, smoothing, losses);
+    else
+      hipLaunchKernelGGL((ce_fused_kernel<D, false>), grid, block, 0, st, logits, ld, labels, V, ignore_index, scale, smoothing, losses);
+  })
+  FMSA_CHECK_LAUNCH();
+  return FMSA_OK;
+}

@@ -2,8 +2,9 @@
 ModelPatcher rules (reference: fms_acceleration_foak/framework_plugin_fast_kernels.py:31-222).
 
 Switches with kernels behind them in this build: `fused_lora` (rule suffixes "qkvo", "mlp"),
-`fast_rms_layernorm` ("rms") and `fast_rope_embeddings` ("rope").  `fast_loss` is accepted and
-validated so that existing YAML files load unchanged, but it selects no rule here.
+`fast_rms_layernorm` ("rms"), `fast_rope_embeddings` ("rope"), `fast_loss: true` ("cross-ent",
+"custom-loss") and `fast_loss: fused_ce_liger` ("fused-lce": llama, mistral and granite, as in the
+reference).
 """
 from __future__ import annotations
 

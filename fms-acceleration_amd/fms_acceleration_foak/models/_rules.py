@@ -1,7 +1,8 @@
 """Shared construction of the patch rules: `<arch>-qkvo` / `<arch>-mlp` (fused LoRA; the
 architectures differ only in their attention / MLP classes, reference models/llama.py:73-123,
 mistral.py:70-119, granite.py:78-128), `<arch>-rms` (RMS layer norm forward replaced, llama.py:65-69)
-and `<arch>-rope` (the modelling module's apply_rotary_pos_emb replaced, llama.py:154-161)."""
+`<arch>-rope` (the modelling module's apply_rotary_pos_emb replaced, llama.py:154-161) and the loss
+rule (`<arch>-custom-loss` on transformers >= 4.46, else `<arch>-cross-ent`, llama.py:129-149)."""
 from __future__ import annotations
 
 import warnings
@@ -69,3 +70,33 @@ def norm_rope_rules(arch: str, rms_cls, modeling_module: str):
             import_and_maybe_reload=(f"{modeling_module}.apply_rotary_pos_emb", fast_rope_embedding, None),
         ),
     ]
+
+
+def loss_rules(arch: str, causal_lm_cls, modeling_module: str):
+    """The fast cross-entropy rule: newer transformers route the loss through `model.loss_function`
+    (LOSS_MAPPING), older ones instantiate torch.nn.CrossEntropyLoss inside the modelling module."""
+    import transformers  # pylint: disable=import-outside-toplevel
+    from packaging.version import Version  # pylint: disable=import-outside-toplevel
+
+    from ..kernels.unsloth import FastCrossEntropyLoss, replace_custom_loss_when_triggered  # pylint: disable=import-outside-toplevel
+
+    if Version(transformers.__version__) >= Version("4.46"):
+        return [
+            ModelPatcherRule(
+                rule_id=f"{arch}-custom-loss",
+                trigger=ModelPatcherTrigger(check=replace_custom_loss_when_triggered(causal_lm_cls, custom_loss_type=f"{arch}-custom-loss")),
+            )
+        ]
+    return [
+        ModelPatcherRule(
+            rule_id=f"{arch}-cross-ent",
+            import_and_maybe_reload=("torch.nn.CrossEntropyLoss", FastCrossEntropyLoss, modeling_module),
+        )
+    ]
+
+
+def fused_lce_rules(arch: str, causal_lm_cls):
+    """`<arch>-fused-lce`: the causal-LM forward with the lm_head matmul and the loss fused."""
+    from ..fused_ops.liger_ce import lce_forward  # pylint: disable=import-outside-toplevel
+
+    return [ModelPatcherRule(rule_id=f"{arch}-fused-lce", trigger=ModelPatcherTrigger(check=causal_lm_cls), forward=lce_forward)]

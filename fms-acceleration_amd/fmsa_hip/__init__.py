@@ -41,6 +41,9 @@ EXPORTED_SYMBOLS = (
     "fmsa_rms_layernorm_fwd",
     "fmsa_rms_layernorm_bwd",
     "fmsa_rope_embedding",
+    "fmsa_cross_entropy_fwd",
+    "fmsa_cross_entropy_bwd",
+    "fmsa_cross_entropy_fused",
 )
 
 
@@ -143,6 +146,9 @@ def lib() -> ctypes.CDLL:
                                          c_int, c_void_p]
     L.fmsa_rope_embedding.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int,
                                       c_int, c_void_p]
+    L.fmsa_cross_entropy_fwd.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+    L.fmsa_cross_entropy_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]
+    L.fmsa_cross_entropy_fused.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int64, c_void_p, c_float, c_void_p, c_void_p]
     for name in EXPORTED_SYMBOLS:
         getattr(L, name)  # AttributeError here means the library is stale: rebuild it
     _lib = L
@@ -405,3 +411,43 @@ def rope_embedding_(q2d, cos2d, sin2d, n_heads: int, head_dim: int, backward: bo
                                      head_dim, cos2d.shape[0], int(backward), _DTYPE_ENUM[q2d.dtype], _DTYPE_ENUM[cos2d.dtype],
                                      _stream(q2d)))
     return q2d
+
+
+def cross_entropy_fwd(logits2d, labels):
+    """(losses [M] fp32, logsumexp [M] fp32); labels int64 [M], -100 ignored."""
+    if not (logits2d.is_cuda and labels.is_cuda):
+        raise RuntimeError("fmsa_hip needs GPU tensors")
+    M, V = logits2d.shape
+    assert logits2d.stride(1) == 1 and labels.dtype == torch.int64 and labels.is_contiguous() and labels.numel() == M
+    losses = torch.empty(M, dtype=torch.float32, device=logits2d.device)
+    lse = torch.empty(M, dtype=torch.float32, device=logits2d.device)
+    _check("fmsa_cross_entropy_fwd", lib().fmsa_cross_entropy_fwd(_ptr(logits2d), logits2d.stride(0), _ptr(labels), M, V,
+                                                                  _DTYPE_ENUM[logits2d.dtype], _ptr(losses), _ptr(lse), _stream(logits2d)))
+    return losses, lse
+
+
+def cross_entropy_bwd_(logits2d, dlosses, lse, labels):
+    """Overwrites logits2d with the gradient and returns it; dlosses [M] fp32 (any stride, 0 included)."""
+    M, V = logits2d.shape
+    assert dlosses.dtype == torch.float32 and dlosses.numel() == M and dlosses.dim() == 1
+    _check("fmsa_cross_entropy_bwd", lib().fmsa_cross_entropy_bwd(_ptr(logits2d), logits2d.stride(0), _ptr(dlosses), dlosses.stride(0),
+                                                                  _ptr(lse), _ptr(labels), M, V, _DTYPE_ENUM[logits2d.dtype],
+                                                                  _stream(logits2d)))
+    return logits2d
+
+
+def cross_entropy_fused_(logits2d, labels, scale=None, label_smoothing=0.0, ignore_index=-100, losses_out=None):
+    """Overwrites logits2d with scale * d(loss)/d(logits) and returns (losses [M] fp32, already scaled;
+    logits2d).  `scale` is a 1-element fp32 GPU tensor (None = 1)."""
+    if not (logits2d.is_cuda and labels.is_cuda):
+        raise RuntimeError("fmsa_hip needs GPU tensors")
+    M, V = logits2d.shape
+    assert logits2d.stride(1) == 1 and labels.dtype == torch.int64 and labels.is_contiguous() and labels.numel() == M
+    assert scale is None or (scale.is_cuda and scale.dtype == torch.float32 and scale.numel() == 1)
+    losses = losses_out if losses_out is not None else torch.empty(M, dtype=torch.float32, device=logits2d.device)
+    assert losses.dtype == torch.float32 and losses.is_contiguous() and losses.numel() == M
+    _check("fmsa_cross_entropy_fused",
+           lib().fmsa_cross_entropy_fused(_ptr(logits2d), logits2d.stride(0), _ptr(labels), M, V, _DTYPE_ENUM[logits2d.dtype],
+                                          int(ignore_index), _ptr(scale) if scale is not None else None, float(label_smoothing),
+                                          _ptr(losses), _stream(logits2d)))
+    return losses, logits2d

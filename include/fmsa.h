@@ -228,6 +228,35 @@ int fmsa_rope_embedding(void* Q, int64_t ldq, const void* cos, const void* sin, 
                         int n_heads, int head_dim, int cs_rows, int backward, int q_dtype, int cs_dtype,
                         void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Cross entropy over the vocabulary (kernels/unsloth/cross_entropy_loss.py:22-73 forward,
+ * :138-190 backward; any vocabulary size in one pass, so the reference's chunked variant :76-135 has
+ * no separate counterpart).  logits [M, V] of dtype F32 / BF16 / F16, labels int64 [M], -100 = ignore.
+ *   fwd: logsumexp[m] = log sum_v exp(x[m, v]);  losses[m] = logsumexp[m] - x[m, label] (0 if ignored)
+ *   bwd: in place, logits[m, v] <- dloss[m] * (exp(x[m, v] - logsumexp[m]) - [v == label]);
+ *        dloss is read with stride dloss_stride (0 for the expanded scalar of a mean reduction).
+ * 16-byte vector accesses when V % 8 == 0 and rows are 16-byte aligned, element accesses otherwise.
+ * ------------------------------------------------------------------------------------------ */
+int fmsa_cross_entropy_fwd(const void* logits, int64_t ld, const int64_t* labels, int M, int V, int dtype,
+                           float* losses, float* logsumexp, void* stream);
+int fmsa_cross_entropy_bwd(void* logits, int64_t ld, const float* dloss, int64_t dloss_stride,
+                           const float* logsumexp, const int64_t* labels, int M, int V, int dtype,
+                           void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Loss and logits gradient in one launch, for a loss head that consumes its logits chunk by chunk
+ * (fused_ops/liger_ce/cross_entropy.py:33-186, called from
+ * fused_ops/liger_ce/fused_linear_cross_entropy_loss.py:107-121).  In place on logits [M, V]:
+ *   losses[m]   = scale * ((1 - ls) (lse - x[m, label]) + ls * lse - (ls / V) sum_v x[m, v])
+ *   logits[m,v] <- scale * (softmax(x[m])[v] - ls / V - [v == label] (1 - ls))
+ * with ls = label_smoothing in [0, 1]; rows whose label equals ignore_index (or lies outside [0, V))
+ * get loss 0 and a zero gradient row.  `scale` points at ONE fp32 in device memory (1 / number of
+ * valid labels for a mean reduction) or is NULL for 1.
+ * ------------------------------------------------------------------------------------------ */
+int fmsa_cross_entropy_fused(void* logits, int64_t ld, const int64_t* labels, int M, int V, int dtype,
+                             int64_t ignore_index, const float* scale, float label_smoothing, float* losses,
+                             void* stream);
+
 #ifdef __cplusplus
 }
 #endif

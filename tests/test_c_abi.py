@@ -133,3 +133,20 @@ def test_norm_rope_validation():
     assert rp(0x1000, 256, 0x2000, 0x3000, 64, 8, 4, 24, 8, 0, 1, 1, None) == -2          # head_dim % 16
     assert rp(0x1000, 128, 0x2000, 0x3000, 64, 8, 4, 64, 8, 0, 1, 1, None) == -2          # ldq < heads * head_dim
     assert rp(0x1000, 256, 0x2000, 0x3000, 64, 8, 4, 64, 0, 0, 1, 1, None) == -2          # no cos rows
+
+
+def test_cross_entropy_validation():
+    lib = fmsa_hip.lib()
+    f = lib.fmsa_cross_entropy_fwd
+    assert f(0x1000, 64, None, 8, 64, 2, 0x2000, 0x3000, None) == -1
+    assert f(0x1000, 32, 0x4000, 8, 64, 2, 0x2000, 0x3000, None) == -2   # ld < V
+    assert f(0x1000, 64, 0x4000, 8, 64, 9, 0x2000, 0x3000, None) == -4
+    b = lib.fmsa_cross_entropy_bwd
+    assert b(0x1000, 64, None, 1, 0x2000, 0x4000, 8, 64, 2, None) == -1
+    assert b(0x1000, 64, 0x5000, -1, 0x2000, 0x4000, 8, 64, 2, None) == -2
+    u = lib.fmsa_cross_entropy_fused
+    assert u(0x1000, 64, None, 8, 64, 2, -100, None, 0.0, 0x2000, None) == -1
+    assert u(0x1000, 64, 0x4000, 8, 64, 2, -100, None, 0.0, None, None) == -1
+    assert u(0x1000, 32, 0x4000, 8, 64, 2, -100, None, 0.0, 0x2000, None) == -2   # ld < V
+    assert u(0x1000, 64, 0x4000, 8, 64, 2, -100, None, 1.5, 0x2000, None) == -2   # smoothing outside [0, 1]
+    assert u(0x1000, 64, 0x4000, 8, 64, 7, -100, None, 0.0, 0x2000, None) == -4

@@ -45,7 +45,8 @@ def _patched_copy(module, cfg):
         for rule in llama.get_mp_rules("auto_gptq", cfg):
             ModelPatcher.register(rule)
         patch_model(twin)
-        n_patched = len(ModelPatcher.history)
+        # the rope rule swaps a function of the modeling module: it is not one of the twin's patched forwards
+        n_patched = sum(1 for h in ModelPatcher.history if not h.rule_id.endswith("-rope"))
     return twin, n_patched
 
 

@@ -83,14 +83,15 @@ def test_checkpoint_to_patched_training_step(tmp_path):
 
     loss_ref, grads_ref = step(plain)
     plugin = FastKernelsAccelerationPlugin({"training": {"fused_ops_and_kernels": {
-        "fused_lora": True, "fast_rms_layernorm": True, "fast_rope_embeddings": True}}})
+        "fused_lora": True, "fast_loss": True, "fast_rms_layernorm": True, "fast_rope_embeddings": True}}})
     original = ml.apply_rotary_pos_emb
     try:
         with instantiate_model_patcher():
             plugin.augmentation(model, type("T", (), {"bf16": True, "fp16": False})(), ())
             patch_model(model)
             done = {h.rule_id for h in ModelPatcher.history}
-            assert {"llama-mlp", "llama-rms", "llama-rope"} <= done and any(d.startswith("llama-qkvo") for d in done)
+            assert {"llama-mlp", "llama-rms", "llama-rope", "llama-custom-loss"} <= done
+            assert any(d.startswith("llama-qkvo") for d in done) and model.loss_type == "llama-custom-loss"
             loss, grads = step(model)
     finally:
         ml.apply_rotary_pos_emb = original

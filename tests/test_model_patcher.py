@@ -149,7 +149,9 @@ def test_fused_lora_rules_patch_llama_modules():
     train_args = type("T", (), {"bf16": True, "fp16": False})()
     with instantiate_model_patcher():
         plugin.augmentation(block, train_args, ())
-        assert set(ModelPatcher.rules) == {
+        archs = ["llama", "mistral", "granite", "mixtral", "granitemoe", "granitemoeshared", "granitemoehybrid"]
+        loss_ids = {f"{a}-custom-loss" for a in archs}  # transformers >= 4.46 here
+        assert set(ModelPatcher.rules) == loss_ids | {
             "llama-qkvo", "llama-mlp", "mistral-qkvo", "mistral-mlp", "granite-qkvo", "granite-mlp",
             "mixtral-qkvo", "granitemoe-qkvo", "granitemoeshared-qkvo", "granitemoehybrid-qkvo"}
         patch_model(block)
@@ -164,7 +166,12 @@ def test_fused_lora_rules_patch_llama_modules():
     block2, _ = _tiny_llama_layer()
     with instantiate_model_patcher():
         plugin.augmentation(block2, train_args, ())
-        assert set(ModelPatcher.rules) == set()
+        assert set(ModelPatcher.rules) == loss_ids
+    # `fast_loss: fused_ce_liger` selects the fused loss head, for the dense-attention families only
+    liger = FastKernelsAccelerationPlugin({"training": {"fused_ops_and_kernels": {"fast_loss": "fused_ce_liger"}}})
+    with instantiate_model_patcher():
+        liger.augmentation(block2, train_args, ())
+        assert set(ModelPatcher.rules) == {"llama-fused-lce", "mistral-fused-lce", "granite-fused-lce"}
     # mixed precision is mandatory on a quantised base
     with instantiate_model_patcher():
         with pytest.raises(AssertionError, match="mixed precision"):
@@ -178,7 +185,7 @@ def test_mlp_rule_dropped_for_non_silu_activation():
     with warnings.catch_warnings(record=True):
         warnings.simplefilter("always")
         ids = [r.rule_id for r in llama.get_mp_rules("auto_gptq", cfg)]
-    assert ids == ["llama-qkvo", "llama-rms", "llama-rope"]
+    assert ids == ["llama-qkvo", "llama-fused-lce", "llama-custom-loss", "llama-rms", "llama-rope"]
 
 
 def test_partial_lora_follows_the_reference_rule_logic():
