@@ -7,23 +7,27 @@
 namespace {
 
 // ---- lora_down ----------------------------------------------------------------------------------
-// One workgroup = 16 * MTL tokens; its 4 waves split C into 4 contiguous quarters and each runs
-// MFMA 16x16x32 over its quarter (X fragments straight from global: 16 rows x 64 B per load; a Wd
-// fragment is loaded once per step and used for all MTL token tiles), then the four partial
-// [16 * MTL x r] tiles are summed through LDS in a fixed order.
-template <typename T, int RT, int MTL>
-__global__ __launch_bounds__(256) void lora_down_kernel(const uint16_t* __restrict__ X, int64_t ldx,
-                                                        const uint16_t* __restrict__ Wd, int M, int C, int r,
-                                                        uint16_t* __restrict__ out, int64_t ldo) {
-  __shared__ float red[4][MTL][RT][64][4];
+// One workgroup = 16 * MTL tokens; its NW waves split C into NW contiguous slices and each runs
+// MFMA 16x16x32 over its slice (X fragments straight from global: 16 rows x 64 B per load; a Wd
+// fragment is loaded once per step and used for all MTL token tiles).  The kernel lives on memory
+// latency, so a workgroup is up to 16 waves: that many independent load streams per CU are what
+// keeps enough bytes in flight.  The NW partial [16 * MTL x r] tiles are summed through LDS in a
+// fixed order: the upper half of the waves hands its tiles to the lower half, whose sums are then
+// added up by all threads.
+template <typename T, int RT, int MTL, int NW>
+__global__ __launch_bounds__(64 * NW) void lora_down_kernel(const uint16_t* __restrict__ X, int64_t ldx,
+                                                            const uint16_t* __restrict__ Wd, int M, int C, int r,
+                                                            uint16_t* __restrict__ out, int64_t ldo) {
+  constexpr int NH = NW / 2;
+  __shared__ float red[NH][MTL][RT][64][4];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int l16 = lane & 15, q = lane >> 4;
   const int m_base = blockIdx.x * (16 * MTL);
-  // quarter boundaries in units of 32 columns
+  // slice boundaries in units of 32 columns
   const int n32 = (C + 31) / 32;
-  const int per = (n32 + 3) / 4;
-  const int c_begin = wave * per * 32;
+  const int per = (n32 + NW - 1) / NW;
+  const int c_begin = min(C, wave * per * 32);
   const int c_end = min(C, (wave + 1) * per * 32);
 
   f32x4 acc[MTL][RT];
@@ -58,17 +62,29 @@ __global__ __launch_bounds__(256) void lora_down_kernel(const uint16_t* __restri
       for (int u = 0; u < MTL; ++u) acc[u][t] = mfma16<T>(xf[u], wf, acc[u][t]);  // D[i = token][j = rank]
     }
   }
+  if (wave >= NH) {
 #pragma unroll
-  for (int u = 0; u < MTL; ++u)
+    for (int u = 0; u < MTL; ++u)
 #pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) red[wave][u][t][lane][i] = acc[u][t][i];
+      for (int t = 0; t < RT; ++t) *reinterpret_cast<f32x4*>(red[wave - NH][u][t][lane]) = acc[u][t];
+  }
   __syncthreads();
-  // lane l of a tile holds D[4*(l>>4) + i][l & 15]; 256 threads sum MTL*RT*256 outputs
-  for (int o = tid; o < MTL * RT * 256; o += 256) {
+  if (wave < NH) {
+#pragma unroll
+    for (int u = 0; u < MTL; ++u)
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const f32x4 o = *reinterpret_cast<const f32x4*>(red[wave][u][t][lane]);
+        *reinterpret_cast<f32x4*>(red[wave][u][t][lane]) = acc[u][t] + o;
+      }
+  }
+  __syncthreads();
+  // lane l of a tile holds D[4*(l>>4) + i][l & 15]; all threads sum MTL*RT*256 outputs over the NH slots
+  for (int o = tid; o < MTL * RT * 256; o += 64 * NW) {
     const int u = o / (RT * 256), t = (o >> 8) % RT, ln = (o >> 2) & 63, i = o & 3;
-    const float v = (red[0][u][t][ln][i] + red[1][u][t][ln][i]) + (red[2][u][t][ln][i] + red[3][u][t][ln][i]);
+    float v = red[0][u][t][ln][i];
+#pragma unroll
+    for (int w = 1; w < NH; ++w) v += red[w][u][t][ln][i];
     const int row = m_base + 16 * u + 4 * (ln >> 4) + i;
     const int j = 16 * t + (ln & 15);
     if (row < M && j < r) out[(size_t)row * ldo + j] = pack1<T>(v);
@@ -227,16 +243,17 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
                      int64_t ldo, hipStream_t st) {
   // 32 tokens per workgroup once that still leaves a workgroup per CU (halves the re-reads of Wd)
   const int mtl = (M >= 32 * 256 && r <= 64) ? 2 : 1;
-  dim3 grid((M + 16 * mtl - 1) / (16 * mtl)), block(256);
+  constexpr int NW = 8;  // waves per workgroup: measured best of 4 / 8 / 16 at 8192 tokens
+  dim3 grid((M + 16 * mtl - 1) / (16 * mtl)), block(64 * NW);
   const int rt = (r + 15) / 16;
-#define LAUNCH(TT, RT)                                                                                                   \
-  do {                                                                                                                   \
-    if (mtl == 2)                                                                                                        \
-      hipLaunchKernelGGL((lora_down_kernel<TT, RT, 2>), grid, block, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, \
-                         M, C, r, (uint16_t*)out, ldo);                                                                  \
-    else                                                                                                                 \
-      hipLaunchKernelGGL((lora_down_kernel<TT, RT, 1>), grid, block, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, \
-                         M, C, r, (uint16_t*)out, ldo);                                                                  \
+#define LAUNCH(TT, RT)                                                                                                       \
+  do {                                                                                                                       \
+    if (mtl == 2)                                                                                                            \
+      hipLaunchKernelGGL((lora_down_kernel<TT, RT, (RT > 4 ? 1 : 2), NW>), grid, block, 0, st, (const uint16_t*)X, ldx,       \
+                         (const uint16_t*)Wd, M, C, r, (uint16_t*)out, ldo);                                                 \
+    else                                                                                                                     \
+      hipLaunchKernelGGL((lora_down_kernel<TT, RT, 1, NW>), grid, block, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, \
+                         M, C, r, (uint16_t*)out, ldo);                                                                      \
   } while (0)
 #define DISPATCH(TT)            \
   switch (rt) {                 \
