@@ -66,7 +66,7 @@ struct BwdArgs {
 
 FMSA_DEVI BwdProjDev select_proj(const BwdArgs& a, int p) { return p == 0 ? a.p[0] : (p == 1 ? a.p[1] : a.p[2]); }
 
-template <typename T, bool NTAIL>
+template <typename T, bool NTAIL, int MODE>
 __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) {
   // separate arrays per stage buffer: every access names its buffer statically, so the compiler
   // can tell fragment reads of one buffer from the direct loads in flight into the other
@@ -313,51 +313,57 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
 
   // ---- epilogue ---------------------------------------------------------------------------
   // register 4*i0+i1 of acc[mt][j] is dX[m0 + 32*mt + l32][8*(k8base + 8*i0 + 4*half + i1) + 2*wave + j]
+  //
+  // Four passes of 64 tokens.  Each pass (a) "dump": the waves round their accumulators (and the
+  // LoRA product of the pass, formed by a few more MFMAs) into two LDS planes, (b) "sweep": all
+  // 256 threads walk the planes in coalesced order -- lane = (row tid/32 of each group of 8 rows,
+  // 8-column chunk tid%32) -- apply the mode's arithmetic and store.  The code of an epilogue runs
+  // once per tile, so its size is what it costs (instruction fetch): the mode is a template
+  // parameter, the pass loop is a real loop around ONE copy of the sweep, and only the small
+  // dump, which names accumulator registers, exists four times.  All global accesses go through
+  // buffer resources over the tile's rows, so rows past M and columns past K need no branches
+  // (loads return zero, stores are dropped).  The operands the sweep of pass q+1 reads (e and g,
+  // the mask source) are requested during the sweep of pass q, each into the registers the sweep
+  // has just consumed, so no load is ever waited for right after its issue.
   __builtin_amdgcn_s_waitcnt(WAIT_VM0);  // the surplus direct loads of the last stage have landed
   __syncthreads();
+  constexpr bool swiglu = MODE == FMSA_BWD_SWIGLU;
   uint16_t* base_plane = ep_planes;
   uint16_t* lora_plane = base_plane + EP_ROWS * EP_STRIDE;
   bool any_lora = false;
   for (int p = 0; p < a.n_proj; ++p) any_lora = any_lora || (select_proj(a, p).r > 0);
   const int kcol_lane = 8 * (k8base + l32) + 2 * wave;  // column whose A^T row this lane feeds to the LoRA MFMA
   const int k_tile0 = 8 * k8base;
-  // Coalesced side of the epilogue: lane = (row tid/32 of each group of 8 rows, 8-column chunk
-  // tid%32).  All global accesses go through buffer resources over the tile's rows, so rows past M
-  // and columns past K need no branches (loads return zero, stores are dropped), and the loads of a
-  // whole 64-row pass (e and g, or the mask source) are in flight one pass ahead of their use.
-  const bool swiglu = a.mode == FMSA_BWD_SWIGLU;
   const int chunk = tid & 31;
   const uint32_t col_dead = (k_tile0 + 8 * chunk) < K ? 0u : 0x80000000u;
   const uint32_t eg_row_bytes = __builtin_amdgcn_readfirstlane((uint32_t)(a.ldeg * 2));
   const uint32_t dx_row_bytes = __builtin_amdgcn_readfirstlane((uint32_t)(a.lddx * 2));
   const uint32_t mk_row_bytes = __builtin_amdgcn_readfirstlane((uint32_t)(a.ldmask * 2));
+  const bool has_mask = a.mask_src != nullptr && any_lora;
   const __amdgpu_buffer_rsrc_t e_rsrc = make_rsrc(a.e + (size_t)m0 * a.ldeg, swiglu ? (size_t)rows_valid * a.ldeg * 2 : 0);
   const __amdgpu_buffer_rsrc_t g_rsrc = make_rsrc(a.g + (size_t)m0 * a.ldeg, swiglu ? (size_t)rows_valid * a.ldeg * 2 : 0);
   const __amdgpu_buffer_rsrc_t h_rsrc = make_rsrc(a.h + (size_t)m0 * a.ldeg, swiglu ? (size_t)rows_valid * a.ldeg * 2 : 0);
   const __amdgpu_buffer_rsrc_t dx_rsrc = make_rsrc(a.dX + (size_t)m0 * a.lddx, swiglu ? 0 : (size_t)rows_valid * a.lddx * 2);
+  // without a mask source the resource is empty: its loads cost no traffic and return zeros
   const __amdgpu_buffer_rsrc_t mk_rsrc =
-      make_rsrc(a.mask_src + (size_t)m0 * a.ldmask, a.mask_src ? (size_t)rows_valid * a.ldmask * 2 : 0);
+      make_rsrc(a.mask_src + (size_t)m0 * a.ldmask, has_mask ? (size_t)rows_valid * a.ldmask * 2 : 0);
   const uint32_t eg_voff = (uint32_t)(((tid >> 5) * a.ldeg + k_tile0 + 8 * chunk) * 2) | col_dead;
   const uint32_t dx_voff = (uint32_t)(((tid >> 5) * a.lddx + k_tile0 + 8 * chunk) * 2) | col_dead;
   const uint32_t mk_voff = (uint32_t)(((tid >> 5) * a.ldmask + k_tile0 + 8 * chunk) * 2) | col_dead;
-  u32x4 pre_a[2][EP_ROWS / 8], pre_b[2][EP_ROWS / 8];
-  auto issue_loads = [&](auto q_c) {
-    constexpr int q = decltype(q_c)::value;
-    if (swiglu) {
-#pragma unroll
-      for (int it = 0; it < EP_ROWS / 8; ++it) {
-        pre_a[q & 1][it] = __builtin_amdgcn_raw_buffer_load_b128(e_rsrc, eg_voff, (uint32_t)(EP_ROWS * q + 8 * it) * eg_row_bytes, 0);
-        pre_b[q & 1][it] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, eg_voff, (uint32_t)(EP_ROWS * q + 8 * it) * eg_row_bytes, 0);
-      }
-    } else if (a.mask_src && any_lora) {
-#pragma unroll
-      for (int it = 0; it < EP_ROWS / 8; ++it)
-        pre_a[q & 1][it] = __builtin_amdgcn_raw_buffer_load_b128(mk_rsrc, mk_voff, (uint32_t)(EP_ROWS * q + 8 * it) * mk_row_bytes, 0);
+  constexpr int SWEEP = EP_ROWS * 32 / 256;  // 16-byte chunks per thread and pass
+  u32x4 pre_e[swiglu ? SWEEP : 1], pre_g[swiglu ? SWEEP : 1], pre_m[SWEEP];
+  auto issue_loads = [&](int q, auto it_c) {  // operands of chunk `it` of pass q
+    constexpr int it = decltype(it_c)::value;
+    const uint32_t row = (uint32_t)(EP_ROWS * q + 8 * it);
+    if constexpr (swiglu) {
+      pre_e[it] = __builtin_amdgcn_raw_buffer_load_b128(e_rsrc, eg_voff, row * eg_row_bytes, 0);
+      pre_g[it] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, eg_voff, row * eg_row_bytes, 0);
     }
+    pre_m[it] = __builtin_amdgcn_raw_buffer_load_b128(mk_rsrc, mk_voff, row * mk_row_bytes, 0);
   };
   // LoRA operands of the first 16 ranks of every projection: the A^T fragments of the lane's two
   // columns are the same for all token tiles (loaded once), the T fragments of the two token tiles
-  // of a pass are fetched one pass ahead, so their latency hides behind the coalesced stores.
+  // of a pass are fetched one pass ahead.
   u32x4 af0[3][NT], tf0[3][2];
   bool lora_live[3];
   static_for<0, 3>([&](auto p_c) {
@@ -370,8 +376,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       if (lora_live[p] && row_ok && 8 * half < P.r) af0[p][j] = *reinterpret_cast<const u32x4*>(P.At + (size_t)(kcol_lane + j) * P.r + 8 * half);
     }
   });
-  auto load_tf = [&](auto q_c) {
-    constexpr int q = decltype(q_c)::value;
+  auto load_tf = [&](int q) {
     static_for<0, 3>([&](auto p_c) {
       constexpr int p = decltype(p_c)::value;
       const BwdProjDev& P = a.p[p];
@@ -383,22 +388,20 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       }
     });
   };
-  load_tf(std::integral_constant<int, 0>{});
-  issue_loads(std::integral_constant<int, 0>{});
-
-  static_for<0, MT / 2>([&](auto q_c) {
+  // (a) of pass q: accumulators of token tiles 2q, 2q+1 (+ their LoRA products) -> planes
+  auto dump = [&](auto q_c) {
     constexpr int q = decltype(q_c)::value;
     static_for<0, 2>([&](auto ml_c) {
       constexpr int ml = decltype(ml_c)::value;
       constexpr int mt = 2 * q + ml;
       const int m = m0 + 32 * mt + l32;
       const bool m_ok = m < a.M;
-      f32x16 lora[NT];
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) lora[j][i] = 0.f;
       if (any_lora) {
+        f32x16 lora[NT];
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) lora[j][i] = 0.f;
         static_for<0, 3>([&](auto p_c) {
           constexpr int p = decltype(p_c)::value;
           if (lora_live[p]) {
@@ -430,34 +433,48 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
               for (int i = 0; i < 16; ++i) lora[j][i] += P.s * tmp[j][i];
           }
         });
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int cp = 8 * (i >> 2) + 4 * half + (i & 3);
+          *reinterpret_cast<uint32_t*>(lora_plane + (32 * ml + l32) * EP_STRIDE + 8 * cp + 2 * wave) = pack2<T>(lora[0][i], lora[1][i]);
+        }
       }
       // rounded pairs (tile 0, tile 1) = adjacent output columns -> one 4-byte LDS write
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int cp = 8 * (i >> 2) + 4 * half + (i & 3);
-        const int o = (32 * ml + l32) * EP_STRIDE + 8 * cp + 2 * wave;
-        *reinterpret_cast<uint32_t*>(base_plane + o) = pack2<T>(acc[mt][0][i], acc[mt][1][i]);
-        if (any_lora) *reinterpret_cast<uint32_t*>(lora_plane + o) = pack2<T>(lora[0][i], lora[1][i]);
+        *reinterpret_cast<uint32_t*>(base_plane + (32 * ml + l32) * EP_STRIDE + 8 * cp + 2 * wave) = pack2<T>(acc[mt][0][i], acc[mt][1][i]);
       }
     });
-    __syncthreads();
-      // coalesced pass: 64 rows x 32 chunks of 8 columns; iteration `it` handles row 8*it + tid/32
-    if (q + 1 < MT / 2) {
-      load_tf(std::integral_constant<int, (q + 1 < MT / 2) ? q + 1 : q>{});
-      issue_loads(std::integral_constant<int, (q + 1 < MT / 2) ? q + 1 : q>{});
+  };
+
+  load_tf(0);
+  static_for<0, SWEEP>([&](auto it_c) { issue_loads(0, it_c); });
+
+#pragma clang loop unroll(disable)
+  for (int q = 0; q < MT / 2; ++q) {
+    switch (q) {
+      case 0: dump(I0{}); break;
+      case 1: dump(I1{}); break;
+      case 2: dump(I2{}); break;
+      default: dump(I3{}); break;
     }
-#pragma unroll
-    for (int it = 0; it < EP_ROWS * 32 / 256; ++it) {
+    __syncthreads();
+    const bool more = q + 1 < MT / 2;
+    if (more) load_tf(q + 1);
+    // (b): iteration `it` handles row 8*it + tid/32 of the pass
+    static_for<0, SWEEP>([&](auto it_c) {
+      constexpr int it = decltype(it_c)::value;
       const int row = (tid >> 5) + 8 * it;
       const uint32_t soff_rows = (uint32_t)(EP_ROWS * q + 8 * it);
       const u32x4 bv = *reinterpret_cast<const u32x4*>(base_plane + row * EP_STRIDE + 8 * chunk);
       u32x4 lv = {0u, 0u, 0u, 0u};
       if (any_lora) lv = *reinterpret_cast<const u32x4*>(lora_plane + row * EP_STRIDE + 8 * chunk);
-      if (swiglu) {
-        const u32x4 ev = pre_a[q & 1][it];
-        const u32x4 gv = pre_b[q & 1][it];
-        u32x4 mv = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-        if (a.mask_src) mv = __builtin_amdgcn_raw_buffer_load_b128(mk_rsrc, mk_voff, soff_rows * mk_row_bytes, 0);
+      const u32x4 mv = pre_m[it];
+      if constexpr (swiglu) {
+        const u32x4 ev = pre_e[it];
+        const u32x4 gv = pre_g[it];
+        if (more) issue_loads(q + 1, it_c);
         u32x4 hv, dgv, dev;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
@@ -474,7 +491,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
             const float h = unpack1<T>(pack1<T>(f * g32));
             // LoRA part of dh is masked by (dropout(h) != 0): mask_src holds dropout(h) when a
             // dropout was applied, otherwise h itself (recomputed here) decides
-            const bool keep = a.mask_src ? (mbits != 0) : (h != 0.f);
+            const bool keep = has_mask ? (mbits != 0) : (h != 0.f);
             const float DW = unpack1<T>(pack1<T>(keep ? b32 + l32f : b32));
             hh[j] = h;
             dg[j] = DW * f;                                    // d_g ("df", UL/swiglu.py:77)
@@ -489,23 +506,22 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
         __builtin_amdgcn_raw_buffer_store_b128(dgv, e_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
         __builtin_amdgcn_raw_buffer_store_b128(dev, g_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
       } else {
+        if (more) issue_loads(q + 1, it_c);
         u32x4 ov = bv;
         if (any_lora) {
-          u32x4 mv = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-          if (a.mask_src) mv = pre_a[q & 1][it];
 #pragma unroll
           for (int w = 0; w < 4; ++w) {
-            // +-0 in the mask source count as zero
-            const float l0 = (mv[w] & 0x7fffu) ? unpack_lo<T>(lv[w]) : 0.f;
-            const float l1 = ((mv[w] >> 16) & 0x7fffu) ? unpack_hi<T>(lv[w]) : 0.f;
+            // +-0 in the mask source count as zero; without a mask source nothing is masked
+            const float l0 = (!has_mask || (mv[w] & 0x7fffu)) ? unpack_lo<T>(lv[w]) : 0.f;
+            const float l1 = (!has_mask || ((mv[w] >> 16) & 0x7fffu)) ? unpack_hi<T>(lv[w]) : 0.f;
             ov[w] = pack2<T>(unpack_lo<T>(bv[w]) + l0, unpack_hi<T>(bv[w]) + l1);
           }
         }
         __builtin_amdgcn_raw_buffer_store_b128(ov, dx_rsrc, dx_voff, soff_rows * dx_row_bytes, 0);
       }
-    }
+    });
     __syncthreads();
-  });
+  }
 }
 
 // nsz[g, n] = -fp32(scales[g, n]) * (z[g, n] + zero_offset): exact in fp32 (11-bit x 5-bit).
@@ -568,16 +584,22 @@ int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int m
   a.nbm = (M + BM - 1) / BM;
   a.nbk = (a.K + 255) / 256;
   dim3 grid(a.nbm * a.nbk), block(256);
-#define LAUNCH(TT)                                                                              \
-  do {                                                                                          \
-    if (ntail) hipLaunchKernelGGL((gptq_lora_bwd_dx_kernel<TT, true>), grid, block, 0, st, a);  \
-    else hipLaunchKernelGGL((gptq_lora_bwd_dx_kernel<TT, false>), grid, block, 0, st, a);       \
+#define LAUNCH_M(TT, MD)                                                                           \
+  do {                                                                                             \
+    if (ntail) hipLaunchKernelGGL((gptq_lora_bwd_dx_kernel<TT, true, MD>), grid, block, 0, st, a);  \
+    else hipLaunchKernelGGL((gptq_lora_bwd_dx_kernel<TT, false, MD>), grid, block, 0, st, a);       \
+  } while (0)
+#define LAUNCH(TT)                                           \
+  do {                                                       \
+    if (mode == FMSA_BWD_SWIGLU) LAUNCH_M(TT, FMSA_BWD_SWIGLU); \
+    else LAUNCH_M(TT, FMSA_BWD_LINEAR);                      \
   } while (0)
   if (act_dtype == FMSA_BF16)
     LAUNCH(bf16_t);
   else
     LAUNCH(f16_t);
 #undef LAUNCH
+#undef LAUNCH_M
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }
