@@ -475,32 +475,30 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
         const u32x4 ev = pre_e[it];
         const u32x4 gv = pre_g[it];
         if (more) issue_loads(q + 1, it_c);
+        // Two adjacent columns at a time: every rounding to the storage type is one packed
+        // conversion whose two halves are read back as fp32 (UL/swiglu.py:69-88 rounds f, h, DW and
+        // DW * g to the storage type; their products with fp32 factors are rounded once, on store).
         u32x4 hv, dgv, dev;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-          float hh[2], dg[2], de[2];
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            const float e32 = j ? unpack_hi<T>(ev[w]) : unpack_lo<T>(ev[w]);
-            const float g32 = j ? unpack_hi<T>(gv[w]) : unpack_lo<T>(gv[w]);
-            const float b32 = j ? unpack_hi<T>(bv[w]) : unpack_lo<T>(bv[w]);
-            const float l32f = j ? unpack_hi<T>(lv[w]) : unpack_lo<T>(lv[w]);
-            const uint32_t mbits = (j ? (mv[w] >> 16) : mv[w]) & 0x7fffu;
-            const float se = sigmoidf_(e32);
-            const float f = unpack1<T>(pack1<T>(se * e32));
-            const float h = unpack1<T>(pack1<T>(f * g32));
-            // LoRA part of dh is masked by (dropout(h) != 0): mask_src holds dropout(h) when a
-            // dropout was applied, otherwise h itself (recomputed here) decides
-            const bool keep = has_mask ? (mbits != 0) : (h != 0.f);
-            const float DW = unpack1<T>(pack1<T>(keep ? b32 + l32f : b32));
-            hh[j] = h;
-            dg[j] = DW * f;                                    // d_g ("df", UL/swiglu.py:77)
-            const float dgt = unpack1<T>(pack1<T>(DW * g32));  // dg = DW * g in storage dtype (:79)
-            de[j] = dgt * se * (1.0f + e32 * (1.0f - se));     // d_e (:81-83)
-          }
-          hv[w] = pack2<T>(hh[0], hh[1]);
-          dgv[w] = pack2<T>(dg[0], dg[1]);
-          dev[w] = pack2<T>(de[0], de[1]);
+          const float e0 = unpack_lo<T>(ev[w]), e1 = unpack_hi<T>(ev[w]);
+          const float g0 = unpack_lo<T>(gv[w]), g1 = unpack_hi<T>(gv[w]);
+          const float b0 = unpack_lo<T>(bv[w]), b1 = unpack_hi<T>(bv[w]);
+          const float se0 = sigmoidf_(e0), se1 = sigmoidf_(e1);
+          const uint32_t fp = pack2<T>(se0 * e0, se1 * e1);  // f = silu(e)
+          const float f0 = unpack_lo<T>(fp), f1 = unpack_hi<T>(fp);
+          const uint32_t hp = pack2<T>(f0 * g0, f1 * g1);  // h = f * g
+          // LoRA part of dh is masked by (dropout(h) != 0): mask_src holds dropout(h) when a
+          // dropout was applied, otherwise h itself (recomputed here) decides; +-0 count as zero
+          const uint32_t sel = has_mask ? mv[w] : hp;
+          const float s0 = b0 + unpack_lo<T>(lv[w]), s1 = b1 + unpack_hi<T>(lv[w]);
+          const uint32_t dwp = pack2<T>((sel & 0x7fffu) ? s0 : b0, (sel & 0x7fff0000u) ? s1 : b1);
+          const float DW0 = unpack_lo<T>(dwp), DW1 = unpack_hi<T>(dwp);
+          const uint32_t tp = pack2<T>(DW0 * g0, DW1 * g1);  // dg = DW * g in storage dtype (:79)
+          hv[w] = hp;
+          dgv[w] = pack2<T>(DW0 * f0, DW1 * f1);  // d_g ("df", :77)
+          dev[w] = pack2<T>(unpack_lo<T>(tp) * se0 * (1.0f + e0 * (1.0f - se0)),   // d_e (:81-83)
+                            unpack_hi<T>(tp) * se1 * (1.0f + e1 * (1.0f - se1)));
         }
         __builtin_amdgcn_raw_buffer_store_b128(hv, h_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
         __builtin_amdgcn_raw_buffer_store_b128(dgv, e_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
