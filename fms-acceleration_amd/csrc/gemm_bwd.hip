@@ -324,7 +324,8 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
   // buffer resources over the tile's rows, so rows past M and columns past K need no branches
   // (loads return zero, stores are dropped).  The operands the sweep of pass q+1 reads (e and g,
   // the mask source) are requested during the sweep of pass q, each into the registers the sweep
-  // has just consumed, so no load is ever waited for right after its issue.
+  // has just finished with, so no load is ever waited for right after its issue and no value
+  // has to be copied between registers (a copy would wait for its load) where the loop closes.
   __builtin_amdgcn_s_waitcnt(WAIT_VM0);  // the surplus direct loads of the last stage have landed
   __syncthreads();
   constexpr bool swiglu = MODE == FMSA_BWD_SWIGLU;
@@ -474,7 +475,6 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       if constexpr (swiglu) {
         const u32x4 ev = pre_e[it];
         const u32x4 gv = pre_g[it];
-        if (more) issue_loads(q + 1, it_c);
         // Two adjacent columns at a time: every rounding to the storage type is one packed
         // conversion whose two halves are read back as fp32 (UL/swiglu.py:69-88 rounds f, h, DW and
         // DW * g to the storage type; their products with fp32 factors are rounded once, on store).
@@ -504,7 +504,6 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
         __builtin_amdgcn_raw_buffer_store_b128(dgv, e_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
         __builtin_amdgcn_raw_buffer_store_b128(dev, g_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
       } else {
-        if (more) issue_loads(q + 1, it_c);
         u32x4 ov = bv;
         if (any_lora) {
 #pragma unroll
@@ -517,6 +516,9 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
         }
         __builtin_amdgcn_raw_buffer_store_b128(ov, dx_rsrc, dx_voff, soff_rows * dx_row_bytes, 0);
       }
+      // the operands of this chunk are dead now: the request for the next pass can reuse their registers
+      __builtin_amdgcn_sched_barrier(0);
+      if (more) issue_loads(q + 1, it_c);
     });
     __syncthreads();
   }
