@@ -67,7 +67,8 @@ def build(verbose: bool = False, extra_flags=()) -> str:
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         list(pool.map(compile_one, zip(SOURCES, objs)))
     tmp = LIB_PATH + ".tmp"
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs])
+    # --no-undefined: a kernel whose host stub was not emitted must fail the link, not the first call
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--no-undefined", "-o", tmp, *objs])
     os.replace(tmp, LIB_PATH)
     if verbose:
         print("built", LIB_PATH)
