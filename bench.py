@@ -308,6 +308,17 @@ def main():
         }
         result["kernels"] = {k: {"ms": v[0], "tflops": v[1] / v[0] / 1e9, "launches_per_step": v[2] / args.steps}
                              for k, v in kt.items()}
+    if not args.no_kernel_timing:
+        # spread of the step time: the K steps a third time with one event per step boundary
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+        marks[0].record()
+        for i in range(args.steps):
+            step()
+            marks[i + 1].record()
+        torch.cuda.synchronize()
+        per = sorted(a.elapsed_time(b) for a, b in zip(marks[:-1], marks[1:]))
+        q = lambda p: per[min(len(per) - 1, int(round(p * (len(per) - 1))))]  # noqa: E731
+        result["ms_per_step_quantiles"] = {"p10": q(0.1), "p50": q(0.5), "p90": q(0.9)}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.cpu_sample_tokens)
     print(json.dumps(result))

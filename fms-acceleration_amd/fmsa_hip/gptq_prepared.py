@@ -7,6 +7,7 @@ import torch
 
 import fmsa_hip
 
+
 class PreparedWeight:
     """The C-ABI view of one QuantLinear.  For an act-order g_idx the packed rows are re-ordered
     once (fmsa_gptq_permute_rows) so that the group of row k' is k' // group_size; `perm` then
@@ -46,7 +47,7 @@ class PreparedWeight:
 
 def prepare(qweight, scales, qzeros, g_idx, bits) -> PreparedWeight:
     key = (qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(), g_idx.data_ptr(), g_idx._version,
-           qweight._version, int(getattr(qzeros, "offset", 0) or 0))
+           qweight._version, scales._version, qzeros._version, int(getattr(qzeros, "offset", 0) or 0))
     cached = getattr(qweight, "_fmsa_prepared", None)
     if cached is None or cached[0] != key:
         cached = (key, PreparedWeight(qweight, scales, qzeros, g_idx, bits))
