@@ -6,7 +6,6 @@ exp2 / log2 (losses 2e-5 relative; gradients 1e-5 of the scale for fp32 logits, 
 of the largest reference entry."""
 import pytest
 import torch
-import torch.nn.functional as F
 
 from oracle import cross_entropy as oce
 from tests.helpers import randn
