@@ -35,6 +35,7 @@ from typing import Optional
 import torch
 
 import fmsa_hip
+from fmsa_hip.gptq_prepared import prepare as _prepare  # per-weight C-ABI view, cached on the qweight tensor
 
 
 # ----------------------------------------------------------------------------------------------
@@ -106,8 +107,6 @@ def get_lora_parameters(proj):
     dropout = proj.lora_dropout[active] if hasattr(proj, "lora_dropout") else None
     return qstate, bias, A, B, s, dropout
 
-
-from fmsa_hip.gptq_prepared import prepare as _prepare  # per-weight C-ABI view, cached on the qweight tensor
 
 
 # ----------------------------------------------------------------------------------------------
