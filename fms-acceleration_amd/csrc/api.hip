@@ -32,6 +32,7 @@ int launch_ce_bwd(void* logits, int64_t ld, const float* dloss, int64_t dloss_st
 int launch_ce_fused(void* logits, int64_t ld, const int64_t* labels, int M, int V, int dtype, int vec, int64_t ignore_index,
                     const float* scale, float smoothing, float* losses, hipStream_t st);
 int launch_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, hipStream_t st);
+int launch_nf4_prepare(const fmsa_nf4_weight* w, int32_t* qweight_out, float* block_scale_out, hipStream_t st);
 int launch_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype, hipStream_t st);
 int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, int M, int I, int64_t ld, int act_dtype,
                       hipStream_t st);
@@ -42,11 +43,20 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline bool is_act(int d) { return d == FMSA_BF16 || d == FMSA_F16; }
 
 int check_weight(const fmsa_gptq_weight* w, int group_multiple) {
-  if (!w->qweight || !w->scales || !w->qzeros) return FMSA_ERR_NULL;
+  if (w->format != FMSA_WEIGHT_AFFINE && w->format != FMSA_WEIGHT_CODEBOOK) return FMSA_ERR_SHAPE;
+  if (!w->qweight) return FMSA_ERR_NULL;
   if (w->K <= 0 || w->N <= 0 || w->group_size <= 0) return FMSA_ERR_SHAPE;
   if (w->K % 32 != 0 || w->N % 32 != 0) return FMSA_ERR_SHAPE;  // qlinear_tritonv2.py:57-60
-  if (w->zero_offset != 0 && w->zero_offset != 1) return FMSA_ERR_SHAPE;
-  if (!aligned16(w->qweight) || !aligned16(w->scales) || !aligned16(w->qzeros)) return FMSA_ERR_ALIGN;
+  if (w->format == FMSA_WEIGHT_CODEBOOK) {
+    if (!w->code || !w->block_scale) return FMSA_ERR_NULL;
+    if (w->K % w->group_size != 0) return FMSA_ERR_SHAPE;
+    if (w->g_idx) return FMSA_ERR_UNSUPPORTED;
+    if (!aligned16(w->qweight) || !aligned16(w->block_scale)) return FMSA_ERR_ALIGN;
+  } else {
+    if (!w->scales || !w->qzeros) return FMSA_ERR_NULL;
+    if (w->zero_offset != 0 && w->zero_offset != 1) return FMSA_ERR_SHAPE;
+    if (!aligned16(w->qweight) || !aligned16(w->scales) || !aligned16(w->qzeros)) return FMSA_ERR_ALIGN;
+  }
   if (group_multiple > 0) {
     // The fused kernels assume the group of row k is k / group_size: act-order weights must be
     // repacked with fmsa_gptq_permute_rows first.  The forward needs one group per 16-wide MFMA
@@ -82,7 +92,7 @@ const char* fmsa_strerror(int code) {
   }
 }
 
-int fmsa_abi_version(void) { return 2; }
+int fmsa_abi_version(void) { return 3; }
 
 int fmsa_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, void* stream) {
   if (!w || !out) return FMSA_ERR_NULL;
@@ -150,6 +160,7 @@ int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, in
   for (int p = 0; p < n_proj; ++p) {
     const fmsa_fwd_proj& s = projs[p];
     if (int rc = check_weight(&s.w, 16)) return rc;
+    if (s.w.format != projs[0].w.format) return FMSA_ERR_UNSUPPORTED;  // one kernel flavour per launch
     if (s.w.K != K) return FMSA_ERR_SHAPE;
     if (!s.Y) return FMSA_ERR_NULL;
     if (s.ldy < s.w.N) return FMSA_ERR_SHAPE;
@@ -183,11 +194,12 @@ int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mod
   for (int p = 0; p < n_proj; ++p) {
     const fmsa_bwd_proj& s = projs[p];
     if (int rc = check_weight(&s.w, 8)) return rc;
+    if (s.w.format != projs[0].w.format) return FMSA_ERR_UNSUPPORTED;  // one kernel flavour per launch
     if (s.w.group_size < 32) return FMSA_ERR_UNSUPPORTED;  // at most 8 groups per 256 output columns
     if (s.w.K != K) return FMSA_ERR_SHAPE;
-    if (!s.dY || !s.nsz) return FMSA_ERR_NULL;
+    if (!s.dY || (!s.nsz && s.w.format != FMSA_WEIGHT_CODEBOOK)) return FMSA_ERR_NULL;
     if (s.lddy < s.w.N) return FMSA_ERR_SHAPE;
-    if (!aligned16(s.nsz)) return FMSA_ERR_ALIGN;
+    if (s.nsz && !aligned16(s.nsz)) return FMSA_ERR_ALIGN;
     if (!aligned16(s.dY) || s.lddy % 8 != 0) return FMSA_ERR_ALIGN;
     if (int rc = check_rank(s.r)) return rc;
     if (s.r > 0) {
@@ -238,6 +250,7 @@ int fmsa_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h_out,
 int fmsa_gptq_make_nsz(const fmsa_gptq_weight* w, float* out, void* stream) {
   if (!w || !out) return FMSA_ERR_NULL;
   if (int rc = check_weight(w, 0)) return rc;
+  if (w->format != FMSA_WEIGHT_AFFINE) return FMSA_ERR_UNSUPPORTED;  // a code-book weight has no zero points
   if (!aligned16(out)) return FMSA_ERR_ALIGN;
   return launch_gptq_nsz(w, out, (hipStream_t)stream);
 }
@@ -259,6 +272,16 @@ int fmsa_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, void* s
   if (out_dtype != FMSA_F16 && out_dtype != FMSA_BF16 && out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
   if (!aligned16(out) || (reinterpret_cast<uintptr_t>(w->packed) & 7u)) return FMSA_ERR_ALIGN;
   return launch_nf4_dequant(w, out_dtype, out, (hipStream_t)stream);
+}
+
+int fmsa_nf4_prepare(const fmsa_nf4_weight* w, int32_t* qweight_out, float* block_scale_out, void* stream) {
+  if (!w || !qweight_out || !block_scale_out) return FMSA_ERR_NULL;
+  if (!w->packed || !w->absmax_q || !w->absmax2 || !w->code2) return FMSA_ERR_NULL;
+  if (w->N <= 0 || w->K <= 0 || w->blocksize <= 0 || w->blocksize2 <= 0) return FMSA_ERR_SHAPE;
+  if (w->K % 8 != 0 || w->blocksize % 8 != 0 || w->K % w->blocksize != 0) return FMSA_ERR_SHAPE;
+  if (w->K / 8 > 65535 || w->K / w->blocksize > 65535) return FMSA_ERR_UNSUPPORTED;  // grid.y
+  if (!aligned16(qweight_out) || !aligned16(block_scale_out) || (reinterpret_cast<uintptr_t>(w->packed) & 3u)) return FMSA_ERR_ALIGN;
+  return launch_nf4_prepare(w, qweight_out, block_scale_out, (hipStream_t)stream);
 }
 
 namespace {

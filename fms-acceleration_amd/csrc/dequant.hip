@@ -4,12 +4,15 @@
 #include "common.h"
 
 // W[k, n] for k = 8*k8 .. 8*k8+7, n = 8*n8 .. 8*n8+7 per thread.
-template <typename OutT, bool kF32>
+// CODEBOOK: W = code[q] * block_scale[k / group_size, n] (scales, qzeros, g_idx unused).
+template <typename OutT, bool kF32, bool CODEBOOK>
 __global__ __launch_bounds__(256) void gptq_dequant_kernel(const int32_t* __restrict__ qweight,
                                                            const uint16_t* __restrict__ scales,
                                                            const int32_t* __restrict__ qzeros,
                                                            const int32_t* __restrict__ g_idx, int K, int N,
                                                            int group_size, int n_groups, int zero_offset,
+                                                           const float* __restrict__ code,
+                                                           const float* __restrict__ block_scale,
                                                            void* __restrict__ out) {
   const int n8 = blockIdx.x * blockDim.x + threadIdx.x;
   const int k8 = blockIdx.y;
@@ -21,18 +24,24 @@ __global__ __launch_bounds__(256) void gptq_dequant_kernel(const int32_t* __rest
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int k = k8 * 8 + j;
-    int g = g_idx ? g_idx[k] : k / group_size;
-    if (g < 0) g += n_groups;  // UL/gptq/triton/kernels.py:88-91
-    const u32x4 sc = *reinterpret_cast<const u32x4*>(scales + (size_t)g * N + n0);
-    const uint32_t zw = (uint32_t)qzeros[(size_t)g * (N / 8) + n8];
     float v[8];
+    if constexpr (CODEBOOK) {
+      const float* bs = block_scale + (size_t)(k / group_size) * N + n0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t sbits = (i & 1) ? (sc[i >> 1] >> 16) : (sc[i >> 1] & 0xffffu);
-      const float sf = fp16_bits_to_f32((uint16_t)sbits);
-      const int q = (int)((qw[i] >> (4 * j)) & 0xF);
-      const int z = (int)((zw >> (4 * i)) & 0xF) + zero_offset;
-      v[i] = sf * (float)(q - z);  // exact in fp32
+      for (int i = 0; i < 8; ++i) v[i] = code[(qw[i] >> (4 * j)) & 0xF] * bs[i];
+    } else {
+      int g = g_idx ? g_idx[k] : k / group_size;
+      if (g < 0) g += n_groups;  // UL/gptq/triton/kernels.py:88-91
+      const u32x4 sc = *reinterpret_cast<const u32x4*>(scales + (size_t)g * N + n0);
+      const uint32_t zw = (uint32_t)qzeros[(size_t)g * (N / 8) + n8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t sbits = (i & 1) ? (sc[i >> 1] >> 16) : (sc[i >> 1] & 0xffffu);
+        const float sf = fp16_bits_to_f32((uint16_t)sbits);
+        const int q = (int)((qw[i] >> (4 * j)) & 0xF);
+        const int z = (int)((zw >> (4 * i)) & 0xF) + zero_offset;
+        v[i] = sf * (float)(q - z);  // exact in fp32
+      }
     }
     if constexpr (kF32) {
       f32x4* op = reinterpret_cast<f32x4*>(reinterpret_cast<float*>(out) + (size_t)k * N + n0);
@@ -51,13 +60,21 @@ int launch_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, hip
   const int n_groups = (w->K + w->group_size - 1) / w->group_size;
   dim3 block(64);
   dim3 grid((w->N / 8 + 63) / 64, w->K / 8);
-#define ARGS w->qweight, w->scales, w->qzeros, w->g_idx, w->K, w->N, w->group_size, n_groups, w->zero_offset, out
-  if (out_dtype == FMSA_F16)
-    hipLaunchKernelGGL((gptq_dequant_kernel<f16_t, false>), grid, block, 0, st, ARGS);
-  else if (out_dtype == FMSA_BF16)
-    hipLaunchKernelGGL((gptq_dequant_kernel<bf16_t, false>), grid, block, 0, st, ARGS);
+#define ARGS w->qweight, w->scales, w->qzeros, w->g_idx, w->K, w->N, w->group_size, n_groups, w->zero_offset, w->code, w->block_scale, out
+#define LAUNCH(CB)                                                                           \
+  do {                                                                                       \
+    if (out_dtype == FMSA_F16)                                                               \
+      hipLaunchKernelGGL((gptq_dequant_kernel<f16_t, false, CB>), grid, block, 0, st, ARGS);  \
+    else if (out_dtype == FMSA_BF16)                                                         \
+      hipLaunchKernelGGL((gptq_dequant_kernel<bf16_t, false, CB>), grid, block, 0, st, ARGS); \
+    else                                                                                     \
+      hipLaunchKernelGGL((gptq_dequant_kernel<float, true, CB>), grid, block, 0, st, ARGS);   \
+  } while (0)
+  if (w->format == FMSA_WEIGHT_CODEBOOK)
+    LAUNCH(true);
   else
-    hipLaunchKernelGGL((gptq_dequant_kernel<float, true>), grid, block, 0, st, ARGS);
+    LAUNCH(false);
+#undef LAUNCH
 #undef ARGS
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;

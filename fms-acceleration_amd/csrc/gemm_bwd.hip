@@ -41,7 +41,8 @@ constexpr int EP_STRIDE = 264;  // elements per staged row (256 + 8)
 struct BwdProjDev {
   const int32_t* qweight;
   const uint16_t* scales;
-  const float* nsz;  // [G, N] = -scale * (zero + zero_offset)
+  const float* nsz;  // [G, N] = -scale * (zero + zero_offset); code-book format: the block scales [G, N]
+  const float* code;  // code-book format: 16 entries
   const uint16_t* dY;
   int64_t lddy;
   const uint16_t* T;
@@ -66,7 +67,8 @@ struct BwdArgs {
 
 FMSA_DEVI BwdProjDev select_proj(const BwdArgs& a, int p) { return p == 0 ? a.p[0] : (p == 1 ? a.p[1] : a.p[2]); }
 
-template <typename T, bool NTAIL, int MODE>
+// CODEBOOK: W = code[q] * block_scale[group, n] instead of the affine scale * (q - zero).
+template <typename T, bool NTAIL, int MODE, bool CODEBOOK>
 __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) {
   // separate arrays per stage buffer: every access names its buffer statically, so the compiler
   // can tell fragment reads of one buffer from the direct loads in flight into the other
@@ -167,7 +169,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     const int tb_elem = (wave == 0) ? 2 : 4;  // bytes per table element
     const int tb_g = (wave == 0) ? (lane >> 3) : (4 * (wave - 1) + (lane >> 4));
     const int tb_col = (wave == 0) ? 8 * (lane & 7) : 4 * (lane & 15);  // first column of the lane's chunk
-    const __amdgpu_buffer_rsrc_t sc_rsrc = make_rsrc(P.scales, (size_t)n_groups * N * 2);
+    const __amdgpu_buffer_rsrc_t sc_rsrc = make_rsrc(P.scales, CODEBOOK ? 0 : (size_t)n_groups * N * 2);
     const __amdgpu_buffer_rsrc_t nz_rsrc = make_rsrc(P.nsz, (size_t)n_groups * N * 4);
     const __amdgpu_buffer_rsrc_t tb_rsrc = (wave == 0) ? sc_rsrc : nz_rsrc;
     const bool tb_live = (wave < 3) && (g0 + tb_g) < n_groups;
@@ -245,10 +247,63 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       wf[par][1][2] = pack2<T>(__builtin_fmaf(sfv[4], ubyte0(hi1), nzv[4]), __builtin_fmaf(sfv[5], ubyte1(hi1), nzv[5]));
       wf[par][1][3] = pack2<T>(__builtin_fmaf(sfv[6], ubyte2(hi1), nzv[6]), __builtin_fmaf(sfv[7], ubyte3(hi1), nzv[7]));
     };
+    // Code-book flavour of prep in two phases (see the forward kernel): (a) fragment reads, byte
+    // shuffles, address arithmetic and the 16 table gathers; (b) the multiplies by the block scales of
+    // the lane's 8 columns and the conversions.
+    const float lut = CODEBOOK ? P.code[lane & 15] : 0.f;
+    uint32_t gath[NT][8];
+    u32x4 bs_lo, bs_hi;  // block scales of the fragment's 8 columns
+    auto prep_a = [&](auto sb_c, auto t_c, auto par_c) {
+      constexpr int t = decltype(t_c)::value;
+      constexpr int par = decltype(par_c)::value;
+      const char* lq = wq_buf(sb_c);
+      const char* lt = tb_buf(sb_c);
+      const u32x4 q0 = *reinterpret_cast<const u32x4*>(lq + wq_r[t][0]);
+      const u32x4 q1 = *reinterpret_cast<const u32x4*>(lq + wq_r[t][1]);
+      bs_lo = *reinterpret_cast<const u32x4*>(lt + nz_r + t * 64);
+      bs_hi = *reinterpret_cast<const u32x4*>(lt + nz_r + t * 64 + 16);
+      const char* lr = dy_buf(sb_c) + dy_r[t];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2);
+      const uint32_t p01 = __builtin_amdgcn_perm(q0[1], q0[0], sel_pair);
+      const uint32_t p23 = __builtin_amdgcn_perm(q0[3], q0[2], sel_pair);
+      const uint32_t p45 = __builtin_amdgcn_perm(q1[1], q1[0], sel_pair);
+      const uint32_t p67 = __builtin_amdgcn_perm(q1[3], q1[2], sel_pair);
+      const uint32_t x0 = __builtin_amdgcn_perm(p23, p01, 0x05040100u);  // byte i: (tile 1 << 4 | tile 0) of column n + i
+      const uint32_t x1 = __builtin_amdgcn_perm(p67, p45, 0x05040100u);  // columns n + 4 .. n + 7
+      const uint32_t a0[2] = {opaque((x0 << 2) & 0x3C3C3C3Cu), opaque((x0 >> 2) & 0x3C3C3C3Cu)};  // [tile]: 4 * nibble
+      const uint32_t a1[2] = {opaque((x1 << 2) & 0x3C3C3C3Cu), opaque((x1 >> 2) & 0x3C3C3C3Cu)};
+      const int li = (int)__float_as_uint(lut);
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          gath[j][b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((a0[j] >> (8 * b)) & 0xffu), li);
+          gath[j][4 + b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((a1[j] >> (8 * b)) & 0xffu), li);
+        }
+    };
+    auto prep_b = [&](auto par_c) {
+      constexpr int par = decltype(par_c)::value;
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        wf[par][j][0] = pack2<T>(__uint_as_float(gath[j][0]) * __uint_as_float(bs_lo[0]), __uint_as_float(gath[j][1]) * __uint_as_float(bs_lo[1]));
+        wf[par][j][1] = pack2<T>(__uint_as_float(gath[j][2]) * __uint_as_float(bs_lo[2]), __uint_as_float(gath[j][3]) * __uint_as_float(bs_lo[3]));
+        wf[par][j][2] = pack2<T>(__uint_as_float(gath[j][4]) * __uint_as_float(bs_hi[0]), __uint_as_float(gath[j][5]) * __uint_as_float(bs_hi[1]));
+        wf[par][j][3] = pack2<T>(__uint_as_float(gath[j][6]) * __uint_as_float(bs_hi[2]), __uint_as_float(gath[j][7]) * __uint_as_float(bs_hi[3]));
+      }
+    };
     auto mfma_step = [&](auto par_c) {
       constexpr int par = decltype(par_c)::value;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[par][j], xf[par][mt], acc[mt][j]);
+    };
+    auto mfma_half = [&](auto par_c, auto h_c) {
+      constexpr int par = decltype(par_c)::value;
+      constexpr int h = decltype(h_c)::value;
+#pragma unroll
+      for (int mt = h * (MT / 2); mt < (h + 1) * (MT / 2); ++mt)
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[par][j], xf[par][mt], acc[mt][j]);
     };
@@ -267,6 +322,34 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       }
       __builtin_amdgcn_sched_barrier(0);
     };
+    // code-book halves: (a) 8 MFMAs with 12 fragment reads, 16 gathers (4 LDS-pipe instructions per
+    // MFMA, the reads first) and the ~30 shuffle / address instructions; (b) 8 MFMAs with the 24
+    // multiplies / conversions and, in the last step of a stage, the 11 direct loads
+    auto interleave_a = [&]() {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x080, 3, 0);
+        if (i >= 4) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto interleave_b = [&](auto with_vmem_c) {
+      constexpr bool with_vmem = decltype(with_vmem_c)::value;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+        if (with_vmem) {
+          if (i < 3)
+            __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+          else
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
     using WithVmem = std::integral_constant<bool, true>;
     using NoVmem = std::integral_constant<bool, false>;
 
@@ -275,24 +358,30 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     // makes all four waves' parts visible and closes the reads of buffer SB, so step 3 can issue
     // the loads of stage s+2 into it while preparing step 0 of stage s+1 from the other buffer.
     // The last two stages re-load the final stage (no branch); that data is never used.
+    auto step = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c) {
+      if constexpr (CODEBOOK) {
+        prep_a(nb_c, nt_c, nx_c);
+        mfma_half(cur_c, I0{});
+        interleave_a();
+        prep_b(nx_c);
+        mfma_half(cur_c, I1{});
+        interleave_b(vmem_c);
+      } else {
+        prep(nb_c, nt_c, nx_c);
+        mfma_step(cur_c);
+        interleave(vmem_c);
+      }
+    };
     auto stage = [&](int s, auto sb_c) {
       constexpr int SB = decltype(sb_c)::value;
       using S1 = std::integral_constant<int, SB ^ 1>;
-      prep(sb_c, I1{}, I1{});
-      mfma_step(I0{});
-      interleave(NoVmem{});
-      prep(sb_c, I2{}, I0{});
-      mfma_step(I1{});
-      interleave(NoVmem{});
-      prep(sb_c, I3{}, I1{});
-      mfma_step(I0{});
-      interleave(NoVmem{});
+      step(sb_c, I1{}, I1{}, I0{}, NoVmem{});
+      step(sb_c, I2{}, I0{}, I1{}, NoVmem{});
+      step(sb_c, I3{}, I1{}, I0{}, NoVmem{});
       __builtin_amdgcn_s_waitcnt(WAIT_VM0);
       __syncthreads();
       load_stage(min(s + 2, n_stages - 1), sb_c);
-      prep(S1{}, I0{}, I0{});
-      mfma_step(I1{});
-      interleave(WithVmem{});
+      step(S1{}, I0{}, I0{}, I1{}, WithVmem{});
     };
 
     __syncthreads();  // the previous projection's last LDS reads are done
@@ -300,7 +389,12 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     __builtin_amdgcn_s_waitcnt(WAIT_VM0);
     __syncthreads();
     load_stage(min(1, n_stages - 1), I1{});
-    prep(I0{}, I0{}, I0{});
+    if constexpr (CODEBOOK) {
+      prep_a(I0{}, I0{}, I0{});
+      prep_b(I0{});
+    } else {
+      prep(I0{}, I0{}, I0{});
+    }
 
     const int n_full = n_stages & ~1;
     int s = 0;
@@ -565,7 +659,8 @@ int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int m
     BwdProjDev& d = a.p[p];
     d.qweight = s.w.qweight;
     d.scales = s.w.scales;
-    d.nsz = s.nsz;
+    d.nsz = s.w.format == FMSA_WEIGHT_CODEBOOK ? s.w.block_scale : s.nsz;
+    d.code = s.w.code;
     d.dY = (const uint16_t*)s.dY;
     d.lddy = s.lddy;
     d.T = (const uint16_t*)s.T;
@@ -584,10 +679,16 @@ int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int m
   a.nbm = (M + BM - 1) / BM;
   a.nbk = (a.K + 255) / 256;
   dim3 grid(a.nbm * a.nbk), block(256);
-#define LAUNCH_M(TT, MD)                                                                           \
-  do {                                                                                             \
-    if (ntail) hipLaunchKernelGGL((gptq_lora_bwd_dx_kernel<TT, true, MD>), grid, block, 0, st, a);  \
-    else hipLaunchKernelGGL((gptq_lora_bwd_dx_kernel<TT, false, MD>), grid, block, 0, st, a);       \
+  const bool codebook = projs[0].w.format == FMSA_WEIGHT_CODEBOOK;  // api.hip: all projections of a launch share the format
+#define LAUNCH_C(TT, MD, CB)                                                                           \
+  do {                                                                                                 \
+    if (ntail) hipLaunchKernelGGL((gptq_lora_bwd_dx_kernel<TT, true, MD, CB>), grid, block, 0, st, a);  \
+    else hipLaunchKernelGGL((gptq_lora_bwd_dx_kernel<TT, false, MD, CB>), grid, block, 0, st, a);       \
+  } while (0)
+#define LAUNCH_M(TT, MD)                  \
+  do {                                    \
+    if (codebook) LAUNCH_C(TT, MD, true); \
+    else LAUNCH_C(TT, MD, false);         \
   } while (0)
 #define LAUNCH(TT)                                           \
   do {                                                       \
@@ -600,6 +701,7 @@ int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int m
     LAUNCH(f16_t);
 #undef LAUNCH
 #undef LAUNCH_M
+#undef LAUNCH_C
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }

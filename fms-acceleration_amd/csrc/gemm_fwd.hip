@@ -34,6 +34,8 @@ struct FwdProjDev {
   const int32_t* qweight;
   const uint16_t* scales;
   const int32_t* qzeros;
+  const float* code;         // code-book format only
+  const float* block_scale;  // code-book format only: fp32 [K / group_size, N]
   const uint16_t* U;
   int64_t ldu;
   const uint16_t* B;
@@ -59,7 +61,9 @@ struct FwdArgs {
 FMSA_DEVI FwdProjDev select_proj(const FwdArgs& a, int p) { return p == 0 ? a.p[0] : (p == 1 ? a.p[1] : a.p[2]); }
 
 // GPS = scale groups per 64-wide K stage: 1 for group_size % 64 == 0, 2 / 4 for group sizes 32 / 16.
-template <typename T, int GPS, bool KTAIL>
+// CODEBOOK: the nibbles index a 16-entry table and one fp32 scale per (group, column) multiplies the
+// entry (W = code[q] * block_scale); otherwise the affine GPTQ form W = scale * (q - zero).
+template <typename T, int GPS, bool KTAIL, bool CODEBOOK>
 __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // two separate arrays (not one 2-D array): every access names its buffer statically, which is
   // what lets the compiler see that fragment reads of one buffer do not depend on the direct loads
@@ -111,7 +115,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   const char* scbase[NT];
   const char* zbase[NT];
   int Np[NT], zshift[NT], gs[NT];
-  float zoff[NT];
+  float zoff[NT], lut[NT];  // lut: this lane's entry of the projection's code book (lanes 0..15 serve as the table)
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
     const FwdProjDev P = select_proj(a, pj[j]);
@@ -122,7 +126,8 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     Np[j] = __builtin_amdgcn_readfirstlane(P.N);
     gs[j] = __builtin_amdgcn_readfirstlane(P.group_size);
     qbase[j] = reinterpret_cast<const char*>(P.qweight);
-    scbase[j] = reinterpret_cast<const char*>(P.scales);
+    scbase[j] = CODEBOOK ? reinterpret_cast<const char*>(P.block_scale) : reinterpret_cast<const char*>(P.scales);
+    lut[j] = CODEBOOK ? P.code[lane & 15] : 0.f;
     zbase[j] = reinterpret_cast<const char*>(P.qzeros);
     zshift[j] = 4 * (col & 7);
     zoff[j] = (float)P.zero_offset;
@@ -170,10 +175,10 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     const int n_groups = (K + gs[j] - 1) / gs[j];
     n_groups_j[j] = n_groups;
     q_rsrc[j] = make_rsrc(qbase[j], (size_t)(K >> 3) * Np[j] * 4);
-    sc_rsrc[j] = make_rsrc(scbase[j], (size_t)n_groups * Np[j] * 2);
-    z_rsrc[j] = make_rsrc(zbase[j], (size_t)n_groups * (Np[j] >> 3) * 4);
+    sc_rsrc[j] = make_rsrc(scbase[j], (size_t)n_groups * Np[j] * (CODEBOOK ? 4 : 2));
+    z_rsrc[j] = make_rsrc(zbase[j], CODEBOOK ? 0 : (size_t)n_groups * (Np[j] >> 3) * 4);
     q_off[j] = (uint32_t)((half * Np[j] + col0[j] + l32) * 4);
-    sc_off[j] = (uint32_t)((col0[j] + l32) * 2);
+    sc_off[j] = (uint32_t)((col0[j] + l32) * (CODEBOOK ? 4 : 2));
     z_off[j] = (uint32_t)(((col0[j] + l32) >> 3) * 4);
     q_step_bytes[j] = (uint32_t)Np[j] * 8;    // two packed rows per 16-wide K step
     q_stage_bytes[j] = (uint32_t)Np[j] * 32;  // eight packed rows per stage
@@ -184,7 +189,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // stage ahead together with X.
   uint32_t qw[NBUF][NT][4];
   uint16_t sc_raw[NBUF][NT][GPS];
-  uint32_t zw_raw[NBUF][NT][GPS];
+  uint32_t zw_raw[NBUF][NT][GPS];  // code-book format: the fp32 block scale
   float sf[NT][GPS], sf16[NT][GPS], nsz[NT][GPS];
   // group index of the stage being loaded, advanced without a division when GPS == 1
   int g_ld[NT], k_in_g[NT];
@@ -226,8 +231,12 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
           gu = (ku < K ? ku : st * BK) / gs[j];
         }
         gu = __builtin_amdgcn_readfirstlane(gu);  // uniform; keeps the scalar offsets out of vector registers
-        sc_raw[SB][j][u] = __builtin_amdgcn_raw_buffer_load_b16(sc_rsrc[j], sc_off[j], (uint32_t)gu * Np[j] * 2, 0);
-        zw_raw[SB][j][u] = __builtin_amdgcn_raw_buffer_load_b32(z_rsrc[j], z_off[j], (uint32_t)gu * (Np[j] >> 3) * 4, 0);
+        if constexpr (CODEBOOK) {
+          zw_raw[SB][j][u] = __builtin_amdgcn_raw_buffer_load_b32(sc_rsrc[j], sc_off[j], (uint32_t)gu * Np[j] * 4, 0);
+        } else {
+          sc_raw[SB][j][u] = __builtin_amdgcn_raw_buffer_load_b16(sc_rsrc[j], sc_off[j], (uint32_t)gu * Np[j] * 2, 0);
+          zw_raw[SB][j][u] = __builtin_amdgcn_raw_buffer_load_b32(z_rsrc[j], z_off[j], (uint32_t)gu * (Np[j] >> 3) * 4, 0);
+        }
       }
       if constexpr (GPS == 1) {  // uniform scalar bookkeeping, no division
         k_in_g[j] += BK;
@@ -244,10 +253,14 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     for (int j = 0; j < NT; ++j) {
 #pragma unroll
       for (int u = 0; u < GPS; ++u) {
-        sf[j][u] = fp16_bits_to_f32(sc_raw[SB][j][u]);
-        sf16[j][u] = sf[j][u] * 0.0625f;
-        const float z = (float)((zw_raw[SB][j][u] >> zshift[j]) & 0xFu) + zoff[j];
-        nsz[j][u] = -sf[j][u] * z;  // exact: 11-bit x 5-bit
+        if constexpr (CODEBOOK) {
+          sf[j][u] = __uint_as_float(zw_raw[SB][j][u]);
+        } else {
+          sf[j][u] = fp16_bits_to_f32(sc_raw[SB][j][u]);
+          sf16[j][u] = sf[j][u] * 0.0625f;
+          const float z = (float)((zw_raw[SB][j][u] >> zshift[j]) & 0xFu) + zoff[j];
+          nsz[j][u] = -sf[j][u] * z;  // exact: 11-bit x 5-bit
+        }
       }
     }
   };
@@ -267,10 +280,53 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 #pragma unroll
     for (int j = 0; j < NT; ++j) wf[par][j] = dequant8<T>(qw[SB][j][t], sf[j][t * GPS / 4], sf16[j][t * GPS / 4], nsz[j][t * GPS / 4]);
   };
+  // Code-book flavour in two phases, so that a step's first 8 MFMAs cover the table gathers and its
+  // last 8 the arithmetic on what they returned.  Phase a: the 8 X fragments and the 16 gathers
+  // (ds_bpermute from the lane-resident table; element 2b / 2b+1 of a word in gath[j][b] / [4 + b]).
+  uint32_t gath[NT][8];
+  auto prefetch_a = [&](auto sb_c, auto t_c, auto par_c) {
+    constexpr int SB = decltype(sb_c)::value;
+    constexpr int t = decltype(t_c)::value;
+    constexpr int par = decltype(par_c)::value;
+    const char* lr = lds_buf(sb_c) + lds_r_off[t];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const uint32_t w = qw[SB][j][t];
+      const uint32_t e = opaque((w << 2) & 0x3C3C3C3Cu);  // byte b: 4 * nibble 2b (a lane's byte address)
+      const uint32_t o = opaque((w >> 2) & 0x3C3C3C3Cu);  // byte b: 4 * nibble 2b+1
+      const int li = (int)__float_as_uint(lut[j]);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        gath[j][b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((e >> (8 * b)) & 0xffu), li);
+        gath[j][4 + b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((o >> (8 * b)) & 0xffu), li);
+      }
+    }
+  };
+  // phase b: code * block scale in fp32, one rounding
+  auto prefetch_b = [&](auto t_c, auto par_c) {
+    constexpr int t = decltype(t_c)::value;
+    constexpr int par = decltype(par_c)::value;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const float sc = sf[j][t * GPS / 4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) wf[par][j][b] = pack2<T>(__uint_as_float(gath[j][b]) * sc, __uint_as_float(gath[j][4 + b]) * sc);
+    }
+  };
   auto mfma_step = [&](auto par_c) {
     constexpr int par = decltype(par_c)::value;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[par][j], xf[par][mt], acc[mt][j]);
+  };
+  auto mfma_half = [&](auto par_c, auto h_c) {
+    constexpr int par = decltype(par_c)::value;
+    constexpr int h = decltype(h_c)::value;
+#pragma unroll
+    for (int mt = h * (MT / 2); mt < (h + 1) * (MT / 2); ++mt)
 #pragma unroll
       for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[par][j], xf[par][mt], acc[mt][j]);
   };
@@ -294,6 +350,33 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);  // nothing from the next step (or the stage hand-over) moves up
   };
+  // code-book halves: (a) 8 MFMAs with the address arithmetic (3 VALU) and 3 LDS-pipe instructions
+  // each (8 fragment reads + 16 gathers); (b) 8 MFMAs with the 24 multiplies / conversions and, in the
+  // last step of a stage, the global loads of a later stage
+  auto interleave_a = [&]() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+      __builtin_amdgcn_sched_group_barrier(0x080, 3, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto interleave_b = [&](auto with_vmem_c) {
+    constexpr bool with_vmem = decltype(with_vmem_c)::value;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+      if (with_vmem) {
+        if (i < 2)
+          __builtin_amdgcn_sched_group_barrier(0x020, 3, 0);
+        else
+          __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
   using WithVmem = std::integral_constant<bool, true>;
   using NoVmem = std::integral_constant<bool, false>;
   using I0 = std::integral_constant<int, 0>;
@@ -308,25 +391,33 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // stage has just vacated.  The last two stages re-load the final stage (no branch); that data
   // is never read.
   constexpr int WAIT_VM0 = 0x0F70;  // s_waitcnt vmcnt(0) only
+  // one 16-wide K step: the MFMAs of parity `cur` while fragments and weights of (buffer nb, step nt)
+  // are produced into parity `nx`
+  auto step = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c) {
+    if constexpr (CODEBOOK) {
+      prefetch_a(nb_c, nt_c, nx_c);
+      mfma_half(cur_c, I0{});
+      interleave_a();
+      prefetch_b(nt_c, nx_c);
+      mfma_half(cur_c, I1{});
+      interleave_b(vmem_c);
+    } else {
+      prefetch(nb_c, nt_c, nx_c);
+      mfma_step(cur_c);
+      interleave(vmem_c);
+    }
+  };
   auto stage = [&](int s, auto sb_c) {
     constexpr int SB = decltype(sb_c)::value;
     using S1 = std::integral_constant<int, SB ^ 1>;
-    prefetch(sb_c, I1{}, I1{});
-    mfma_step(I0{});
-    interleave(NoVmem{});
-    prefetch(sb_c, I2{}, I0{});
-    mfma_step(I1{});
-    interleave(NoVmem{});
-    prefetch(sb_c, I3{}, I1{});
-    mfma_step(I0{});
-    interleave(NoVmem{});
+    step(sb_c, I1{}, I1{}, I0{}, NoVmem{});
+    step(sb_c, I2{}, I0{}, I1{}, NoVmem{});
+    step(sb_c, I3{}, I1{}, I0{}, NoVmem{});
     __builtin_amdgcn_s_waitcnt(WAIT_VM0);
     commit_stage(S1{});
     __syncthreads();
     load_stage(min(s + 2, n_stages - 1), sb_c);
-    prefetch(S1{}, I0{}, I0{});
-    mfma_step(I1{});
-    interleave(WithVmem{});
+    step(S1{}, I0{}, I0{}, I1{}, WithVmem{});
   };
 
   load_stage(0, I0{});
@@ -334,7 +425,12 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   commit_stage(I0{});
   __syncthreads();
   load_stage(min(1, n_stages - 1), I1{});
-  prefetch(I0{}, I0{}, I0{});
+  if constexpr (CODEBOOK) {
+    prefetch_a(I0{}, I0{}, I0{});
+    prefetch_b(I0{}, I0{});
+  } else {
+    prefetch(I0{}, I0{}, I0{});
+  }
 
   // whole pairs in a single-exit loop (slots 0, 1), then the odd stage
   const int n_full = n_stages & ~1;
@@ -531,6 +627,8 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
     d.qweight = s.w.qweight;
     d.scales = s.w.scales;
     d.qzeros = s.w.qzeros;
+    d.code = s.w.code;
+    d.block_scale = s.w.block_scale;
     d.U = (const uint16_t*)s.U;
     d.ldu = s.ldu;
     d.B = (const uint16_t*)s.B;
@@ -555,11 +653,17 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
     if (gsz % 64 != 0) gps = (gsz % 32 == 0) ? (gps > 2 ? gps : 2) : 4;
   }
   const bool ktail = (a.K % BK) != 0;
-#define LAUNCH2(TT, KT)                                                                          \
-  do {                                                                                           \
-    if (gps == 1) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, KT>), grid, block, 0, st, a);  \
-    else if (gps == 2) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 2, KT>), grid, block, 0, st, a); \
-    else hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 4, KT>), grid, block, 0, st, a);           \
+  const bool codebook = projs[0].w.format == FMSA_WEIGHT_CODEBOOK;  // api.hip: all projections of a launch share the format
+#define LAUNCH3(TT, KT, CB)                                                                          \
+  do {                                                                                               \
+    if (gps == 1) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, KT, CB>), grid, block, 0, st, a);  \
+    else if (gps == 2) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 2, KT, CB>), grid, block, 0, st, a); \
+    else hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 4, KT, CB>), grid, block, 0, st, a);           \
+  } while (0)
+#define LAUNCH2(TT, KT)          \
+  do {                           \
+    if (codebook) LAUNCH3(TT, KT, true); \
+    else LAUNCH3(TT, KT, false); \
   } while (0)
 #define LAUNCH(TT)            \
   do {                        \
@@ -572,6 +676,7 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
     LAUNCH(f16_t);
 #undef LAUNCH
 #undef LAUNCH2
+#undef LAUNCH3
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }

@@ -52,7 +52,55 @@ __global__ __launch_bounds__(256) void nf4_dequant_kernel(const uint8_t* __restr
   }
 }
 
+// Re-layout for the fused GEMM kernels.  One thread per output word: (k8, n) takes the four bytes
+// of row n that hold elements 8*k8 .. 8*k8+7 (even element in the high nibble) and writes them
+// with element j in bits 4j .. 4j+3; threads of a workgroup share k8 and walk n, so the stores are
+// coalesced (the 4-byte reads are strided by K/2 bytes: a one-time cost on a frozen weight).
+__global__ __launch_bounds__(256) void nf4_words_kernel(const uint8_t* __restrict__ packed, int N, int K,
+                                                        int32_t* __restrict__ qweight_out) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  const int k8 = blockIdx.y;
+  if (n >= N) return;
+  const uint32_t bytes = *reinterpret_cast<const uint32_t*>(packed + ((size_t)n * K + 8 * (size_t)k8) / 2);
+  uint32_t word = 0;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const uint32_t byte = (bytes >> (8 * b)) & 0xffu;
+    word |= (byte >> 4) << (8 * b);           // element 2b
+    word |= (byte & 0xFu) << (8 * b + 4);     // element 2b + 1
+  }
+  qweight_out[(size_t)k8 * N + n] = (int32_t)word;
+}
+
+// block_scale[kb, n] = absmax of block (n, kb), i.e. of flat block n * (K / blocksize) + kb
+__global__ __launch_bounds__(256) void nf4_block_scale_kernel(const uint8_t* __restrict__ absmax_q,
+                                                              const float* __restrict__ absmax2,
+                                                              const float* __restrict__ code2, float offset, int N,
+                                                              int blocks_per_row, int blocksize2,
+                                                              float* __restrict__ out) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  const int kb = blockIdx.y;
+  if (n >= N) return;
+  const uint32_t b = (uint32_t)n * (uint32_t)blocks_per_row + (uint32_t)kb;
+  float absmax;
+  {
+#pragma clang fp contract(off)
+    const float prod = code2[absmax_q[b]] * absmax2[b / blocksize2];
+    absmax = prod + offset;
+  }
+  out[(size_t)kb * N + n] = absmax;
+}
+
 }  // namespace
+
+int launch_nf4_prepare(const fmsa_nf4_weight* w, int32_t* qweight_out, float* block_scale_out, hipStream_t st) {
+  dim3 block(256);
+  hipLaunchKernelGGL(nf4_words_kernel, dim3((w->N + 255) / 256, w->K / 8), block, 0, st, w->packed, w->N, w->K, qweight_out);
+  hipLaunchKernelGGL(nf4_block_scale_kernel, dim3((w->N + 255) / 256, w->K / w->blocksize), block, 0, st, w->absmax_q, w->absmax2,
+                     w->code2, w->offset, w->N, w->K / w->blocksize, w->blocksize2, block_scale_out);
+  FMSA_CHECK_LAUNCH();
+  return FMSA_OK;
+}
 
 int launch_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, hipStream_t st) {
   const int64_t n = (int64_t)w->N * w->K;

@@ -1,0 +1,316 @@
+"""What the GPTQ- and the NF4-flavoured fused LoRA functions share: the per-projection operand
+bundle, adapter stacking, and the forward / backward bodies of LoRA_W, LoRA_QKV and LoRA_MLP on the
+libfmsa_hip kernels (reference: fused_ops/unsloth_lora/gptq/fast_lora.py:143-435, 466-711, 742-846
+and its bnb twin fused_ops/unsloth_lora/bnb/fast_lora.py).  The two flavours differ only in how a
+projection's frozen base weight is described to the kernels (`_Proj.w`, an affine GPTQ weight or a
+code-book weight) and in the argument lists of their autograd functions.
+
+  forward   U = Xd A^T                 (fmsa_lora_down, streams X once)
+            Y = X deq(W) + s U B^T     (fmsa_gptq_lora_fwd: nibble unpack in registers -> MFMA,
+                                        LoRA / bias / SwiGLU in the epilogue)
+  backward  T = dY B                   (fmsa_lora_down)
+            dA = s T^T Xd, dB = s dY^T U   (fmsa_lora_grad, deterministic)
+            dX = dY deq(W)^T + (Xd != 0) * T (s A)      (fmsa_gptq_lora_bwd_dx)
+"""
+from __future__ import annotations
+
+import torch
+
+import fmsa_hip
+
+
+# ----------------------------------------------------------------------------------------------
+# small helpers shared by the three functions
+# ----------------------------------------------------------------------------------------------
+def _act_dtype(X):
+    if X.dtype in (torch.float16, torch.bfloat16):
+        return X.dtype
+    if torch.is_autocast_enabled():
+        return torch.get_autocast_gpu_dtype()
+    raise TypeError(f"fused GPTQ-LoRA ops compute in float16 / bfloat16, got {X.dtype} outside autocast")
+
+
+def _as2d(X, dtype):
+    X2 = X.reshape(-1, X.shape[-1])
+    if X2.dtype != dtype:
+        X2 = X2.to(dtype)
+    return X2 if X2.is_contiguous() else X2.contiguous()
+
+
+def _apply_dropout(X2, dropout):
+    """Post-dropout input of the LoRA branch (matmul_lora :155-163).  Returns X2 itself when the
+    module is absent or an identity."""
+    if dropout is None or isinstance(dropout, torch.nn.Identity):
+        return X2
+    if isinstance(dropout, torch.Tensor):
+        return X2 * dropout.reshape(X2.shape).to(X2.dtype)
+    Xd = dropout(X2)
+    return Xd if Xd.is_contiguous() else Xd.contiguous()
+
+
+def _same(a, b):
+    """Same memory seen the same way (tensors that went through save_for_backward come back as new
+    objects)."""
+    return a is b or (a is not None and b is not None and a.data_ptr() == b.data_ptr()
+                      and a.shape == b.shape and a.stride() == b.stride())
+
+
+def _dropped_inputs(X2, projs, dropouts):
+    """Post-dropout input of each projection's LoRA branch; X2 itself (the same object) where no
+    dropout applies, which is what lets projections share passes over it."""
+    return [_apply_dropout(X2, d) if p.r else X2 for p, d in zip(projs, dropouts)]
+
+
+class _Proj:
+    """One projection's operands in the forms the kernels take."""
+
+    def __init__(self, w, bias, A, B, S, dtype):
+        self.w = w  # prepared weight: .struct (C-ABI view), .K, .N, .perm (act-order) and .nsz
+        self.bias = None if bias is None else bias.to(dtype)
+        self.A_param, self.B_param = A, B
+        self.r = 0 if A is None else A.shape[0]
+        self.s = 0.0 if S is None else float(S)
+        self.dtype = dtype
+        # activation-type copies of the adapter in the four layouts the kernels read (one launch,
+        # see pack): A [r, K], A^T [K, r], B [N, r], B^T [r, N]
+        self.A = self.At = self.B = self.Bt = None
+
+    def pack(self, A16_out=None):
+        if self.r:
+            self.A, self.At, self.B, self.Bt = fmsa_hip.lora_pack(self.A_param, self.B_param, self.dtype, A16_out)
+
+    # the kernels walk K in the repacked order for act-order weights
+    def to_kernel_order(self, X2):
+        return X2 if self.w.perm is None else fmsa_hip.permute_cols(X2, self.w.perm, gather=True)
+
+    def from_kernel_order(self, dXp):
+        return dXp if self.w.perm is None else fmsa_hip.permute_cols(dXp, self.w.perm, gather=False)
+
+    def fwd_dict(self, U):
+        return {"w": self.w.struct, "U": U, "B": self.B, "bias": self.bias, "r": self.r, "s": self.s}
+
+    def bwd_dict(self, dY2, T, mask_src):
+        At = None
+        if self.r:
+            At = self.At  # [K, r]
+            if self.w.perm is not None:
+                At = At[self.w.perm.long()].contiguous()
+                mask_src = None if mask_src is None else fmsa_hip.permute_cols(mask_src, self.w.perm, gather=True)
+        return {"w": self.w.struct, "nsz": self.w.nsz, "dY": dY2, "T": T, "At": At, "mask_src": mask_src if self.r else None,
+                "r": self.r, "s": self.s}
+
+    def lora_grads(self, T, Xd, U, dY2):
+        """dA [r, K] = s T^T Xd and dB [N, r] = s dY^T U, in the dtypes of the parameters."""
+        if not self.r:
+            return None, None
+        dA = fmsa_hip.lora_grad(T, Xd, self.s, False, self.A_param.dtype)
+        dB = fmsa_hip.lora_grad(U, dY2, self.s, True, self.B_param.dtype)
+        return dA, dB
+
+
+class _Stack:
+    """Adapters of projections that read the same (post-dropout) input, stacked: one pass over the
+    input gives all their U = Xd A^T (forward) and, with equal scalings, all their dA = s T^T Xd
+    (backward).  `cols[i]` is the column range of projection i inside the stacked [M, R] matrices."""
+
+    def __init__(self, projs, dtype, device):
+        self.R = sum(p.r for p in projs)
+        self.K = projs[0].w.K
+        self.A_cat = torch.empty((self.R, self.K), dtype=dtype, device=device)
+        self.cols, o = [], 0
+        for p in projs:
+            self.cols.append((o, o + p.r))
+            p.pack(self.A_cat[o : o + p.r])
+            o += p.r
+        self.same_s = all(p.s == projs[0].s for p in projs)
+
+
+def _pack_group(projs, Xds, dtype):
+    """Packs the adapters of a group of projections; returns a _Stack when they can share passes
+    over the input (all adapted, one post-dropout input, none act-order, total rank <= 128)."""
+    live = [p for p in projs if p.r]
+    if (len(live) == len(projs) and len(projs) > 1 and all(_same(Xd, Xds[0]) for Xd in Xds)
+            and all(p.w.perm is None for p in projs) and sum(p.r for p in projs) <= 128):
+        return _Stack(projs, dtype, Xds[0].device)
+    for p in projs:
+        p.pack()
+    return None
+
+
+def _lora_down_all(projs, Xds, stack):
+    if stack is not None:
+        U_cat = fmsa_hip.lora_down(Xds[0], stack.A_cat)
+        return [U_cat[:, a:b] for a, b in stack.cols]
+    return [fmsa_hip.lora_down(Xd, p.A) if p.r else None for p, Xd in zip(projs, Xds)]
+
+
+def _linear_forward(projs, X2, Xds, stack=None):
+    """Y_p = X deq(W_p) + s U_p B_p^T for projections sharing X2.  One launch when no weight is
+    act-order; otherwise one launch per projection on its own column-permuted copy of X."""
+    Us = _lora_down_all(projs, Xds, stack)
+    if all(p.w.perm is None for p in projs):
+        outs = fmsa_hip.gptq_lora_fwd(X2, [p.fwd_dict(U) for p, U in zip(projs, Us)])
+    else:
+        outs = [fmsa_hip.gptq_lora_fwd(p.to_kernel_order(X2), [p.fwd_dict(U)])[0] for p, U in zip(projs, Us)]
+    return outs, Us
+
+
+def _adapter_grads(projs, dYs, Xds, Us, stack):
+    """(Ts, [(dA, dB)]) of projections sharing their input.  T_p = dY_p B_p; dA_p = s T_p^T Xd;
+    dB_p = s dY_p^T U_p.  With a stack the T's are written side by side and one pass over Xd gives
+    every dA."""
+    if stack is not None:
+        M = dYs[0].shape[0]
+        T_cat = torch.empty((M, stack.R), dtype=dYs[0].dtype, device=dYs[0].device)
+        Ts = [fmsa_hip.lora_down(dY, p.Bt, out=T_cat[:, a:b]) for p, dY, (a, b) in zip(projs, dYs, stack.cols)]
+        grads = []
+        if stack.same_s and all(p.A_param.dtype == projs[0].A_param.dtype for p in projs):
+            dA_cat = fmsa_hip.lora_grad(T_cat, Xds[0], projs[0].s, False, projs[0].A_param.dtype)
+            dAs = [dA_cat[a:b] for a, b in stack.cols]
+        else:
+            dAs = [fmsa_hip.lora_grad(T, Xds[0], p.s, False, p.A_param.dtype) for p, T in zip(projs, Ts)]
+        for p, dY, U, dA in zip(projs, dYs, Us, dAs):
+            grads.append((dA, fmsa_hip.lora_grad(U, dY, p.s, True, p.B_param.dtype)))
+        return Ts, grads
+    Ts, grads = [], []
+    for p, dY, Xd, U in zip(projs, dYs, Xds, Us):
+        T = fmsa_hip.lora_down(dY, p.Bt) if p.r else None
+        Ts.append(T)
+        grads.append(p.lora_grads(T, Xd, U, dY))
+    return Ts, grads
+
+
+def _linear_backward_dx(projs, dYs, Ts, Xds, M, K):
+    """dX = sum_p dY_p deq(W_p)^T + mask (.) sum_p s_p T_p A_p.  One launch when the projections share
+    one mask source (no dropout, or one dropout module applied once) and none is act-order; otherwise
+    one launch per projection (each with its own mask / column order) and a sum."""
+    masks = [Xd for p, Xd in zip(projs, Xds) if p.r]
+    one_mask = all(_same(m, masks[0]) for m in masks)
+    if one_mask and all(p.w.perm is None for p in projs):
+        return fmsa_hip.gptq_lora_bwd_dx([p.bwd_dict(dY, T, Xd) for p, dY, T, Xd in zip(projs, dYs, Ts, Xds)], M, K)
+    dX = None
+    for p, dY, T, Xd in zip(projs, dYs, Ts, Xds):
+        part = p.from_kernel_order(fmsa_hip.gptq_lora_bwd_dx([p.bwd_dict(dY, T, Xd)], M, K))
+        dX = part.float() if dX is None else dX.add_(part)  # summed in fp32, rounded once
+    return dX.to(dYs[0].dtype) if len(projs) > 1 else part
+
+
+# ----------------------------------------------------------------------------------------------
+# bodies of the three autograd functions; `ctx` is the function's context object
+# ----------------------------------------------------------------------------------------------
+def w_forward(ctx, X, p, dropout, dtype):
+    X2 = _as2d(X, dtype)
+    p.pack()
+    Xd = _apply_dropout(X2, dropout) if p.r else X2
+    (Y,), (U,) = _linear_forward([p], X2, [Xd])
+    ctx.proj = p
+    ctx.act_dtype = dtype
+    ctx.x_shape, ctx.x_dtype = X.shape, X.dtype
+    ctx.save_for_backward(Xd, U) if p.r else ctx.save_for_backward()
+    return Y.view(*X.shape[:-1], p.w.N)
+
+
+def w_backward(ctx, dY):
+    """(dX, dA, dB)"""
+    p = ctx.proj
+    dY2 = _as2d(dY, ctx.act_dtype)
+    M, K = dY2.shape[0], p.w.K
+    dA = dB = None
+    T = Xd = None
+    if p.r:
+        Xd, U = ctx.saved_tensors
+        T = fmsa_hip.lora_down(dY2, p.Bt)
+        dA, dB = p.lora_grads(T, Xd, U, dY2)
+    dX = _linear_backward_dx([p], [dY2], [T], [Xd], M, K)
+    return dX.view(ctx.x_shape).to(ctx.x_dtype), dA, dB
+
+
+def qkv_forward(ctx, X, projs, dropouts, dtype):
+    X2 = _as2d(X, dtype)
+    Xds = _dropped_inputs(X2, projs, dropouts)
+    stack = _pack_group(projs, Xds, dtype)
+    outs, Us = _linear_forward(projs, X2, Xds, stack)
+    ctx.projs, ctx.stack = projs, stack
+    ctx.act_dtype = dtype
+    ctx.x_shape, ctx.x_dtype = X.shape, X.dtype
+    # tensors that may be None (disabled adapters) cannot go through save_for_backward as a
+    # fixed-length tuple; store how many were saved per projection
+    saved, ctx.layout = [], []
+    for Xd, U, p in zip(Xds, Us, projs):
+        ctx.layout.append(bool(p.r))
+        if p.r:
+            saved += [Xd, U]
+    ctx.save_for_backward(*saved)
+    return tuple(y.view(*X.shape[:-1], p.w.N) for y, p in zip(outs, projs))
+
+
+def qkv_backward(ctx, dQ, dK, dV):
+    """(dX, [(dA, dB)] * 3)"""
+    projs = ctx.projs
+    saved = list(ctx.saved_tensors)
+    K = projs[0].w.K
+    dYs = [_as2d(dY, ctx.act_dtype) for dY in (dQ, dK, dV)]  # dK may arrive non-contiguous (gptq/fast_lora.py:631)
+    Xds, Us = [], []
+    for has in ctx.layout:
+        Xds.append(saved.pop(0) if has else None)
+        Us.append(saved.pop(0) if has else None)
+    Ts, grads = _adapter_grads(projs, dYs, Xds, Us, ctx.stack)
+    M = dYs[0].shape[0]
+    dX = _linear_backward_dx(projs, dYs, Ts, Xds, M, K)
+    return dX.view(ctx.x_shape).to(ctx.x_dtype), grads
+
+
+def mlp_forward(ctx, X, gate, up, down, dropouts, dtype):
+    dropout_gate, dropout_up, dropout_down = dropouts
+    X2 = _as2d(X, dtype)
+    Xg, Xu = _dropped_inputs(X2, (gate, up), (dropout_gate, dropout_up))
+    stack = _pack_group([gate, up], [Xg, Xu], dtype)
+    down.pack()
+    fused = gate.w.perm is None and up.w.perm is None
+    if fused:
+        Ug, Uu = _lora_down_all([gate, up], [Xg, Xu], stack)
+        e, g, h = fmsa_hip.gptq_lora_fwd(X2, [gate.fwd_dict(Ug), up.fwd_dict(Uu)], fmsa_hip.FWD_SWIGLU)
+    else:
+        (e, g), (Ug, Uu) = _linear_forward([gate, up], X2, [Xg, Xu], stack)
+        h = fmsa_hip.swiglu_fwd(e, g)
+    hd = _apply_dropout(h, dropout_down) if down.r else h
+    (out,), (Ud,) = _linear_forward([down], h, [hd])
+    ctx.projs, ctx.stack = (gate, up, down), stack
+    ctx.x_shape, ctx.x_dtype = X.shape, X.dtype
+    ctx.down_dropped = hd is not h
+    none = X2.new_empty(0)
+    ctx.save_for_backward(Xg, Xu, e, g, hd if ctx.down_dropped else none,
+                          Ug if gate.r else none, Uu if up.r else none, Ud if down.r else none)
+    return out.view(*X.shape[:-1], down.w.N)
+
+
+def mlp_backward(ctx, dY):
+    """(dX, (dA_gate, dB_gate), (dA_up, dB_up), (dA_down, dB_down))"""
+    gate, up, down = ctx.projs
+    Xg, Xu, e, g, hd, Ug, Uu, Ud = ctx.saved_tensors
+    dY2 = _as2d(dY, e.dtype)
+    M, H, I = dY2.shape[0], gate.w.K, down.w.K
+
+    # ---- down projection: dh, then SwiGLU backward in place (e <- d_g, g <- d_e) -----------
+    Td = fmsa_hip.lora_down(dY2, down.Bt) if down.r else None
+    mask_h = hd if ctx.down_dropped else None
+    if down.w.perm is None:
+        h = fmsa_hip.gptq_lora_bwd_dx([down.bwd_dict(dY2, Td, mask_h)], M, I, fmsa_hip.BWD_SWIGLU, e=e, g=g)
+    else:
+        # un-fused epilogue for a repacked (act-order) weight: dh in kernel order, scatter back,
+        # then the standalone SwiGLU backward.  The mask of the LoRA part is (dropout(h) != 0).
+        h_now = fmsa_hip.swiglu_fwd(e, g)
+        dh = down.from_kernel_order(
+            fmsa_hip.gptq_lora_bwd_dx([down.bwd_dict(dY2, Td, mask_h if mask_h is not None else h_now)], M, I))
+        h = fmsa_hip.swiglu_bwd(dh, e, g)
+    d_g, d_e = e, g
+    dAd = dBd = None
+    if down.r:
+        # the reference forms both down-projection grads from the recomputed h (gptq/fast_lora.py:369-370)
+        Ud_b = fmsa_hip.lora_down(h, down.A) if ctx.down_dropped else Ud
+        dAd, dBd = down.lora_grads(Td, h, Ud_b, dY2)
+
+    # ---- up / gate: adapter grads, then dX over the concatenated contraction ---------------
+    (Tg, Tu), ((dAg, dBg), (dAu, dBu)) = _adapter_grads([gate, up], [d_e, d_g], [Xg, Xu], [Ug, Uu], ctx.stack)
+    dX = _linear_backward_dx([up, gate], [d_g, d_e], [Tu, Tg], [Xu, Xg], M, H)
+    return dX.view(ctx.x_shape).to(ctx.x_dtype), (dAg, dBg), (dAu, dBu), (dAd, dBd)

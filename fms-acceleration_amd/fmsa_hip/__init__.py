@@ -37,6 +37,7 @@ EXPORTED_SYMBOLS = (
     "fmsa_swiglu_bwd",
     "fmsa_gptq_make_nsz",
     "fmsa_nf4_dequant",
+    "fmsa_nf4_prepare",
     "fmsa_lora_pack",
     "fmsa_rms_layernorm_fwd",
     "fmsa_rms_layernorm_bwd",
@@ -57,7 +58,14 @@ class GptqWeight(Structure):
         ("N", c_int32),
         ("group_size", c_int32),
         ("zero_offset", c_int32),
+        ("format", c_int32),
+        ("reserved", c_int32),
+        ("code", c_void_p),
+        ("block_scale", c_void_p),
     ]
+
+
+WEIGHT_AFFINE, WEIGHT_CODEBOOK = 0, 1
 
 
 class Nf4Weight(Structure):
@@ -138,6 +146,7 @@ def lib() -> ctypes.CDLL:
     L.fmsa_swiglu_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
     L.fmsa_gptq_make_nsz.argtypes = [POINTER(GptqWeight), c_void_p, c_void_p]
     L.fmsa_nf4_dequant.argtypes = [POINTER(Nf4Weight), c_int, c_void_p, c_void_p]
+    L.fmsa_nf4_prepare.argtypes = [POINTER(Nf4Weight), c_void_p, c_void_p, c_void_p]
     L.fmsa_lora_pack.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p]
     L.fmsa_rms_layernorm_fwd.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p,
@@ -191,8 +200,26 @@ def make_weight(qweight, scales, qzeros, g_idx, group_size: int, zero_offset: in
     assert qweight.is_contiguous() and qzeros.is_contiguous() and scales.is_contiguous()
     return GptqWeight(
         qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
-        None if g_idx is None else g_idx.data_ptr(), K, N, int(group_size), int(zero_offset),
+        None if g_idx is None else g_idx.data_ptr(), K, N, int(group_size), int(zero_offset), WEIGHT_AFFINE, 0, None, None,
     )
+
+
+def make_codebook_weight(qweight, code, block_scale, group_size: int) -> GptqWeight:
+    """GptqWeight of a 4-bit code-book weight in the word layout (what nf4_prepare returns):
+    W[k, n] = code[q[k, n]] * block_scale[k // group_size, n]."""
+    K, N = qweight.shape[0] * 8, qweight.shape[1]
+    assert qweight.dtype == torch.int32 and code.dtype == torch.float32 and block_scale.dtype == torch.float32
+    assert qweight.is_contiguous() and code.is_contiguous() and block_scale.is_contiguous()
+    assert code.numel() == 16 and block_scale.shape == (K // group_size, N)
+    return GptqWeight(qweight.data_ptr(), None, None, None, K, N, int(group_size), 0, WEIGHT_CODEBOOK, 0,
+                      code.data_ptr(), block_scale.data_ptr())
+
+
+def weight_dequant(w: GptqWeight, device, out_dtype=torch.float16):
+    """Dense [K, N] of any GptqWeight (affine or code-book), one rounding to out_dtype."""
+    out = torch.empty((w.K, w.N), dtype=out_dtype, device=device)
+    _check("fmsa_gptq_dequant", lib().fmsa_gptq_dequant(ctypes.byref(w), _DTYPE_ENUM[out_dtype], _ptr(out), _stream(out)))
+    return out
 
 
 # ---- thin tensor-level wrappers ------------------------------------------------------------------
@@ -348,6 +375,18 @@ def nf4_dequant(packed, absmax_q, absmax2, code2, code, offset: float, shape, bl
     out = torch.empty((N, K), dtype=out_dtype, device=packed.device)
     _check("fmsa_nf4_dequant", lib().fmsa_nf4_dequant(ctypes.byref(w), _DTYPE_ENUM[out_dtype], _ptr(out), _stream(out)))
     return out
+
+
+def nf4_prepare(packed, absmax_q, absmax2, code2, offset: float, shape, blocksize: int, blocksize2: int):
+    """(qweight int32 [K/8, N], block_scale fp32 [K / blocksize, N]) of an NF4 tensor [N, K]: the
+    one-time re-layout the fused kernels read (see make_codebook_weight)."""
+    N, K = shape
+    w = Nf4Weight(packed.data_ptr(), absmax_q.data_ptr(), absmax2.data_ptr(), code2.data_ptr(), None, float(offset), N, K,
+                  blocksize, blocksize2)
+    qweight = torch.empty((K // 8, N), dtype=torch.int32, device=packed.device)
+    block_scale = torch.empty((K // blocksize, N), dtype=torch.float32, device=packed.device)
+    _check("fmsa_nf4_prepare", lib().fmsa_nf4_prepare(ctypes.byref(w), _ptr(qweight), _ptr(block_scale), _stream(qweight)))
+    return qweight, block_scale
 
 
 def lora_pack(A, B, act_dtype, A16_out=None):

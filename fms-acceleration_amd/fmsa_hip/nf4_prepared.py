@@ -1,0 +1,50 @@
+"""Per-weight preparation of a bitsandbytes NF4 tensor for the fused kernels, cached on the weight
+tensor: the codes re-laid into the word layout the GEMM kernels read and the double-quantised
+absmax expanded to one fp32 scale per (block, output column).  The base weight is frozen, so this
+happens once; `code[q] * block_scale` reproduces the library's dequantised values bit for bit."""
+from __future__ import annotations
+
+import torch
+
+import fmsa_hip
+
+
+class PreparedNf4Weight:
+    """The C-ABI view (`struct`, code-book format) of one NF4 linear of shape [N, K]."""
+
+    __slots__ = ("struct", "K", "N", "group_size", "perm", "nsz", "_keep")
+
+    def __init__(self, W, quant_state):
+        if isinstance(quant_state, list):
+            raise NotImplementedError("list-style (pre-0.42 bitsandbytes) quant states are not supported")
+        state2 = quant_state.state2
+        if state2 is None or quant_state.absmax.dtype != torch.uint8:
+            raise NotImplementedError("only double-quantised NF4 weights (compress_statistics=True) are supported")
+        data = W.data if isinstance(W, torch.nn.Parameter) else W
+        if not data.is_cuda:
+            raise RuntimeError("fused NF4-LoRA ops need the quantised weight on the GPU")
+        N, K = tuple(quant_state.shape)
+        bs = int(quant_state.blocksize)
+        if K % bs != 0 or bs % 32 != 0 or K % 32 != 0 or N % 32 != 0:
+            raise NotImplementedError(
+                f"the fused NF4 kernels need in_features % blocksize == 0, blocksize % 32 == 0 and both features "
+                f"divisible by 32 (got [{N}, {K}], blocksize {bs})")
+        qweight, block_scale = fmsa_hip.nf4_prepare(data.reshape(-1), quant_state.absmax, state2.absmax, state2.code,
+                                                    float(quant_state.offset), (N, K), bs, int(state2.blocksize))
+        code = quant_state.code.to(device=data.device, dtype=torch.float32).contiguous()
+        self.K, self.N, self.group_size = K, N, bs
+        self.perm = None  # no act-order for NF4
+        self.nsz = None   # the input-gradient kernel reads block_scale through the struct
+        self._keep = (qweight, block_scale, code)
+        self.struct = fmsa_hip.make_codebook_weight(qweight, code, block_scale, bs)
+
+
+def prepare(W, quant_state) -> PreparedNf4Weight:
+    data = W.data if isinstance(W, torch.nn.Parameter) else W
+    key = (data.data_ptr(), data._version, quant_state.absmax.data_ptr(), quant_state.absmax._version,
+           float(quant_state.offset), tuple(quant_state.shape), int(quant_state.blocksize))
+    cached = getattr(W, "_fmsa_prepared", None)
+    if cached is None or cached[0] != key:
+        cached = (key, PreparedNf4Weight(W, quant_state))
+        W._fmsa_prepared = cached
+    return cached[1]

@@ -55,7 +55,15 @@ int fmsa_abi_version(void);
  * W[k, n] = fp32(scales[g, n]) * (q[k, n] - (z[g, n] + zero_offset)),  g = g_idx[k]
  * zero_offset is 1 for checkpoints in the AutoGPTQ v1 zero-point format and 0 otherwise
  * (UL/gptq/fast_lora.py:100-101, UL/gptq/triton/kernels.py:113-116).
+ *
+ * format FMSA_WEIGHT_CODEBOOK describes a 4-bit code-book weight in the same word layout, which is
+ * what fmsa_nf4_prepare makes of a bitsandbytes NF4 tensor so that the fused kernels below can
+ * read it: nibble j of qweight[k8, n] indexes `code` (16 fp32 entries) and
+ *   W[k, n] = code[q[k, n]] * block_scale[k / group_size, n]      (fp32 product, one rounding)
+ * with block_scale fp32 [K / group_size, N]; scales, qzeros, g_idx and zero_offset are unused.
  * ------------------------------------------------------------------------------------------ */
+enum fmsa_weight_format { FMSA_WEIGHT_AFFINE = 0, FMSA_WEIGHT_CODEBOOK = 1 };
+
 typedef struct fmsa_gptq_weight {
   const int32_t* qweight;
   const uint16_t* scales;
@@ -65,6 +73,10 @@ typedef struct fmsa_gptq_weight {
   int32_t N;          /* out-features, N % 32 == 0                               */
   int32_t group_size; /* > 0; G = ceil(K / group_size)                           */
   int32_t zero_offset;
+  int32_t format;     /* enum fmsa_weight_format                                  */
+  int32_t reserved;   /* 0                                                        */
+  const float* code;        /* CODEBOOK: 16 entries                               */
+  const float* block_scale; /* CODEBOOK: [K / group_size, N]                      */
 } fmsa_gptq_weight;
 
 /* Replaces dequant248 (UL/gptq/triton/kernels.py:125-153): materialises W[K, N] row-major in
@@ -206,6 +218,15 @@ typedef struct fmsa_nf4_weight {
 } fmsa_nf4_weight;
 
 int fmsa_nf4_dequant(const fmsa_nf4_weight* w /*host*/, int out_dtype, void* out, void* stream);
+
+/* One-time re-layout of an NF4 weight for the fused kernels (the base weight is frozen): the codes
+ * of W[n, k] move into the word layout of fmsa_gptq_weight (qweight_out int32 [K/8, N], nibble j of
+ * word [k8, n] = code index of W[n, 8*k8 + j]) and the double-quantised absmax is expanded to
+ * block_scale_out fp32 [K / blocksize, N] with the arithmetic of fmsa_nf4_dequant, so that
+ * code[q] * block_scale reproduces its values bit for bit.  K % blocksize == 0, blocksize % 8 == 0,
+ * K % 8 == 0.  No counterpart in the reference, which always materialises the dense weight
+ * (UL/utils.py:250-283). */
+int fmsa_nf4_prepare(const fmsa_nf4_weight* w /*host*/, int32_t* qweight_out, float* block_scale_out, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * The two bandwidth-bound operators next to the q/k/v projections.  x_dtype / w_dtype / q_dtype /

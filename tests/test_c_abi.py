@@ -28,13 +28,43 @@ def test_header_and_library_agree():
 
 
 def test_struct_layouts_match_the_header():
-    assert ctypes.sizeof(fmsa_hip.GptqWeight) == 48
-    assert ctypes.sizeof(fmsa_hip.FwdProj) == 104
-    assert ctypes.sizeof(fmsa_hip.BwdProj) == 120
+    assert ctypes.sizeof(fmsa_hip.GptqWeight) == 72
+    assert ctypes.sizeof(fmsa_hip.FwdProj) == 128
+    assert ctypes.sizeof(fmsa_hip.BwdProj) == 144
 
 
 def _w(K=64, N=64, gs=64, q=0x1000, s=0x2000, z=0x3000, g=None, zo=0):
-    return fmsa_hip.GptqWeight(q, s, z, g, K, N, gs, zo)
+    return fmsa_hip.GptqWeight(q, s, z, g, K, N, gs, zo, fmsa_hip.WEIGHT_AFFINE, 0, None, None)
+
+
+def _cb(K=64, N=64, gs=64, q=0x1000, code=0x7000, bs=0x8000, g=None, fmt=None):
+    """A code-book weight (what fmsa_nf4_prepare produces)."""
+    return fmsa_hip.GptqWeight(q, None, None, g, K, N, gs, 0, fmsa_hip.WEIGHT_CODEBOOK if fmt is None else fmt, 0, code, bs)
+
+
+def test_codebook_weight_validation():
+    lib = fmsa_hip.lib()
+    f = lib.fmsa_gptq_dequant
+    assert f(ctypes.byref(_cb(code=None)), 0, 0x1000, None) == -1
+    assert f(ctypes.byref(_cb(bs=None)), 0, 0x1000, None) == -1
+    assert f(ctypes.byref(_cb(fmt=2)), 0, 0x1000, None) == -2        # unknown format
+    assert f(ctypes.byref(_cb(K=96, gs=64)), 0, 0x1000, None) == -2  # K % group_size
+    assert f(ctypes.byref(_cb(g=0x9000)), 0, 0x1000, None) == -5     # no act-order for a code book
+    assert f(ctypes.byref(_cb(bs=0x8004)), 0, 0x1000, None) == -3
+    assert lib.fmsa_gptq_make_nsz(ctypes.byref(_cb()), 0x1000, None) == -5  # no zero points to tabulate
+    # a launch takes projections of one format only
+    fw = lambda w: fmsa_hip.FwdProj(w, None, 0, None, None, 0x6000, 64, 0, 0.0)  # noqa: E731
+    arr = (fmsa_hip.FwdProj * 2)(fw(_w()), fw(_cb()))
+    assert lib.fmsa_gptq_lora_fwd(arr, 2, 0x9000, 64, 8, 0, None, 0, 1, None) == -5
+    p = lib.fmsa_nf4_prepare
+    nf4 = lambda **kw: fmsa_hip.Nf4Weight(*[kw.get(k, d) for k, d in (  # noqa: E731
+        ("packed", 0x1000), ("absmax_q", 0x2000), ("absmax2", 0x3000), ("code2", 0x4000), ("code", None), ("offset", 0.0),
+        ("N", 64), ("K", 128), ("blocksize", 64), ("blocksize2", 256))])
+    assert p(ctypes.byref(nf4()), None, 0x6000, None) == -1
+    assert p(ctypes.byref(nf4(absmax_q=None)), 0x5000, 0x6000, None) == -1
+    assert p(ctypes.byref(nf4(K=96)), 0x5000, 0x6000, None) == -2        # K % blocksize
+    assert p(ctypes.byref(nf4(blocksize=0)), 0x5000, 0x6000, None) == -2
+    assert p(ctypes.byref(nf4()), 0x5004, 0x6000, None) == -3
 
 
 def test_dequant_validation():

@@ -64,6 +64,12 @@ def test_nf4_dequant_bit_exact(gold):
                                  _dev(onf4.NF4), float(gold["nf4.offset"]), shape, int(gold["nf4.blocksize"]),
                                  int(gold["nf4.blocksize2"]), dtype)
         assert torch.equal(W.cpu(), _t16(gold[f"nf4.{name}"], dtype))
+    # the same values through the one-time re-layout the fused kernels read
+    qw, bs = fmsa_hip.nf4_prepare(_dev(gold["nf4.packed"]), _dev(gold["nf4.absmax_q"]), _dev(gold["nf4.absmax2"]), _dev(gold["nf4.code2"]),
+                                  float(gold["nf4.offset"]), shape, int(gold["nf4.blocksize"]), int(gold["nf4.blocksize2"]))
+    code = _dev(onf4.NF4)
+    Wt = fmsa_hip.weight_dequant(fmsa_hip.make_codebook_weight(qw, code, bs, int(gold["nf4.blocksize"])), qw.device, torch.bfloat16)
+    assert torch.equal(Wt.t().contiguous().cpu(), _t16(gold["nf4.W_bf16"]))
 
 
 def test_lora_w_vectors(gold):

@@ -1,5 +1,6 @@
-"""NF4 path: the dequantisation kernel bit-exact against the CPU oracle (whose own parity with
-bitsandbytes is unpinned: the library is absent and the reference holds no NF4 vectors), and the
+"""NF4 path: the dequantisation kernel and the one-time re-layout for the fused kernels bit-exact
+against the CPU oracle (whose own parity with bitsandbytes is unpinned: the library is absent and the
+reference holds no NF4 vectors), the code-book flavour of the fused GEMM kernels and the
 bitsandbytes-flavoured fused operators against the oracle's unfused graph."""
 import numpy as np
 import pytest
@@ -155,3 +156,57 @@ def test_lora_w_dropout_mask():
     assert olora.max_rel_err(xg.grad, dx_ref) < TOL
     assert olora.max_rel_err(lin.lora_A["default"].weight.grad, dA_ref) < TOL
     assert olora.max_rel_err(lin.lora_B["default"].weight.grad, dB_ref) < TOL
+
+
+def _prepared(N, K, seed, blocksize=64):
+    """(code-book GptqWeight struct, tensors kept alive, oracle quantisation dict) of a random [N, K] weight."""
+    import fmsa_hip
+
+    rng = np.random.default_rng(seed)
+    q = onf4.quantize((rng.standard_normal((N, K)) * rng.uniform(0.005, 0.05, size=(N, 1))).astype(np.float32), blocksize)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+    qw, bs = fmsa_hip.nf4_prepare(dev(q["packed"]), dev(q["absmax_q"]), dev(q["absmax2"]), dev(q["code2"]), float(q["offset"]),
+                                  (N, K), blocksize, 256)
+    code = dev(onf4.NF4)
+    return fmsa_hip.make_codebook_weight(qw, code, bs, blocksize), (qw, bs, code), q
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,K,blocksize", [(96, 512, 64), (32, 64, 64), (256, 4096, 64), (160, 1024, 128), (64, 256, 32)])
+def test_nf4_prepare_bit_exact(N, K, blocksize, dtype):
+    """code[q] * block_scale of the re-laid weight == the dequantisation kernel's (and the oracle's) values:
+    what the fused kernels feed the MFMA is the library's dense weight, bit for bit."""
+    import fmsa_hip
+
+    w, keep, q = _prepared(N, K, N + K, blocksize)
+    W = fmsa_hip.weight_dequant(w, torch.device("cuda"), dtype)  # [K, N]
+    assert torch.equal(W.cpu(), onf4.dequant(q, _NAME[dtype]).t().contiguous())
+    assert keep[0].shape == (K // 8, N) and keep[1].shape == (K // blocksize, N)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,N,r,blocksize", [(200, 256, 96, 16, 64), (512, 1024, 512, 8, 64), (64, 1056, 288, 32, 32), (300, 512, 256, 16, 128)])
+def test_codebook_kernels(M, K, N, r, blocksize, dtype):
+    """Forward (LoRA + bias) and input gradient (LoRA with a mask) of the code-book kernel flavour."""
+    import fmsa_hip
+
+    w, keep, q = _prepared(N, K, 3 * N + K, blocksize)
+    W = onf4.dequant(q, "fp32").t().contiguous()  # [K, N]
+    A, B = olora.make_lora(K, N, r, 5)
+    A16, B16 = A.to(dtype), B.to(dtype)
+    x = randn((M, K), 6, dtype)
+    x[::7, ::5] = 0  # masked entries of the LoRA part of dX
+    bias = randn((N,), 7, dtype, scale=0.1)
+    s = 2.0
+    xd = x.cuda()
+    U = fmsa_hip.lora_down(xd, A16.cuda())
+    (y,) = fmsa_hip.gptq_lora_fwd(xd, [{"w": w, "U": U, "B": B16.cuda(), "bias": bias.cuda(), "r": r, "s": s}])
+    y_ref = olora.lora_linear(x.float(), W, A16.float(), B16.float(), s, bias.float())
+    assert olora.max_rel_err(y.cpu(), y_ref) < TOL
+    dy = randn((M, N), 8, dtype)
+    dyd = dy.cuda()
+    T = fmsa_hip.lora_down(dyd, B16.t().contiguous().cuda())
+    dx = fmsa_hip.gptq_lora_bwd_dx([{"w": w, "nsz": None, "dY": dyd, "T": T, "At": A16.t().contiguous().cuda(), "mask_src": xd,
+                                     "r": r, "s": s}], M, K)
+    dx_ref, _, _ = olora.lora_w_manual(x.float(), W, A16.float(), B16.float(), s, dy.float())
+    assert olora.max_rel_err(dx.cpu(), dx_ref) < TOL
