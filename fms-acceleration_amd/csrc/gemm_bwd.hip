@@ -248,12 +248,13 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       wf[par][1][3] = pack2<T>(__builtin_fmaf(sfv[6], ubyte2(hi1), nzv[6]), __builtin_fmaf(sfv[7], ubyte3(hi1), nzv[7]));
     };
     // Code-book flavour of prep in two phases (see the forward kernel): (a) fragment reads, byte
-    // shuffles, address arithmetic and the 16 table gathers; (b) the multiplies by the block scales of
-    // the lane's 8 columns and the conversions.
+    // shuffles, address arithmetic and the 16 table gathers under the first 8 MFMAs of a step; (b) the
+    // multiplies by the block scales of the lane's 8 columns and the conversions under the last 8.
     const float lut = CODEBOOK ? P.code[lane & 15] : 0.f;
     uint32_t gath[NT][8];
     u32x4 bs_lo, bs_hi;  // block scales of the fragment's 8 columns
-    auto prep_a = [&](auto sb_c, auto t_c, auto par_c) {
+    // the same work without MFMAs in between, for the very first step of a projection
+    auto prep_first = [&](auto sb_c, auto t_c, auto par_c) {
       constexpr int t = decltype(t_c)::value;
       constexpr int par = decltype(par_c)::value;
       const char* lq = wq_buf(sb_c);
@@ -269,10 +270,10 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       const uint32_t p23 = __builtin_amdgcn_perm(q0[3], q0[2], sel_pair);
       const uint32_t p45 = __builtin_amdgcn_perm(q1[1], q1[0], sel_pair);
       const uint32_t p67 = __builtin_amdgcn_perm(q1[3], q1[2], sel_pair);
-      const uint32_t x0 = __builtin_amdgcn_perm(p23, p01, 0x05040100u);  // byte i: (tile 1 << 4 | tile 0) of column n + i
-      const uint32_t x1 = __builtin_amdgcn_perm(p67, p45, 0x05040100u);  // columns n + 4 .. n + 7
-      const uint32_t a0[2] = {opaque((x0 << 2) & 0x3C3C3C3Cu), opaque((x0 >> 2) & 0x3C3C3C3Cu)};  // [tile]: 4 * nibble
-      const uint32_t a1[2] = {opaque((x1 << 2) & 0x3C3C3C3Cu), opaque((x1 >> 2) & 0x3C3C3C3Cu)};
+      const uint32_t x0 = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+      const uint32_t x1 = __builtin_amdgcn_perm(p67, p45, 0x05040100u);
+      const uint32_t a0[2] = {(x0 << 2) & 0x3C3C3C3Cu, (x0 >> 2) & 0x3C3C3C3Cu};
+      const uint32_t a1[2] = {(x1 << 2) & 0x3C3C3C3Cu, (x1 >> 2) & 0x3C3C3C3Cu};
       const int li = (int)__float_as_uint(lut);
 #pragma unroll
       for (int j = 0; j < NT; ++j)
@@ -281,6 +282,60 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
           gath[j][b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((a0[j] >> (8 * b)) & 0xffu), li);
           gath[j][4 + b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((a1[j] >> (8 * b)) & 0xffu), li);
         }
+    };
+    // Phase a of step (sb, t) into parity `par`, written slot by slot under the first 8 MFMAs of the
+    // running step (parity `cur`): the order below IS the schedule (a fence closes every slot), because the
+    // dependency chain  word reads -> byte shuffles -> addresses -> gathers  has to be spread by hand.
+    auto phase_a = [&](auto sb_c, auto t_c, auto par_c, auto cur_c) {
+      constexpr int t = decltype(t_c)::value;
+      constexpr int par = decltype(par_c)::value;
+      constexpr int cur = decltype(cur_c)::value;
+      const char* lq = wq_buf(sb_c);
+      const char* lt = tb_buf(sb_c);
+      const char* lr = dy_buf(sb_c) + dy_r[t];
+      const int li = (int)__float_as_uint(lut);
+      auto mfma_slot = [&](int slot) { acc[slot >> 1][slot & 1] = mfma32<T>(wf[cur][slot & 1], xf[cur][slot >> 1], acc[slot >> 1][slot & 1]); };
+      auto frag = [&](int mt) { xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2); };
+      auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+      mfma_slot(0);
+      const u32x4 q0 = *reinterpret_cast<const u32x4*>(lq + wq_r[t][0]);
+      const u32x4 q1 = *reinterpret_cast<const u32x4*>(lq + wq_r[t][1]);
+      bs_lo = *reinterpret_cast<const u32x4*>(lt + nz_r + t * 64);
+      fence();
+      mfma_slot(1);
+      bs_hi = *reinterpret_cast<const u32x4*>(lt + nz_r + t * 64 + 16);
+      frag(0);
+      frag(1);
+      fence();
+      mfma_slot(2);
+      frag(2);
+      frag(3);
+      frag(4);
+      const uint32_t p01 = __builtin_amdgcn_perm(q0[1], q0[0], sel_pair);
+      const uint32_t p23 = __builtin_amdgcn_perm(q0[3], q0[2], sel_pair);
+      const uint32_t p45 = __builtin_amdgcn_perm(q1[1], q1[0], sel_pair);
+      const uint32_t p67 = __builtin_amdgcn_perm(q1[3], q1[2], sel_pair);
+      fence();
+      mfma_slot(3);
+      frag(5);
+      frag(6);
+      frag(7);
+      const uint32_t x0 = __builtin_amdgcn_perm(p23, p01, 0x05040100u);  // byte i: (tile 1 << 4 | tile 0) of column n + i
+      const uint32_t x1 = __builtin_amdgcn_perm(p67, p45, 0x05040100u);  // columns n + 4 .. n + 7
+      // [tile]: byte i = 4 * nibble = the byte address of the table's lane
+      const uint32_t a0[2] = {(x0 << 2) & 0x3C3C3C3Cu, (x0 >> 2) & 0x3C3C3C3Cu};
+      const uint32_t a1[2] = {(x1 << 2) & 0x3C3C3C3Cu, (x1 >> 2) & 0x3C3C3C3Cu};
+      fence();
+      // 4 gathers per MFMA: (tile j, columns 0-3 or 4-7)
+      static_for<0, 4>([&](auto u_c) {
+        constexpr int u = decltype(u_c)::value;
+        constexpr int j = u >> 1;
+        mfma_slot(4 + u);
+        const uint32_t a = (u & 1) ? a1[j] : a0[j];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) gath[j][4 * (u & 1) + b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((a >> (8 * b)) & 0xffu), li);
+        fence();
+      });
     };
     auto prep_b = [&](auto par_c) {
       constexpr int par = decltype(par_c)::value;
@@ -322,19 +377,8 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       }
       __builtin_amdgcn_sched_barrier(0);
     };
-    // code-book halves: (a) 8 MFMAs with 12 fragment reads, 16 gathers (4 LDS-pipe instructions per
-    // MFMA, the reads first) and the ~30 shuffle / address instructions; (b) 8 MFMAs with the 24
-    // multiplies / conversions and, in the last step of a stage, the 11 direct loads
-    auto interleave_a = [&]() {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x080, 3, 0);
-        if (i >= 4) __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    };
+    // code-book phase b: 8 MFMAs with the 24 multiplies / conversions and, in the last step of a stage, the
+    // 11 direct loads
     auto interleave_b = [&](auto with_vmem_c) {
       constexpr bool with_vmem = decltype(with_vmem_c)::value;
 #pragma unroll
@@ -360,9 +404,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     // The last two stages re-load the final stage (no branch); that data is never used.
     auto step = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c) {
       if constexpr (CODEBOOK) {
-        prep_a(nb_c, nt_c, nx_c);
-        mfma_half(cur_c, I0{});
-        interleave_a();
+        phase_a(nb_c, nt_c, nx_c, cur_c);
         prep_b(nx_c);
         mfma_half(cur_c, I1{});
         interleave_b(vmem_c);
@@ -390,7 +432,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     __syncthreads();
     load_stage(min(1, n_stages - 1), I1{});
     if constexpr (CODEBOOK) {
-      prep_a(I0{}, I0{}, I0{});
+      prep_first(I0{}, I0{}, I0{});
       prep_b(I0{});
     } else {
       prep(I0{}, I0{}, I0{});
