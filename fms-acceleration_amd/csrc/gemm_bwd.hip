@@ -182,28 +182,32 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     u32x4 xf[2][MT], wf[2][NT];
 
     // direct loads of stage `st` into buffer SB
-    auto load_stage = [&](int st, auto sb_c) {
+    // direct load number `idx` of stage `st` into buffer SB: 0-7 dY, 8-9 words, 10 tables
+    auto load_piece = [&](int st, auto sb_c, auto idx_c) {
+      constexpr int idx = decltype(idx_c)::value;
       const uint32_t n0 = (uint32_t)st * BK;
-      uint32_t dy_poison[2] = {0u, 0u}, wq_poison[2] = {0u, 0u}, tb_poison = 0u;
-      if constexpr (NTAIL) {  // N % 64 == 32: the upper half of the last stage lies past N
-        dy_poison[0] = ((int)n0 + 8 * dy_chunk_even < N) ? 0u : 0x80000000u;
-        dy_poison[1] = ((int)n0 + 8 * (dy_chunk_even ^ 4) < N) ? 0u : 0x80000000u;
-        wq_poison[0] = ((int)n0 + 4 * wq_chunk[0] < N) ? 0u : 0x80000000u;
-        wq_poison[1] = ((int)n0 + 4 * wq_chunk[1] < N) ? 0u : 0x80000000u;
-        tb_poison = ((int)n0 + tb_col < N) ? 0u : 0x80000000u;
-      }
-      char* ldy = dy_buf(sb_c) + wave * (64 * BK * 2);
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(dy_rsrc, (__attribute__((address_space(3))) void*)(ldy + i * (8 * BK * 2)), 16,
-                                                 dy_off[i] | dy_poison[i & 1], n0 * 2, 0, 0);
-      char* lwq = wq_buf(sb_c) + wave * 2048;
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
+      if constexpr (idx < 8) {
+        uint32_t poison = 0u;
+        if constexpr (NTAIL) poison = ((int)n0 + 8 * (dy_chunk_even ^ (4 * (idx & 1))) < N) ? 0u : 0x80000000u;
+        char* ldy = dy_buf(sb_c) + wave * (64 * BK * 2);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(dy_rsrc, (__attribute__((address_space(3))) void*)(ldy + idx * (8 * BK * 2)), 16,
+                                                 dy_off[idx] | poison, n0 * 2, 0, 0);
+      } else if constexpr (idx < 10) {
+        constexpr int i = idx - 8;
+        uint32_t poison = 0u;
+        if constexpr (NTAIL) poison = ((int)n0 + 4 * wq_chunk[i] < N) ? 0u : 0x80000000u;
+        char* lwq = wq_buf(sb_c) + wave * 2048;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(q_rsrc, (__attribute__((address_space(3))) void*)(lwq + i * 1024), 16,
-                                                 wq_off[i] | wq_poison[i], n0 * 4, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(tb_rsrc, (__attribute__((address_space(3))) void*)(tb_buf(sb_c) + wave * 1024), 16,
-                                               tb_off | tb_poison, n0 * (uint32_t)tb_elem, 0, 0);
+                                                 wq_off[i] | poison, n0 * 4, 0, 0);
+      } else {
+        uint32_t poison = 0u;
+        if constexpr (NTAIL) poison = ((int)n0 + tb_col < N) ? 0u : 0x80000000u;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(tb_rsrc, (__attribute__((address_space(3))) void*)(tb_buf(sb_c) + wave * 1024), 16,
+                                                 tb_off | poison, n0 * (uint32_t)tb_elem, 0, 0);
+      }
+    };
+    auto load_stage = [&](int st, auto sb_c) {
+      static_for<0, 11>([&](auto i_c) { load_piece(st, sb_c, i_c); });
     };
     // LDS -> registers for step t of buffer SB: the 8 dY fragments and the two unpacked weight
     // fragments, into parity `par`
@@ -402,28 +406,100 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     // makes all four waves' parts visible and closes the reads of buffer SB, so step 3 can issue
     // the loads of stage s+2 into it while preparing step 0 of stage s+1 from the other buffer.
     // The last two stages re-load the final stage (no branch); that data is never used.
-    auto step = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c) {
+    // The affine step written slot by slot: the 16 MFMAs of parity `cur`, each followed by its share of
+    // the work that produces step (nb, nt) into parity `nx` -- word / table / fragment reads first, the
+    // byte shuffles once the words are back, then one unpacked fragment register (2 conversions, 2
+    // multiply-adds, 1 packed conversion) per MFMA -- and, when `st_next` >= 0, one direct load of stage
+    // `st_next` into buffer `lb` per MFMA from the fifth on.  A scheduling fence closes every slot: the
+    // order below is the schedule.
+    auto step_affine = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c, int st_next, auto lb_c) {
+      constexpr int t = decltype(nt_c)::value;
+      constexpr int par = decltype(nx_c)::value;
+      constexpr int cur = decltype(cur_c)::value;
+      constexpr bool with_vmem = decltype(vmem_c)::value;
+      const char* lq = wq_buf(nb_c);
+      const char* lt = tb_buf(nb_c);
+      const char* lr = dy_buf(nb_c) + dy_r[t];
+      auto mfma_slot = [&](int slot) { acc[slot >> 1][slot & 1] = mfma32<T>(wf[cur][slot & 1], xf[cur][slot >> 1], acc[slot >> 1][slot & 1]); };
+      auto frag = [&](int mt) { xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2); };
+      auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+      mfma_slot(0);
+      const u32x4 q0 = *reinterpret_cast<const u32x4*>(lq + wq_r[t][0]);
+      const u32x4 q1 = *reinterpret_cast<const u32x4*>(lq + wq_r[t][1]);
+      const u32x4 sc = *reinterpret_cast<const u32x4*>(lt + sc_r + t * 32);
+      fence();
+      mfma_slot(1);
+      const u32x4 nz0 = *reinterpret_cast<const u32x4*>(lt + nz_r + t * 64);
+      const u32x4 nz1 = *reinterpret_cast<const u32x4*>(lt + nz_r + t * 64 + 16);
+      frag(0);
+      fence();
+      mfma_slot(2);
+      frag(1);
+      frag(2);
+      // this wave's byte of the 8 words: low nibble = column tile 0 (k = 8*k8 + 2*wave), high = tile 1
+      const uint32_t p01 = __builtin_amdgcn_perm(q0[1], q0[0], sel_pair);
+      const uint32_t p23 = __builtin_amdgcn_perm(q0[3], q0[2], sel_pair);
+      const uint32_t p45 = __builtin_amdgcn_perm(q1[1], q1[0], sel_pair);
+      const uint32_t p67 = __builtin_amdgcn_perm(q1[3], q1[2], sel_pair);
+      fence();
+      mfma_slot(3);
+      frag(3);
+      frag(4);
+      const uint32_t x0 = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+      const uint32_t x1 = __builtin_amdgcn_perm(p67, p45, 0x05040100u);
+      // nib[tile][half]: byte i = nibble of column n + 4*half + i
+      const uint32_t nib[2][2] = {{opaque(x0 & 0x0F0F0F0Fu), opaque(x1 & 0x0F0F0F0Fu)},
+                                  {opaque((x0 >> 4) & 0x0F0F0F0Fu), opaque((x1 >> 4) & 0x0F0F0F0Fu)}};
+      fence();
+      // fragment register `reg` of tile `j`: columns n + 2*reg, n + 2*reg + 1; value = scale * nibble + (-scale * zero)
+      auto piece = [&](auto j_c, auto reg_c) {
+        constexpr int j = decltype(j_c)::value;
+        constexpr int reg = decltype(reg_c)::value;
+        const uint32_t src = nib[j][reg >> 1];
+        const uint32_t sw = sc[reg];
+        const float s0 = fp16_bits_to_f32((uint16_t)(sw & 0xffffu)), s1 = fp16_bits_to_f32((uint16_t)(sw >> 16));
+        const u32x4& nz = (reg < 2) ? nz0 : nz1;
+        const float z0 = __uint_as_float(nz[2 * (reg & 1)]), z1 = __uint_as_float(nz[2 * (reg & 1) + 1]);
+        float b0, b1;
+        if constexpr ((reg & 1) == 0) {
+          b0 = ubyte0(src);
+          b1 = ubyte1(src);
+        } else {
+          b0 = ubyte2(src);
+          b1 = ubyte3(src);
+        }
+        wf[par][j][reg] = pack2<T>(__builtin_fmaf(s0, b0, z0), __builtin_fmaf(s1, b1, z1));
+      };
+      static_for<0, 12>([&](auto u_c) {
+        constexpr int u = decltype(u_c)::value;  // slots 4 .. 15
+        mfma_slot(4 + u);
+        if constexpr (u < 3) frag(5 + u);
+        if constexpr (u < 8) piece(std::integral_constant<int, (u >> 2)>{}, std::integral_constant<int, (u & 3)>{});
+        if constexpr (with_vmem && u < 11) load_piece(st_next, lb_c, u_c);
+        fence();
+      });
+    };
+    auto step = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c, int st_next, auto lb_c) {
       if constexpr (CODEBOOK) {
         phase_a(nb_c, nt_c, nx_c, cur_c);
         prep_b(nx_c);
         mfma_half(cur_c, I1{});
         interleave_b(vmem_c);
       } else {
-        prep(nb_c, nt_c, nx_c);
-        mfma_step(cur_c);
-        interleave(vmem_c);
+        step_affine(nb_c, nt_c, nx_c, cur_c, vmem_c, st_next, lb_c);
       }
     };
     auto stage = [&](int s, auto sb_c) {
       constexpr int SB = decltype(sb_c)::value;
       using S1 = std::integral_constant<int, SB ^ 1>;
-      step(sb_c, I1{}, I1{}, I0{}, NoVmem{});
-      step(sb_c, I2{}, I0{}, I1{}, NoVmem{});
-      step(sb_c, I3{}, I1{}, I0{}, NoVmem{});
+      step(sb_c, I1{}, I1{}, I0{}, NoVmem{}, 0, sb_c);
+      step(sb_c, I2{}, I0{}, I1{}, NoVmem{}, 0, sb_c);
+      step(sb_c, I3{}, I1{}, I0{}, NoVmem{}, 0, sb_c);
       __builtin_amdgcn_s_waitcnt(WAIT_VM0);
       __syncthreads();
-      load_stage(min(s + 2, n_stages - 1), sb_c);
-      step(S1{}, I0{}, I0{}, I1{}, WithVmem{});
+      const int st_next = min(s + 2, n_stages - 1);
+      if constexpr (CODEBOOK) load_stage(st_next, sb_c);  // spread under phase b by the group barriers
+      step(S1{}, I0{}, I0{}, I1{}, WithVmem{}, st_next, sb_c);
     };
 
     __syncthreads();  // the previous projection's last LDS reads are done
