@@ -109,23 +109,6 @@ template <> FMSA_DEVI f32x4 mfma16<f16_t>(u32x4 a, u32x4 b, f32x4 c) {
 }
 
 // ---- buffer resources ----------------------------------------------------------------------------
-// Code-book flavour of dequant8: the 8 nibbles of `w` index a 16-entry fp32 table that lives in the
-// wave itself -- `lut_lane` is this lane's entry code[lane & 15] and ds_bpermute fetches the entry
-// of lane q for every lane (a register-to-register gather through the LDS crossbar, no memory).
-// value = code[q] * scale in fp32, one rounding to the storage type.
-template <typename T> FMSA_DEVI u32x4 dequant8_code(uint32_t w, float scale, float lut_lane) {
-  const uint32_t e = opaque((w << 2) & 0x3C3C3C3Cu);  // byte b: 4 * nibble 2b   (a lane's byte address)
-  const uint32_t o = opaque((w >> 2) & 0x3C3C3C3Cu);  // byte b: 4 * nibble 2b+1
-  const int li = (int)__float_as_uint(lut_lane);
-  auto look = [&](uint32_t addr) { return __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute((int)addr, li)) * scale; };
-  u32x4 r;
-  r[0] = pack2<T>(look(e & 0xffu), look(o & 0xffu));
-  r[1] = pack2<T>(look((e >> 8) & 0xffu), look((o >> 8) & 0xffu));
-  r[2] = pack2<T>(look((e >> 16) & 0xffu), look((o >> 16) & 0xffu));
-  r[3] = pack2<T>(look(e >> 24), look(o >> 24));
-  return r;
-}
-
 // Raw buffer descriptor over [base, base + bytes): loads through it take a 32-bit per-lane offset
 // plus a scalar offset, and a lane offset at or past `bytes` returns zero instead of faulting.
 // The descriptor must live in scalar registers: base and size are wave-uniform by construction and
