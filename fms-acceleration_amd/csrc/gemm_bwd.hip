@@ -409,9 +409,10 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
     // The affine step written slot by slot: the 16 MFMAs of parity `cur`, each followed by its share of
     // the work that produces step (nb, nt) into parity `nx` -- word / table / fragment reads first, the
     // byte shuffles once the words are back, then one unpacked fragment register (2 conversions, 2
-    // multiply-adds, 1 packed conversion) per MFMA -- and, when `st_next` >= 0, one direct load of stage
-    // `st_next` into buffer `lb` per MFMA from the fifth on.  A scheduling fence closes every slot: the
-    // order below is the schedule.
+    // multiply-adds, 1 packed conversion) per MFMA -- and, in the last step of a stage, the 11 direct loads of
+    // stage `st_next` into buffer `lb`, placed where a slot has room (under the read slots, under every second
+    // unpack slot and under the last four MFMAs).  A scheduling fence closes every slot: the order below is
+    // the schedule.
     auto step_affine = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c, int st_next, auto lb_c) {
       constexpr int t = decltype(nt_c)::value;
       constexpr int par = decltype(nx_c)::value;
@@ -423,19 +424,25 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       auto mfma_slot = [&](int slot) { acc[slot >> 1][slot & 1] = mfma32<T>(wf[cur][slot & 1], xf[cur][slot >> 1], acc[slot >> 1][slot & 1]); };
       auto frag = [&](int mt) { xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2); };
       auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+      auto dma = [&](auto idx_c) {
+        if constexpr (with_vmem) load_piece(st_next, lb_c, idx_c);
+      };
       mfma_slot(0);
       const u32x4 q0 = *reinterpret_cast<const u32x4*>(lq + wq_r[t][0]);
       const u32x4 q1 = *reinterpret_cast<const u32x4*>(lq + wq_r[t][1]);
       const u32x4 sc = *reinterpret_cast<const u32x4*>(lt + sc_r + t * 32);
+      dma(std::integral_constant<int, 0>{});
       fence();
       mfma_slot(1);
       const u32x4 nz0 = *reinterpret_cast<const u32x4*>(lt + nz_r + t * 64);
       const u32x4 nz1 = *reinterpret_cast<const u32x4*>(lt + nz_r + t * 64 + 16);
       frag(0);
+      dma(std::integral_constant<int, 1>{});
       fence();
       mfma_slot(2);
       frag(1);
       frag(2);
+      dma(std::integral_constant<int, 2>{});
       // this wave's byte of the 8 words: low nibble = column tile 0 (k = 8*k8 + 2*wave), high = tile 1
       const uint32_t p01 = __builtin_amdgcn_perm(q0[1], q0[0], sel_pair);
       const uint32_t p23 = __builtin_amdgcn_perm(q0[3], q0[2], sel_pair);
@@ -445,6 +452,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
       mfma_slot(3);
       frag(3);
       frag(4);
+      dma(std::integral_constant<int, 3>{});
       const uint32_t x0 = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
       const uint32_t x1 = __builtin_amdgcn_perm(p67, p45, 0x05040100u);
       // nib[tile][half]: byte i = nibble of column n + 4*half + i
@@ -475,7 +483,8 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
         mfma_slot(4 + u);
         if constexpr (u < 3) frag(5 + u);
         if constexpr (u < 8) piece(std::integral_constant<int, (u >> 2)>{}, std::integral_constant<int, (u & 3)>{});
-        if constexpr (with_vmem && u < 11) load_piece(st_next, lb_c, u_c);
+        if constexpr (u >= 8) dma(std::integral_constant<int, u - 4>{});            // slots 12-15: loads 4-7
+        if constexpr (u == 0 || u == 2 || u == 4) dma(std::integral_constant<int, 8 + u / 2>{});  // loads 8-10
         fence();
       });
     };
