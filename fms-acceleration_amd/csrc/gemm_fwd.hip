@@ -420,6 +420,34 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     step(S1{}, I0{}, I0{}, I1{}, WithVmem{});
   };
 
+  // LoRA operands of ranks 0..15 (the whole adapter up to rank 16): direct loads into the epilogue planes,
+  // which are idle until the epilogue, issued here so that their latency is not exposed after the main loop.
+  // KB (8u + mt): rows 32mt..32mt+31 of U of the tile's u-th projection, 16 B per (row, rank half) at slot
+  // 2 * row + half.  KB (16 + NT * wave + j): the same for the wave's 32 rows of B of column tile j.
+  // Ranks past r and rows past M / N arrive as zeros through the range check.
+  char* const lora_lds = reinterpret_cast<char*>(ep_planes);
+  static_assert(sizeof(ep_planes) >= (16 + 4 * NT) * 1024, "LoRA operands must fit into the epilogue planes");
+  const bool lora_any = (a.p[0].r | a.p[1].r | a.p[2].r) != 0;
+  if (lora_any) {
+    const int prow = lane >> 1, phalf = lane & 1;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const FwdProjDev P = select_proj(a, pj[j]);
+      const int rp = __builtin_amdgcn_readfirstlane(P.r);
+      const uint32_t dead = (8 * phalf < rp) ? 0u : 0x80000000u;
+      if (j == 0 || a.mode == FMSA_FWD_SWIGLU) {  // linear mode: both column tiles belong to one projection
+        const __amdgpu_buffer_rsrc_t u_rs = make_rsrc(P.U + (size_t)m0 * P.ldu, rp > 0 ? (size_t)rows_valid * P.ldu * 2 : 0);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(
+              u_rs, (__attribute__((address_space(3))) void*)(lora_lds + (8 * j + 2 * uwave + i) * 1024), 16,
+              (uint32_t)(((64 * wave + 32 * i + prow) * P.ldu + 8 * phalf) * 2) | dead, 0, 0, 0);
+      }
+      const __amdgpu_buffer_rsrc_t b_rs = make_rsrc(P.B, rp > 0 ? (size_t)P.N * rp * 2 : 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rs, (__attribute__((address_space(3))) void*)(lora_lds + (16 + NT * uwave + j) * 1024),
+                                               16, (uint32_t)(((col0[j] + prow) * rp + 8 * phalf) * 2) | dead, 0, 0, 0);
+    }
+  }
   load_stage(0, I0{});
   __builtin_amdgcn_s_waitcnt(WAIT_VM0);
   commit_stage(I0{});
@@ -466,18 +494,26 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
       u_rsrc[j] = make_rsrc(P.U + (size_t)m0 * P.ldu, rj[j] > 0 ? (size_t)rows_valid * P.ldu * 2 : 0);
       r_max = max(r_max, rj[j]);
     }
+    const uint32_t slot = (uint32_t)(2 * l32 + half) * 16;
+    const int u_region = a.mode == FMSA_FWD_SWIGLU ? 8 : 0;  // KB between the U blocks of column tiles 0 and 1
     for (int j0 = 0; j0 < r_max; j0 += 16) {
       const int ko = j0 + 8 * half;
       u32x4 uf[NT][MT], bw[NT];
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        const bool live = ko < rj[j];
-        const uint32_t dead = live ? 0u : 0x80000000u;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          uf[j][mt] = __builtin_amdgcn_raw_buffer_load_b128(u_rsrc[j], (uint32_t)(((32 * mt + l32) * lduj[j] + ko) * 2) | dead, 0, 0);
         u32x4 bf = {0u, 0u, 0u, 0u};
-        if (live) bf = *reinterpret_cast<const u32x4*>(Bj[j] + (size_t)(col0[j] + l32) * rj[j] + ko);
+        if (j0 == 0) {  // staged in LDS before the main loop
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) uf[j][mt] = *reinterpret_cast<const u32x4*>(lora_lds + (u_region * j + mt) * 1024 + slot);
+          bf = *reinterpret_cast<const u32x4*>(lora_lds + (16 + NT * wave + j) * 1024 + slot);
+        } else {
+          const bool live = ko < rj[j];
+          const uint32_t dead = live ? 0u : 0x80000000u;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            uf[j][mt] = __builtin_amdgcn_raw_buffer_load_b128(u_rsrc[j], (uint32_t)(((32 * mt + l32) * lduj[j] + ko) * 2) | dead, 0, 0);
+          if (live) bf = *reinterpret_cast<const u32x4*>(Bj[j] + (size_t)(col0[j] + l32) * rj[j] + ko);
+        }
 #pragma unroll
         for (int w = 0; w < 4; ++w) bw[j][w] = pack2<T>(sj[j] * unpack_lo<T>(bf[w]), sj[j] * unpack_hi<T>(bf[w]));
       }
