@@ -9,8 +9,8 @@ int launch_permute_cols(const void* in, int64_t ld_in, const int32_t* perm, int 
 int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out, int64_t ldo,
                      hipStream_t st);
 int lora_grad_splits(int M, int C);
-int launch_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
-                     int act_dtype, int out_dtype, void* out, void* workspace, hipStream_t st);
+size_t lora_grad_batch_workspace(const fmsa_lora_grad_job* jobs, int n_jobs, int M);
+int launch_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int act_dtype, void* workspace, hipStream_t st);
 int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,
                          int64_t ldh, int act_dtype, hipStream_t st);
 int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx, void* e,
@@ -135,17 +135,35 @@ size_t fmsa_lora_grad_workspace(int M, int C, int r) {
   return (size_t)lora_grad_splits(M, C) * (size_t)r * (size_t)C * sizeof(float);
 }
 
+size_t fmsa_lora_grad_batch_workspace(const fmsa_lora_grad_job* jobs, int n_jobs, int M) {
+  if (!jobs || n_jobs < 1 || n_jobs > FMSA_LORA_GRAD_MAX_JOBS || M <= 0) return 0;
+  for (int q = 0; q < n_jobs; ++q)
+    if (jobs[q].C <= 0 || jobs[q].r <= 0) return 0;
+  return lora_grad_batch_workspace(jobs, n_jobs, M);
+}
+
+int fmsa_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int act_dtype, void* workspace,
+                         size_t workspace_bytes, void* stream) {
+  if (!jobs) return FMSA_ERR_NULL;
+  if (n_jobs < 1 || n_jobs > FMSA_LORA_GRAD_MAX_JOBS || M <= 0) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  for (int q = 0; q < n_jobs; ++q) {
+    const fmsa_lora_grad_job& j = jobs[q];
+    if (!j.L || !j.R || !j.out) return FMSA_ERR_NULL;
+    if (j.C <= 0 || j.r <= 0 || j.ldr < j.C || j.ldl < j.r) return FMSA_ERR_SHAPE;
+    if (j.C % 8 != 0 || j.ldr % 8 != 0 || j.ldl % 8 != 0 || j.r % 8 != 0 || j.r > 128) return FMSA_ERR_SHAPE;
+    if (j.out_dtype != FMSA_F16 && j.out_dtype != FMSA_BF16 && j.out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
+    if (!aligned16(j.R) || !aligned16(j.L)) return FMSA_ERR_ALIGN;
+  }
+  if (!workspace || workspace_bytes < lora_grad_batch_workspace(jobs, n_jobs, M)) return FMSA_ERR_WORKSPACE;
+  if (!aligned16(workspace)) return FMSA_ERR_ALIGN;
+  return launch_lora_grad_batch(jobs, n_jobs, M, act_dtype, workspace, (hipStream_t)stream);
+}
+
 int fmsa_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
                    int act_dtype, int out_dtype, void* out, void* workspace, size_t workspace_bytes, void* stream) {
-  if (!L || !R || !out) return FMSA_ERR_NULL;
-  if (M <= 0 || C <= 0 || r <= 0 || ldr < C || ldl < r) return FMSA_ERR_SHAPE;
-  if (C % 8 != 0 || ldr % 8 != 0 || ldl % 8 != 0 || r % 8 != 0 || r > 128) return FMSA_ERR_SHAPE;
-  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
-  if (out_dtype != FMSA_F16 && out_dtype != FMSA_BF16 && out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
-  if (!workspace || workspace_bytes < fmsa_lora_grad_workspace(M, C, r)) return FMSA_ERR_WORKSPACE;
-  if (!aligned16(R) || !aligned16(L) || !aligned16(workspace)) return FMSA_ERR_ALIGN;
-  return launch_lora_grad(L, ldl, R, ldr, M, C, r, scale, transpose_out, act_dtype, out_dtype, out, workspace,
-                          (hipStream_t)stream);
+  const fmsa_lora_grad_job job = {L, R, out, ldl, ldr, C, r, scale, transpose_out, out_dtype, 0};
+  return fmsa_lora_grad_batch(&job, 1, M, act_dtype, workspace, workspace_bytes, stream);
 }
 
 int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,

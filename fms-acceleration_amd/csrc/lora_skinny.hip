@@ -105,32 +105,77 @@ constexpr int LG_TM = 32;               // tokens per tile
 constexpr int LG_TC = 128;              // columns of R per workgroup
 constexpr int LG_RSTRIDE = LG_TC + 16;  // elements: 256 B + 32 B pad
 
+// Several gradients over the same M tokens go out as ONE launch of each pass (the dA of stacked
+// adapters and their dB's; a launch of a small gradient alone neither fills the chip nor hides its
+// own start-up): workgroup ids are laid end to end over the jobs.
+struct LoraGradJobDev {
+  const uint16_t* L;
+  const uint16_t* R;
+  void* out;
+  float* partial;  // [splits][r][C] of this job
+  int64_t ldl, ldr;
+  int C, r, splits, rows_per_split;
+  int block_start;   // first workgroup of the job in pass 1
+  int rblock_start;  // ... in pass 2
+  int transpose_out, out_dtype;
+  float scale;
+};
+struct LoraGradArgs {
+  LoraGradJobDev j[FMSA_LORA_GRAD_MAX_JOBS];
+  int n_jobs, M;
+};
+// the job that owns workgroup `block` (wave-uniform), copied field by field: indexing the
+// kernel-argument struct with a runtime value would force a copy of it into scratch memory
+template <bool REDUCE>
+FMSA_DEVI LoraGradJobDev select_job(const LoraGradArgs& a, int block) {
+  LoraGradJobDev J = a.j[0];
+#pragma unroll
+  for (int q = 1; q < FMSA_LORA_GRAD_MAX_JOBS; ++q)
+    if (q < a.n_jobs && block >= (REDUCE ? a.j[q].rblock_start : a.j[q].block_start)) J = a.j[q];
+  return J;
+}
+
 template <typename T, int RT>
-__global__ __launch_bounds__(256) void lora_grad_partial_kernel(const uint16_t* __restrict__ L, int64_t ldl,
-                                                                const uint16_t* __restrict__ R, int64_t ldr, int M,
-                                                                int C, int r, int rows_per_split,
-                                                                float* __restrict__ partial) {
+__global__ __launch_bounds__(256) void lora_grad_partial_kernel(const LoraGradArgs a) {
   constexpr int LSTRIDE = (RT == 1) ? 16 : RT * 16 + 16;  // elements; row pitch = 8 banks mod 32
   __shared__ __attribute__((aligned(16))) uint16_t r_lds[2][LG_TM * LG_RSTRIDE];
   __shared__ __attribute__((aligned(16))) uint16_t l_lds[2][LG_TM * LSTRIDE];
+  const LoraGradJobDev J = select_job<false>(a, blockIdx.x);
+  const uint16_t* __restrict__ L = J.L;
+  const uint16_t* __restrict__ R = J.R;
+  float* __restrict__ partial = J.partial;
+  const int64_t ldl = J.ldl, ldr = J.ldr;
+  const int M = a.M, C = J.C, r = J.r, rows_per_split = J.rows_per_split;
+  const int rt = (r + 15) / 16;  // 16-rank tiles this job uses of the RT the launch is built for
+  const int ncb = (C + LG_TC - 1) / LG_TC;
+  const int local = blockIdx.x - J.block_start;
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int l16 = lane & 15, kg = lane >> 4;
-  const int split = blockIdx.y;
-  const int c0 = blockIdx.x * LG_TC;
+  const int split = local / ncb;
+  const int c0 = (local % ncb) * LG_TC;
   const int m_begin = split * rows_per_split;
   const int m_end = min(M, m_begin + rows_per_split);
   const int n_tiles = (m_end - m_begin + LG_TM - 1) / LG_TM;
 
   // global -> LDS assignment: R tile = 32 rows x 16 chunks of 16 B -> 2 chunks per thread;
-  // L tile = 32 rows x (RT*2) chunks -> threads 0 .. 64*RT-1, one chunk each
+  // L tile = 32 rows x (RT*2) chunks = 64*RT chunks -> LP per thread (chunk tid + 256*p), threads
+  // past the last chunk idle
   const int r_row = tid >> 4, r_chunk = tid & 15;
   const bool r_col_ok = (c0 + 8 * r_chunk) < C;  // C % 8 == 0
-  const int l_row = tid / (2 * RT), l_chunk = tid % (2 * RT);
-  const bool l_thread = tid < 64 * RT;
-  const bool l_col_ok = 8 * l_chunk < r;  // r % 8 == 0
+  constexpr int LP = (64 * RT + 255) / 256;
+  int l_row[LP], l_chunk[LP];
+  bool l_thread[LP], l_col_ok[LP];
+#pragma unroll
+  for (int p = 0; p < LP; ++p) {
+    const int ci = tid + 256 * p;
+    l_row[p] = ci / (2 * RT);
+    l_chunk[p] = ci % (2 * RT);
+    l_thread[p] = ci < 64 * RT;
+    l_col_ok[p] = 8 * l_chunk[p] < r;  // r % 8 == 0
+  }
 
-  u32x4 rst[2], lst;
+  u32x4 rst[2], lst[LP];
   auto load_tile = [&](int tile) {
     const int m0 = m_begin + tile * LG_TM;
 #pragma unroll
@@ -139,17 +184,20 @@ __global__ __launch_bounds__(256) void lora_grad_partial_kernel(const uint16_t* 
       rst[p] = u32x4{0u, 0u, 0u, 0u};
       if (m < m_end && r_col_ok) rst[p] = *reinterpret_cast<const u32x4*>(R + (size_t)m * ldr + c0 + 8 * r_chunk);
     }
-    lst = u32x4{0u, 0u, 0u, 0u};
-    if (l_thread) {
-      const int m = m0 + l_row;
-      if (m < m_end && l_col_ok) lst = *reinterpret_cast<const u32x4*>(L + (size_t)m * ldl + 8 * l_chunk);
+#pragma unroll
+    for (int p = 0; p < LP; ++p) {
+      lst[p] = u32x4{0u, 0u, 0u, 0u};
+      const int m = m0 + l_row[p];
+      if (l_thread[p] && m < m_end && l_col_ok[p]) lst[p] = *reinterpret_cast<const u32x4*>(L + (size_t)m * ldl + 8 * l_chunk[p]);
     }
   };
   auto commit_tile = [&](int buf) {
 #pragma unroll
     for (int p = 0; p < 2; ++p)
       *reinterpret_cast<u32x4*>(&r_lds[buf][(r_row + 16 * p) * LG_RSTRIDE + 8 * r_chunk]) = rst[p];
-    if (l_thread) *reinterpret_cast<u32x4*>(&l_lds[buf][l_row * LSTRIDE + 8 * l_chunk]) = lst;
+#pragma unroll
+    for (int p = 0; p < LP; ++p)
+      if (l_thread[p]) *reinterpret_cast<u32x4*>(&l_lds[buf][l_row[p] * LSTRIDE + 8 * l_chunk[p]]) = lst[p];
   };
   // 8 contraction elements of column `col`: tokens 4*e + kg, e = 0..7
   auto column_frag = [&](const uint16_t* base, int stride, int col) {
@@ -179,13 +227,16 @@ __global__ __launch_bounds__(256) void lora_grad_partial_kernel(const uint16_t* 
     if (tile + 1 < n_tiles) load_tile(tile + 1);
     u32x4 lf[RT], rf[2];
 #pragma unroll
-    for (int t = 0; t < RT; ++t) lf[t] = column_frag(l_lds[buf], LSTRIDE, 16 * t + l16);
+    for (int t = 0; t < RT; ++t)
+      if (t < rt) lf[t] = column_frag(l_lds[buf], LSTRIDE, 16 * t + l16);
 #pragma unroll
     for (int g = 0; g < 2; ++g) rf[g] = column_frag(r_lds[buf], LG_RSTRIDE, 32 * wave + 16 * g + l16);
 #pragma unroll
-    for (int g = 0; g < 2; ++g)
+    for (int t = 0; t < RT; ++t)
+      if (t < rt) {
 #pragma unroll
-      for (int t = 0; t < RT; ++t) acc[g][t] = mfma16<T>(rf[g], lf[t], acc[g][t]);  // D[c][j]
+        for (int g = 0; g < 2; ++g) acc[g][t] = mfma16<T>(rf[g], lf[t], acc[g][t]);  // D[c][j]
+      }
     if (tile + 1 < n_tiles) commit_tile(buf ^ 1);
     __syncthreads();
   }
@@ -209,21 +260,20 @@ __global__ __launch_bounds__(256) void lora_grad_partial_kernel(const uint16_t* 
   }
 }
 
-template <typename OutT, bool kF32>
-__global__ __launch_bounds__(256) void lora_grad_reduce_kernel(const float* __restrict__ partial, int splits, int r,
-                                                               int C, float scale, int transpose_out,
-                                                               void* __restrict__ out) {
-  const int idx = blockIdx.x * blockDim.x + threadIdx.x;  // over r*C, c fastest
+__global__ __launch_bounds__(256) void lora_grad_reduce_kernel(const LoraGradArgs a) {
+  const LoraGradJobDev J = select_job<true>(a, blockIdx.x);
+  const int r = J.r, C = J.C;
+  const int idx = (blockIdx.x - J.rblock_start) * 256 + threadIdx.x;  // over r*C, c fastest
   if (idx >= r * C) return;
   const int j = idx / C, c = idx % C;
   float v = 0.f;
-  for (int s = 0; s < splits; ++s) v += partial[((size_t)s * r + j) * C + c];
-  v *= scale;
-  const size_t o = transpose_out ? ((size_t)c * r + j) : (size_t)idx;
-  if constexpr (kF32)
-    reinterpret_cast<float*>(out)[o] = v;
+  for (int sp = 0; sp < J.splits; ++sp) v += J.partial[((size_t)sp * r + j) * C + c];
+  v *= J.scale;
+  const size_t o = J.transpose_out ? ((size_t)c * r + j) : (size_t)idx;
+  if (J.out_dtype == FMSA_F32)
+    reinterpret_cast<float*>(J.out)[o] = v;
   else
-    reinterpret_cast<uint16_t*>(out)[o] = pack1<OutT>(v);
+    reinterpret_cast<uint16_t*>(J.out)[o] = J.out_dtype == FMSA_BF16 ? pack1<bf16_t>(v) : pack1<f16_t>(v);
 }
 
 }  // namespace
@@ -273,16 +323,46 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
   return FMSA_OK;
 }
 
-int launch_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
-                     int act_dtype, int out_dtype, void* out, void* workspace, hipStream_t st) {
-  const int splits = lora_grad_splits(M, C);
-  int rows_per_split = (M + splits - 1) / splits;
-  rows_per_split = ((rows_per_split + LG_TM - 1) / LG_TM) * LG_TM;
-  dim3 grid1((C + LG_TC - 1) / LG_TC, splits), block(256);
-  const int rt = (r + 15) / 16;
-#define LAUNCH(TT, RT)                                                                                            \
-  hipLaunchKernelGGL((lora_grad_partial_kernel<TT, RT>), grid1, block, 0, st, (const uint16_t*)L, ldl,               \
-                     (const uint16_t*)R, ldr, M, C, r, rows_per_split, (float*)workspace)
+size_t lora_grad_batch_workspace(const fmsa_lora_grad_job* jobs, int n_jobs, int M) {
+  size_t bytes = 0;
+  for (int q = 0; q < n_jobs; ++q)
+    bytes += (size_t)lora_grad_splits(M, jobs[q].C) * (size_t)jobs[q].r * (size_t)jobs[q].C * sizeof(float);
+  return bytes;
+}
+
+int launch_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int act_dtype, void* workspace, hipStream_t st) {
+  LoraGradArgs a{};
+  a.n_jobs = n_jobs;
+  a.M = M;
+  int blocks = 0, rblocks = 0, r_max = 0;
+  size_t ws_off = 0;
+  for (int q = 0; q < n_jobs; ++q) {
+    const fmsa_lora_grad_job& s = jobs[q];
+    LoraGradJobDev& d = a.j[q];
+    d.L = (const uint16_t*)s.L;
+    d.R = (const uint16_t*)s.R;
+    d.out = s.out;
+    d.partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + ws_off);
+    d.ldl = s.ldl;
+    d.ldr = s.ldr;
+    d.C = s.C;
+    d.r = s.r;
+    d.splits = lora_grad_splits(M, s.C);
+    const int rows = (M + d.splits - 1) / d.splits;
+    d.rows_per_split = ((rows + LG_TM - 1) / LG_TM) * LG_TM;
+    d.block_start = blocks;
+    d.rblock_start = rblocks;
+    d.transpose_out = s.transpose_out;
+    d.out_dtype = s.out_dtype;
+    d.scale = s.scale;
+    blocks += ((s.C + LG_TC - 1) / LG_TC) * d.splits;
+    rblocks += (s.r * s.C + 255) / 256;
+    ws_off += (size_t)d.splits * s.r * s.C * sizeof(float);
+    r_max = s.r > r_max ? s.r : r_max;
+  }
+  dim3 grid1(blocks), grid2(rblocks), block(256);
+  const int rt = (r_max + 15) / 16;
+#define LAUNCH(TT, RT) hipLaunchKernelGGL((lora_grad_partial_kernel<TT, RT>), grid1, block, 0, st, a)
 #define DISPATCH(TT)                      \
   switch (rt) {                           \
     case 1: LAUNCH(TT, 1); break;         \
@@ -298,16 +378,7 @@ int launch_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int
 #undef DISPATCH
 #undef LAUNCH
   FMSA_CHECK_LAUNCH();
-  dim3 grid2((r * C + 255) / 256);
-  if (out_dtype == FMSA_F32)
-    hipLaunchKernelGGL((lora_grad_reduce_kernel<float, true>), grid2, block, 0, st, (const float*)workspace, splits, r,
-                       C, scale, transpose_out, out);
-  else if (out_dtype == FMSA_BF16)
-    hipLaunchKernelGGL((lora_grad_reduce_kernel<bf16_t, false>), grid2, block, 0, st, (const float*)workspace, splits,
-                       r, C, scale, transpose_out, out);
-  else
-    hipLaunchKernelGGL((lora_grad_reduce_kernel<f16_t, false>), grid2, block, 0, st, (const float*)workspace, splits, r,
-                       C, scale, transpose_out, out);
+  hipLaunchKernelGGL(lora_grad_reduce_kernel, grid2, block, 0, st, a);
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }

@@ -103,8 +103,8 @@ class _Proj:
         """dA [r, K] = s T^T Xd and dB [N, r] = s dY^T U, in the dtypes of the parameters."""
         if not self.r:
             return None, None
-        dA = fmsa_hip.lora_grad(T, Xd, self.s, False, self.A_param.dtype)
-        dB = fmsa_hip.lora_grad(U, dY2, self.s, True, self.B_param.dtype)
+        dA, dB = fmsa_hip.lora_grad_batch([(T, Xd, self.s, False, self.A_param.dtype),
+                                           (U, dY2, self.s, True, self.B_param.dtype)])
         return dA, dB
 
 
@@ -163,15 +163,17 @@ def _adapter_grads(projs, dYs, Xds, Us, stack):
         M = dYs[0].shape[0]
         T_cat = torch.empty((M, stack.R), dtype=dYs[0].dtype, device=dYs[0].device)
         Ts = [fmsa_hip.lora_down(dY, p.Bt, out=T_cat[:, a:b]) for p, dY, (a, b) in zip(projs, dYs, stack.cols)]
-        grads = []
-        if stack.same_s and all(p.A_param.dtype == projs[0].A_param.dtype for p in projs):
-            dA_cat = fmsa_hip.lora_grad(T_cat, Xds[0], projs[0].s, False, projs[0].A_param.dtype)
-            dAs = [dA_cat[a:b] for a, b in stack.cols]
+        # every gradient of the group in one launch of each pass
+        stacked_dA = stack.same_s and all(p.A_param.dtype == projs[0].A_param.dtype for p in projs)
+        if stacked_dA:
+            jobs = [(T_cat, Xds[0], projs[0].s, False, projs[0].A_param.dtype)]
         else:
-            dAs = [fmsa_hip.lora_grad(T, Xds[0], p.s, False, p.A_param.dtype) for p, T in zip(projs, Ts)]
-        for p, dY, U, dA in zip(projs, dYs, Us, dAs):
-            grads.append((dA, fmsa_hip.lora_grad(U, dY, p.s, True, p.B_param.dtype)))
-        return Ts, grads
+            jobs = [(T, Xds[0], p.s, False, p.A_param.dtype) for p, T in zip(projs, Ts)]
+        n_dA = len(jobs)
+        jobs += [(U, dY, p.s, True, p.B_param.dtype) for p, dY, U in zip(projs, dYs, Us)]
+        outs = fmsa_hip.lora_grad_batch(jobs)
+        dAs = [outs[0][a:b] for a, b in stack.cols] if stacked_dA else outs[:n_dA]
+        return Ts, list(zip(dAs, outs[n_dA:]))
     Ts, grads = [], []
     for p, dY, Xd, U in zip(projs, dYs, Xds, Us):
         T = fmsa_hip.lora_down(dY, p.Bt) if p.r else None

@@ -31,6 +31,8 @@ EXPORTED_SYMBOLS = (
     "fmsa_lora_down",
     "fmsa_lora_grad_workspace",
     "fmsa_lora_grad",
+    "fmsa_lora_grad_batch_workspace",
+    "fmsa_lora_grad_batch",
     "fmsa_gptq_lora_fwd",
     "fmsa_gptq_lora_bwd_dx",
     "fmsa_swiglu_fwd",
@@ -80,6 +82,24 @@ class Nf4Weight(Structure):
         ("K", c_int32),
         ("blocksize", c_int32),
         ("blocksize2", c_int32),
+    ]
+
+
+class LoraGradJob(Structure):
+    """fmsa_lora_grad_job: one scale * L[M, r]^T @ R[M, C] of a batch."""
+
+    _fields_ = [
+        ("L", c_void_p),
+        ("R", c_void_p),
+        ("out", c_void_p),
+        ("ldl", c_int64),
+        ("ldr", c_int64),
+        ("C", c_int32),
+        ("r", c_int32),
+        ("scale", c_float),
+        ("transpose_out", c_int32),
+        ("out_dtype", c_int32),
+        ("reserved", c_int32),
     ]
 
 
@@ -138,6 +158,9 @@ def lib() -> ctypes.CDLL:
     L.fmsa_lora_grad_workspace.argtypes = [c_int, c_int, c_int]
     L.fmsa_lora_grad.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
                                  c_void_p, c_void_p, c_size_t, c_void_p]
+    L.fmsa_lora_grad_batch_workspace.restype = c_size_t
+    L.fmsa_lora_grad_batch_workspace.argtypes = [POINTER(LoraGradJob), c_int, c_int]
+    L.fmsa_lora_grad_batch.argtypes = [POINTER(LoraGradJob), c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]
     L.fmsa_gptq_lora_fwd.argtypes = [POINTER(FwdProj), c_int, c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                                      c_int, c_void_p]
     L.fmsa_gptq_lora_bwd_dx.argtypes = [POINTER(BwdProj), c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p,
@@ -293,6 +316,33 @@ def lora_grad(L, R, scale: float, transpose_out: bool, out_dtype=torch.float32):
            lib().fmsa_lora_grad(_ptr(L), L.stride(0), _ptr(R), R.stride(0), M, C, r, float(scale), int(transpose_out),
                                 act_enum(R.dtype), _DTYPE_ENUM[out_dtype], _ptr(out), _ptr(ws), ws.numel(), _stream(out)))
     return out
+
+
+LORA_GRAD_MAX_JOBS = 8
+
+
+def lora_grad_batch(jobs):
+    """jobs: (L, R, scale, transpose_out, out_dtype) tuples over the same M tokens; returns the list of
+    scale * L^T @ R, each as lora_grad would give it, from one launch of each pass per
+    LORA_GRAD_MAX_JOBS jobs."""
+    outs = []
+    for i in range(0, len(jobs), LORA_GRAD_MAX_JOBS):
+        chunk = jobs[i : i + LORA_GRAD_MAX_JOBS]
+        M = chunk[0][0].shape[0]
+        arr = (LoraGradJob * len(chunk))()
+        for q, (L, R, scale, tr, out_dtype) in enumerate(chunk):
+            r, C = L.shape[1], R.shape[1]
+            assert L.shape[0] == M and R.shape[0] == M and L.stride(1) == 1 and R.stride(1) == 1
+            assert L.dtype == R.dtype == chunk[0][1].dtype
+            out = torch.empty((C, r) if tr else (r, C), dtype=out_dtype, device=R.device)
+            outs.append(out)
+            arr[q] = LoraGradJob(_ptr(L), _ptr(R), _ptr(out), L.stride(0), R.stride(0), C, r, float(scale), int(tr),
+                                 _DTYPE_ENUM[out_dtype], 0)
+        R0 = chunk[0][1]
+        ws = _workspace(lib().fmsa_lora_grad_batch_workspace(arr, len(chunk), M), R0.device)
+        _check("fmsa_lora_grad_batch",
+               lib().fmsa_lora_grad_batch(arr, len(chunk), M, act_enum(R0.dtype), _ptr(ws), ws.numel(), _stream(R0)))
+    return outs
 
 
 def gptq_lora_fwd(x2d, projs: Sequence[dict], mode: int = FWD_LINEAR):

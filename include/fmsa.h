@@ -119,6 +119,28 @@ int fmsa_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int M
                    int transpose_out, int act_dtype, int out_dtype, void* out, void* workspace,
                    size_t workspace_bytes, void* stream);
 
+/* Several such gradients over the same M tokens in one launch of each pass: the adapter gradients
+ * one backward produces (dA of the stacked adapters and every dB, :822-825 for each projection of
+ * LoRA_QKV :657-674 / LoRA_MLP :351-398) are each too small to fill the chip alone.  Job q is
+ * exactly fmsa_lora_grad with its fields; results are bit-identical to separate calls.  All jobs
+ * share M and act_dtype; 1 <= n_jobs <= FMSA_LORA_GRAD_MAX_JOBS; `workspace` holds
+ * fmsa_lora_grad_batch_workspace() bytes (the jobs' partial sums side by side). */
+#define FMSA_LORA_GRAD_MAX_JOBS 8
+typedef struct fmsa_lora_grad_job {
+  const void* L; /* [M, r], row stride ldl */
+  const void* R; /* [M, C], row stride ldr */
+  void* out;     /* [r, C], or [C, r] when transpose_out */
+  int64_t ldl, ldr;
+  int32_t C, r;
+  float scale;
+  int32_t transpose_out;
+  int32_t out_dtype; /* FMSA_F32, FMSA_BF16 or FMSA_F16 */
+  int32_t reserved;
+} fmsa_lora_grad_job;
+size_t fmsa_lora_grad_batch_workspace(const fmsa_lora_grad_job* jobs, int n_jobs, int M);
+int fmsa_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int act_dtype, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
 /* The four activation-type copies of one adapter that the kernels above and below read, in one
  * launch: A16 [r, K], At16 [K, r] from A = lora_A.weight [r, K]; B16 [N, r], Bt16 [r, N] from
  * B = lora_B.weight [N, r].  Each value is the parameter rounded once (RNE) to act_dtype -- the

@@ -31,6 +31,7 @@ def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(fmsa_hip.GptqWeight) == 72
     assert ctypes.sizeof(fmsa_hip.FwdProj) == 128
     assert ctypes.sizeof(fmsa_hip.BwdProj) == 144
+    assert ctypes.sizeof(fmsa_hip.LoraGradJob) == 64
 
 
 def _w(K=64, N=64, gs=64, q=0x1000, s=0x2000, z=0x3000, g=None, zo=0):
@@ -128,6 +129,23 @@ def test_bwd_and_skinny_validation():
     assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 64, 16, 1, 0x3000, 8, None) == -2   # ldout < r
     assert lib.fmsa_lora_grad_workspace(8192, 4096, 16) > 0
     assert lib.fmsa_lora_grad(0x1000, 16, 0x2000, 64, 8, 64, 16, 1.0, 0, 1, 2, 0x3000, None, 0, None) == -6
+    J = fmsa_hip.LoraGradJob
+    job = lambda **kw: J(**{**dict(L=0x1000, R=0x2000, out=0x3000, ldl=16, ldr=64, C=64, r=16, scale=1.0, transpose_out=0,
+                                   out_dtype=2, reserved=0), **kw})
+    gb, gw = lib.fmsa_lora_grad_batch, lib.fmsa_lora_grad_batch_workspace
+    two = (J * 2)(job(), job(C=128, ldr=128, r=8))
+    assert gw(two, 2, 8) == lib.fmsa_lora_grad_workspace(8, 64, 16) + lib.fmsa_lora_grad_workspace(8, 128, 8)
+    assert gw(two, 0, 8) == 0 and gw(two, 9, 8) == 0
+    assert gb(None, 1, 8, 1, 0x4000, 1 << 20, None) == -1
+    assert gb(two, 0, 8, 1, 0x4000, 1 << 20, None) == -2 and gb(two, 9, 8, 1, 0x4000, 1 << 20, None) == -2
+    assert gb(two, 2, 8, 2, 0x4000, 1 << 20, None) == -4                       # fp32 is no activation dtype
+    assert gb((J * 2)(job(), job(out=None)), 2, 8, 1, 0x4000, 1 << 20, None) == -1
+    assert gb((J * 2)(job(), job(r=12)), 2, 8, 1, 0x4000, 1 << 20, None) == -2
+    assert gb((J * 2)(job(), job(ldr=32)), 2, 8, 1, 0x4000, 1 << 20, None) == -2  # rows of R shorter than C
+    assert gb((J * 2)(job(), job(out_dtype=7)), 2, 8, 1, 0x4000, 1 << 20, None) == -4
+    assert gb((J * 2)(job(), job(L=0x1004)), 2, 8, 1, 0x4000, 1 << 20, None) == -3
+    assert gb(two, 2, 8, 1, 0x4000, gw(two, 2, 8) - 1, None) == -6             # workspace one byte short
+    assert gb(two, 2, 8, 1, None, 1 << 20, None) == -6
     assert lib.fmsa_lora_pack(None, 0x1000, 16, 64, 64, 2, 1, None, None, None, None, None) == -1
     assert lib.fmsa_lora_pack(0x1000, 0x2000, 16, 64, 64, 2, 2, None, None, None, None, None) == -4
     assert lib.fmsa_swiglu_fwd(0x1000, 0x2000, 0x3000, 8, 60, 64, 1, None) == -2

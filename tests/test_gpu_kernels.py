@@ -46,7 +46,7 @@ def test_dequant_bit_exact(K, N, gs, act_order, v1):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,C,r", [(512, 2048, 16), (200, 4096, 8), (64, 1056, 64), (33, 96, 24)])
+@pytest.mark.parametrize("M,C,r", [(512, 2048, 16), (200, 4096, 8), (64, 1056, 64), (33, 96, 24), (300, 2048, 96), (8192, 1024, 128)])
 def test_lora_down(M, C, r, dtype):
     import fmsa_hip
 
@@ -58,7 +58,8 @@ def test_lora_down(M, C, r, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,C,r,tr", [(512, 2048, 16, False), (200, 1056, 8, True), (4096, 4096, 16, True), (96, 136, 24, False), (70, 4104, 64, True)])
+@pytest.mark.parametrize("M,C,r,tr", [(512, 2048, 16, False), (200, 1056, 8, True), (4096, 4096, 16, True), (96, 136, 24, False), (70, 4104, 64, True),
+                                      (1000, 2048, 96, False), (333, 520, 128, True)])
 def test_lora_grad(M, C, r, tr, dtype):
     import fmsa_hip
 
@@ -74,6 +75,29 @@ def test_lora_grad(M, C, r, tr, dtype):
     assert torch.equal(out, out2), "two-pass reduction must be run-to-run bit-stable"
     outb = fmsa_hip.lora_grad(dev(L), dev(R), 0.5, tr, dtype).cpu()
     assert olora.max_rel_err(outb, ref) < 5e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_lora_grad_batch_equals_separate_calls(dtype):
+    """Jobs of different widths, ranks, layouts and output types in one launch: each result is bit
+    for bit what fmsa_lora_grad gives for that job alone (checked against the fp32 product above).
+    Ten jobs also cover the split into launches of at most eight."""
+    import fmsa_hip
+
+    M = 1111
+    shapes = [(2048, 48, False, torch.float32), (2048, 16, True, dtype), (520, 16, True, torch.float32), (136, 8, False, dtype),
+              (4104, 64, True, torch.float32), (1056, 96, False, torch.float32), (96, 24, True, dtype), (2048, 16, True, torch.float32),
+              (520, 128, False, dtype), (8, 8, False, torch.float32)]
+    jobs = []
+    for i, (C, r, tr, od) in enumerate(shapes):
+        Lfull = dev(randn((M, r + 8), 70 + i, dtype))  # a column slice: row stride > r
+        jobs.append((Lfull[:, :r], dev(randn((M, C), 90 + i, dtype)), 0.5 + i, tr, od))
+    outs = fmsa_hip.lora_grad_batch(jobs)
+    assert len(outs) == len(jobs)
+    for (L, R, scale, tr, od), out in zip(jobs, outs):
+        single = fmsa_hip.lora_grad(L, R, scale, tr, od)
+        assert out.dtype == od and out.shape == single.shape
+        assert torch.equal(out, single)
 
 
 def _fwd_case(M, K, N, gs, r, dtype, s=2.0, bias=False, seed=0):
