@@ -123,6 +123,14 @@ FMSA_DEVI __amdgpu_buffer_rsrc_t make_rsrc(const void* base, size_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(ub, 0, (int)n, 0x00020000);
 }
 
+// Cache policy of the GEMM epilogues' output stores (the `aux` operand of the buffer-store builtins; bit 1 = nt on
+// gfx94x / gfx950).  A launch writes up to 705 MB that nothing re-reads before the launch ends.  Written with the
+// default policy the tail of it stays dirty in the memory-side cache, and the NEXT kernel pays for the write-back:
+// every line it brings in evicts a dirty one, so a bandwidth-bound kernel right after the gate/up GEMM ran at half
+// speed (86 us instead of 50 us for one pass over h).  Non-temporal stores drain to HBM while the GEMM, which is
+// bound by the matrix pipe, still runs; the GEMM's own duration does not change.
+constexpr int STORE_NT = 2;
+
 // ---- workgroup-id remap: consecutive ids land on different XCDs (id % 8), each with its own
 // L2.  Give every XCD a contiguous range of logical tiles so neighbours share operands in L2.
 FMSA_DEVI int xcd_remap(int pid, int total) {

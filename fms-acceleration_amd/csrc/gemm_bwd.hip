@@ -721,9 +721,9 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
           dev[w] = pack2<T>(unpack_lo<T>(tp) * se0 * (1.0f + e0 * (1.0f - se0)),   // d_e (:81-83)
                             unpack_hi<T>(tp) * se1 * (1.0f + e1 * (1.0f - se1)));
         }
-        __builtin_amdgcn_raw_buffer_store_b128(hv, h_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
-        __builtin_amdgcn_raw_buffer_store_b128(dgv, e_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
-        __builtin_amdgcn_raw_buffer_store_b128(dev, g_rsrc, eg_voff, soff_rows * eg_row_bytes, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(hv, h_rsrc, eg_voff, soff_rows * eg_row_bytes, STORE_NT);
+        __builtin_amdgcn_raw_buffer_store_b128(dgv, e_rsrc, eg_voff, soff_rows * eg_row_bytes, STORE_NT);
+        __builtin_amdgcn_raw_buffer_store_b128(dev, g_rsrc, eg_voff, soff_rows * eg_row_bytes, STORE_NT);
       } else {
         u32x4 ov = bv;
         if (any_lora) {
@@ -735,7 +735,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_kernel(const BwdArgs a) 
             ov[w] = pack2<T>(unpack_lo<T>(bv[w]) + l0, unpack_hi<T>(bv[w]) + l1);
           }
         }
-        __builtin_amdgcn_raw_buffer_store_b128(ov, dx_rsrc, dx_voff, soff_rows * dx_row_bytes, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(ov, dx_rsrc, dx_voff, soff_rows * dx_row_bytes, STORE_NT);
       }
       // the operands of this chunk are dead now: the request for the next pass can reuse their registers
       __builtin_amdgcn_sched_barrier(0);

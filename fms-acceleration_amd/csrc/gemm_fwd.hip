@@ -622,9 +622,9 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
         const int row = crow + 16 * it;
         const uint32_t srow = (uint32_t)(EP_ROWS * q + 16 * it);
         const int o = row * EP_STRIDE_S + 8 * cchunk;
-        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane0 + o), y0_rsrc, y0_voff, srow * y0_row, 0);
-        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane1 + o), y1_rsrc, y1_voff, srow * y1_row, 0);
-        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane2 + o), h_rsrc, h_voff, srow * h_row, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane0 + o), y0_rsrc, y0_voff, srow * y0_row, STORE_NT);
+        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane1 + o), y1_rsrc, y1_voff, srow * y1_row, STORE_NT);
+        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane2 + o), h_rsrc, h_voff, srow * h_row, STORE_NT);
       }
     } else {
 #pragma unroll
@@ -632,7 +632,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
         const int row = crow + 8 * it;
         const uint32_t srow = (uint32_t)(EP_ROWS * q + 8 * it);
         __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane0 + row * EP_STRIDE_L + 8 * cchunk), y0_rsrc,
-                                               y0_voff, srow * y0_row, 0);
+                                               y0_voff, srow * y0_row, STORE_NT);
       }
     }
     __syncthreads();

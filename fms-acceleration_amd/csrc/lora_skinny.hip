@@ -91,6 +91,155 @@ __global__ __launch_bounds__(64 * NW) void lora_down_kernel(const uint16_t* __re
   }
 }
 
+// ---- lora_down, staged ----------------------------------------------------------------------------
+// The same product for the large-M case, with X going through LDS: a direct load of one wave moves a
+// whole 1 KB run of one row (512 columns), where the fragment loads above fetch 64 B of each of 16
+// rows per instruction.  Workgroup = 32 tokens, 8 waves; a stage = 32 rows x 512 columns (32 KB) in
+// one of four LDS buffers, so up to two stages are in flight while a third is multiplied.  Slot c of
+// row m holds chunk c ^ (m & 15) of the row's run (the permutation is applied on the global side: a
+// direct load writes lane p's 16 bytes to slot p), which spreads the 16 rows a fragment read touches
+// over all banks.  Wave w multiplies columns 64w .. 64w+63 of every stage; its Wd fragments come
+// straight from global (L2) one stage ahead.  Partial sums of the 8 waves are added as above.
+template <typename T, int RT>
+__global__ __launch_bounds__(512) void lora_down_staged_kernel(const uint16_t* __restrict__ X, int64_t ldx,
+                                                               const uint16_t* __restrict__ Wd, int M, int C, int r,
+                                                               uint16_t* __restrict__ out, int64_t ldo) {
+  constexpr int NW = 8, NH = 4, MTL = 2, ROWS = 32, SC = 512;
+  static_assert(RT <= 4, "the reduction buffer overlays one stage buffer");
+  // four separate arrays: every access names its buffer statically, so the compiler's wait counts
+  // can tell reads of one buffer from direct loads in flight into the others
+  __shared__ __attribute__((aligned(1024))) uint16_t s0[ROWS * SC];
+  __shared__ __attribute__((aligned(1024))) uint16_t s1[ROWS * SC];
+  __shared__ __attribute__((aligned(1024))) uint16_t s2[ROWS * SC];
+  __shared__ __attribute__((aligned(1024))) uint16_t s3[ROWS * SC];
+  auto buf = [&](auto b_c) -> char* {
+    constexpr int b = decltype(b_c)::value;
+    return reinterpret_cast<char*>(b == 0 ? s0 : (b == 1 ? s1 : (b == 2 ? s2 : s3)));
+  };
+  using B0 = std::integral_constant<int, 0>;
+  using B1 = std::integral_constant<int, 1>;
+  using B2 = std::integral_constant<int, 2>;
+  using B3 = std::integral_constant<int, 3>;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int uwave = __builtin_amdgcn_readfirstlane(wave);
+  const int l16 = lane & 15, q = lane >> 4;
+  const int m_base = blockIdx.x * ROWS;
+  const int rows_valid = min(ROWS, M - m_base);
+  const int n_stages = (C + SC - 1) / SC;
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(X + (size_t)m_base * ldx, (size_t)rows_valid * ldx * 2);
+  const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(Wd, (size_t)r * C * 2);
+
+  // direct loads: wave w moves rows 4w .. 4w+3 of a stage
+  uint32_t d_off[4], d_col[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 4 * wave + i;
+    d_col[i] = 8 * (lane ^ (row & 15));
+    d_off[i] = (uint32_t)((row * ldx + d_col[i]) * 2);
+  }
+  auto dma = [&](int st, auto b_c) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t dead = (st * SC + (int)d_col[i]) < C ? 0u : 0x80000000u;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (__attribute__((address_space(3))) void*)(buf(b_c) + (4 * uwave + i) * (SC * 2)),
+                                               16, d_off[i] | dead, (uint32_t)st * (SC * 2), 0, 0);
+    }
+  };
+  // Wd fragments of the wave's two 32-column steps of a stage
+  uint32_t w_off[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) w_off[t] = (uint32_t)(((16 * t + l16) * (int64_t)C + 8 * q) * 2);
+  auto wld = [&](int st, u32x4(&wf)[2][RT]) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const int c0 = st * SC + 32 * (2 * wave + kk);
+      const uint32_t dead = (c0 + 8 * q) < C ? 0u : 0x80000000u;
+#pragma unroll
+      for (int t = 0; t < RT; ++t) wf[kk][t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (w_off[t] + 2 * c0) | dead, 0, 0);
+    }
+  };
+  f32x4 acc[MTL][RT];
+#pragma unroll
+  for (int u = 0; u < MTL; ++u)
+#pragma unroll
+    for (int t = 0; t < RT; ++t) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto mul = [&](auto b_c, const u32x4(&wf)[2][RT]) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const int chunk = 4 * (2 * wave + kk) + q;
+#pragma unroll
+      for (int u = 0; u < MTL; ++u) {
+        const u32x4 xf = *reinterpret_cast<const u32x4*>(buf(b_c) + (16 * u + l16) * (SC * 2) + ((chunk ^ l16) * 16));
+#pragma unroll
+        for (int t = 0; t < RT; ++t) acc[u][t] = mfma16<T>(xf, wf[kk][t], acc[u][t]);  // D[i = token][j = rank]
+      }
+    }
+  };
+  // s_waitcnt vmcnt(n) only (expcnt / lgkmcnt fields left at their maxima)
+  constexpr int YOUNGER = 8 + 4 * RT;  // loads a wave issues after the direct loads of a stage and before that stage's turn
+  constexpr int WAIT_STEADY = (YOUNGER & 0xF) | ((YOUNGER >> 4) << 14) | 0x0F70;
+  constexpr int YOUNGER0 = 8 + 2 * RT;  // ... for stage 0 (prologue order)
+  constexpr int WAIT_FIRST = (YOUNGER0 & 0xF) | ((YOUNGER0 >> 4) << 14) | 0x0F70;
+  // one stage: its own direct loads have landed -> barrier (all waves' parts are there, and everybody has
+  // left the buffer that is re-filled next) -> requests two and three stages ahead -> multiply
+  u32x4 wa[2][RT], wb[2][RT];
+  auto turn = [&](int st, auto cur_c, auto refill_c, const u32x4(&wcur)[2][RT], u32x4(&wnext)[2][RT]) {
+    if (st == 0)
+      __builtin_amdgcn_s_waitcnt(WAIT_FIRST);
+    else
+      __builtin_amdgcn_s_waitcnt(WAIT_STEADY);
+    // a bare barrier: the fence of __syncthreads() would wait for ALL direct loads in flight (they
+    // are stores to LDS), the two stages ahead included
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    wld(st + 1, wnext);
+    dma(st + 3, refill_c);
+    mul(cur_c, wcur);
+  };
+  dma(0, B0{});
+  dma(1, B1{});
+  dma(2, B2{});
+  wld(0, wa);
+  for (int st = 0; st < n_stages; st += 4) {
+    turn(st, B0{}, B3{}, wa, wb);
+    turn(st + 1, B1{}, B0{}, wb, wa);
+    turn(st + 2, B2{}, B1{}, wa, wb);
+    turn(st + 3, B3{}, B2{}, wb, wa);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the surplus direct loads (all lanes out of range) have landed too
+  __syncthreads();
+
+  float(*red)[MTL][RT][64][4] = reinterpret_cast<float(*)[MTL][RT][64][4]>(s0);  // [NH]: 8 * RT KB <= one stage buffer
+  if (wave >= NH) {
+#pragma unroll
+    for (int u = 0; u < MTL; ++u)
+#pragma unroll
+      for (int t = 0; t < RT; ++t) *reinterpret_cast<f32x4*>(red[wave - NH][u][t][lane]) = acc[u][t];
+  }
+  __syncthreads();
+  if (wave < NH) {
+#pragma unroll
+    for (int u = 0; u < MTL; ++u)
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const f32x4 o = *reinterpret_cast<const f32x4*>(red[wave][u][t][lane]);
+        *reinterpret_cast<f32x4*>(red[wave][u][t][lane]) = acc[u][t] + o;
+      }
+  }
+  __syncthreads();
+  for (int o = tid; o < MTL * RT * 256; o += 64 * NW) {
+    const int u = o / (RT * 256), t = (o >> 8) % RT, ln = (o >> 2) & 63, i = o & 3;
+    float v = red[0][u][t][ln][i];
+#pragma unroll
+    for (int w = 1; w < NH; ++w) v += red[w][u][t][ln][i];
+    const int row = m_base + 16 * u + 4 * (ln >> 4) + i;
+    const int j = 16 * t + (ln & 15);
+    if (row < M && j < r) out[(size_t)row * ldo + j] = pack1<T>(v);
+  }
+}
+
 // ---- lora_grad ----------------------------------------------------------------------------------
 // out[j, c] = sum_m L[m, j] * R[m, c]: the contraction runs over tokens, which is the row index of
 // both row-major operands, so each MFMA fragment (8 consecutive contraction elements per lane) is a
@@ -296,6 +445,31 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
   constexpr int NW = 8;  // waves per workgroup: measured best of 4 / 8 / 16 at 8192 tokens
   dim3 grid((M + 16 * mtl - 1) / (16 * mtl)), block(64 * NW);
   const int rt = (r + 15) / 16;
+  // staged kernel: 32 tokens per workgroup, worth it once that gives every CU a workgroup and the rows are long
+  // enough to amortise its pipeline fill (measured at 8192 tokens: 59 -> 48 us at C = 14336, r = 16; 32 -> 28 us
+  // at C = 4096, r = 48; 20 -> 21 us at C = 4096, r = 16)
+  const bool staged = M >= 32 * 256 && rt <= 4 && (C >= 8192 || (rt >= 2 && C >= 2048));
+  if (staged) {
+    dim3 sgrid((M + 31) / 32), sblock(512);
+#define SLAUNCH(TT, RT)                                                                                                        \
+  hipLaunchKernelGGL((lora_down_staged_kernel<TT, RT>), sgrid, sblock, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, M, C, \
+                     r, (uint16_t*)out, ldo)
+#define SDISPATCH(TT)                \
+  switch (rt) {                      \
+    case 1: SLAUNCH(TT, 1); break;   \
+    case 2: SLAUNCH(TT, 2); break;   \
+    default: SLAUNCH(TT, 4); break;  \
+  }
+    if (act_dtype == FMSA_BF16) {
+      SDISPATCH(bf16_t)
+    } else {
+      SDISPATCH(f16_t)
+    }
+#undef SDISPATCH
+#undef SLAUNCH
+    FMSA_CHECK_LAUNCH();
+    return FMSA_OK;
+  }
 #define LAUNCH(TT, RT)                                                                                                       \
   do {                                                                                                                       \
     if (mtl == 2)                                                                                                            \

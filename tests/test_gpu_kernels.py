@@ -58,6 +58,25 @@ def test_lora_down(M, C, r, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,C,r", [(8192, 8200, 16), (8200, 14336, 32), (8192, 2048, 48), (8222, 9000, 64), (8192, 4096, 24)])
+def test_lora_down_many_tokens(M, C, r, dtype):
+    """From 8192 tokens on, long rows / stacked ranks take the kernel that stages X through LDS: ragged
+    token and column counts (last workgroup of 8 or 30 rows, last 512-column stage of 8 or 296 columns),
+    X as a column slice of a wider matrix and the output as a column slice of a stacked one."""
+    import fmsa_hip
+
+    xw = dev(randn((M, C + 24), 12, dtype))
+    x = xw[:, 8 : 8 + C]  # row stride C + 24, base 16 bytes into the row
+    wd = dev(randn((r, C), 13, dtype, 0.05))
+    ref = x.float() @ wd.float().t()
+    out_cat = torch.full((M, r + 16), 7.0, dtype=dtype, device=x.device)
+    out = fmsa_hip.lora_down(x, wd, out=out_cat[:, 8 : 8 + r])
+    assert olora.max_rel_err(out.cpu(), ref.cpu()) < 5e-3
+    assert torch.all(out_cat[:, :8] == 7.0) and torch.all(out_cat[:, 8 + r :] == 7.0)
+    assert torch.equal(fmsa_hip.lora_down(x, wd), out)  # run-to-run bit-stable, whatever the output stride
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,C,r,tr", [(512, 2048, 16, False), (200, 1056, 8, True), (4096, 4096, 16, True), (96, 136, 24, False), (70, 4104, 64, True),
                                       (1000, 2048, 96, False), (333, 520, 128, True)])
 def test_lora_grad(M, C, r, tr, dtype):
