@@ -17,8 +17,7 @@ int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int m
                             void* g, void* h_out, int64_t ldeg, int act_dtype, hipStream_t st);
 
 int launch_gptq_nsz(const fmsa_gptq_weight* w, float* out, hipStream_t st);
-int launch_lora_pack(const void* A, const void* B, int r, int K, int N, int param_dtype, int act_dtype, void* A16, void* At16,
-                     void* B16, void* Bt16, hipStream_t st);
+int launch_lora_pack_batch(const fmsa_lora_pack_job* jobs, int n_jobs, int act_dtype, hipStream_t st);
 int launch_rms_fwd(const void* X, int64_t ldx, const void* W, int M, int C, float eps, int gemma, int x_dtype, int w_dtype, void* Y,
                    int64_t ldy, float* r, hipStream_t st);
 int launch_rms_bwd(void* dY, int64_t lddy, const void* X, int64_t ldx, const void* W, const float* r, int M, int C, int gemma,
@@ -273,13 +272,23 @@ int fmsa_gptq_make_nsz(const fmsa_gptq_weight* w, float* out, void* stream) {
   return launch_gptq_nsz(w, out, (hipStream_t)stream);
 }
 
+int fmsa_lora_pack_batch(const fmsa_lora_pack_job* jobs, int n_jobs, int act_dtype, void* stream) {
+  if (!jobs) return FMSA_ERR_NULL;
+  if (n_jobs < 1 || n_jobs > FMSA_LORA_PACK_MAX_JOBS) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  for (int q = 0; q < n_jobs; ++q) {
+    const fmsa_lora_pack_job& j = jobs[q];
+    if (!j.A || !j.B) return FMSA_ERR_NULL;
+    if (j.r <= 0 || j.K <= 0 || j.N <= 0) return FMSA_ERR_SHAPE;
+    if (j.param_dtype != FMSA_F32 && j.param_dtype != FMSA_BF16 && j.param_dtype != FMSA_F16) return FMSA_ERR_DTYPE;
+  }
+  return launch_lora_pack_batch(jobs, n_jobs, act_dtype, (hipStream_t)stream);
+}
+
 int fmsa_lora_pack(const void* A, const void* B, int r, int K, int N, int param_dtype, int act_dtype, void* A16, void* At16,
                    void* B16, void* Bt16, void* stream) {
-  if (!A || !B) return FMSA_ERR_NULL;
-  if (r <= 0 || K <= 0 || N <= 0) return FMSA_ERR_SHAPE;
-  if (param_dtype != FMSA_F32 && param_dtype != FMSA_BF16 && param_dtype != FMSA_F16) return FMSA_ERR_DTYPE;
-  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
-  return launch_lora_pack(A, B, r, K, N, param_dtype, act_dtype, A16, At16, B16, Bt16, (hipStream_t)stream);
+  const fmsa_lora_pack_job job = {A, B, A16, At16, B16, Bt16, r, K, N, param_dtype};
+  return fmsa_lora_pack_batch(&job, 1, act_dtype, stream);
 }
 
 int fmsa_nf4_dequant(const fmsa_nf4_weight* w, int out_dtype, void* out, void* stream) {

@@ -72,20 +72,44 @@ template <> FMSA_DEVI float load_param<float>(const void* p, int64_t i) { return
 template <> FMSA_DEVI float load_param<bf16_t>(const void* p, int64_t i) { return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]); }
 template <> FMSA_DEVI float load_param<f16_t>(const void* p, int64_t i) { return fp16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]); }
 
-template <typename TIN, typename T>
-__global__ __launch_bounds__(256) void lora_pack_kernel(const void* __restrict__ A, const void* __restrict__ B, int r, int K, int N,
-                                                        uint16_t* __restrict__ A16, uint16_t* __restrict__ At16,
-                                                        uint16_t* __restrict__ B16, uint16_t* __restrict__ Bt16) {
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+// The adapters of one fused operator go out together (one launch instead of one per projection); workgroup ids
+// are laid end to end over the jobs.
+struct LoraPackArgs {
+  fmsa_lora_pack_job j[FMSA_LORA_PACK_MAX_JOBS];
+  int block_start[FMSA_LORA_PACK_MAX_JOBS];
+  int n_jobs;
+};
+FMSA_DEVI float load_param_rt(const void* p, int64_t i, int dtype) {
+  if (dtype == FMSA_F32) return load_param<float>(p, i);
+  return dtype == FMSA_BF16 ? load_param<bf16_t>(p, i) : load_param<f16_t>(p, i);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void lora_pack_kernel(const LoraPackArgs a) {
+  // the job that owns this workgroup, copied field by field (no runtime index into the argument struct)
+  fmsa_lora_pack_job J = a.j[0];
+  int start = 0;
+#pragma unroll
+  for (int q = 1; q < FMSA_LORA_PACK_MAX_JOBS; ++q)
+    if (q < a.n_jobs && (int)blockIdx.x >= a.block_start[q]) {
+      J = a.j[q];
+      start = a.block_start[q];
+    }
+  const int r = J.r, K = J.K, N = J.N;
+  uint16_t* A16 = reinterpret_cast<uint16_t*>(J.A16);
+  uint16_t* At16 = reinterpret_cast<uint16_t*>(J.At16);
+  uint16_t* B16 = reinterpret_cast<uint16_t*>(J.B16);
+  uint16_t* Bt16 = reinterpret_cast<uint16_t*>(J.Bt16);
+  const int64_t idx = (int64_t)(blockIdx.x - start) * blockDim.x + threadIdx.x;
   if (idx < (int64_t)r * K) {
     const int j = (int)(idx / K), k = (int)(idx % K);
-    const uint16_t v = pack1<T>(load_param<TIN>(A, idx));
+    const uint16_t v = pack1<T>(load_param_rt(J.A, idx, J.param_dtype));
     if (A16) A16[idx] = v;
     if (At16) At16[(int64_t)k * r + j] = v;
   }
   if (idx < (int64_t)N * r) {
     const int n = (int)(idx / r), j = (int)(idx % r);
-    const uint16_t v = pack1<T>(load_param<TIN>(B, idx));
+    const uint16_t v = pack1<T>(load_param_rt(J.B, idx, J.param_dtype));
     if (B16) B16[idx] = v;
     if (Bt16) Bt16[(int64_t)j * N + n] = v;
   }
@@ -120,25 +144,21 @@ int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, i
   return FMSA_OK;
 }
 
-int launch_lora_pack(const void* A, const void* B, int r, int K, int N, int param_dtype, int act_dtype, void* A16, void* At16,
-                     void* B16, void* Bt16, hipStream_t st) {
-  const int64_t n = (int64_t)r * (K > N ? K : N);
-  dim3 grid((unsigned)((n + 255) / 256)), block(256);
-#define LAUNCH(TIN, TT)                                                                                          \
-  hipLaunchKernelGGL((lora_pack_kernel<TIN, TT>), grid, block, 0, st, A, B, r, K, N, (uint16_t*)A16, (uint16_t*)At16, \
-                     (uint16_t*)B16, (uint16_t*)Bt16)
-#define DISPATCH(TT)                                      \
-  do {                                                    \
-    if (param_dtype == FMSA_F32) LAUNCH(float, TT);       \
-    else if (param_dtype == FMSA_BF16) LAUNCH(bf16_t, TT); \
-    else LAUNCH(f16_t, TT);                               \
-  } while (0)
+int launch_lora_pack_batch(const fmsa_lora_pack_job* jobs, int n_jobs, int act_dtype, hipStream_t st) {
+  LoraPackArgs a{};
+  a.n_jobs = n_jobs;
+  int64_t blocks = 0;
+  for (int q = 0; q < n_jobs; ++q) {
+    a.j[q] = jobs[q];
+    a.block_start[q] = (int)blocks;
+    const int64_t n = (int64_t)jobs[q].r * (jobs[q].K > jobs[q].N ? jobs[q].K : jobs[q].N);
+    blocks += (n + 255) / 256;
+  }
+  dim3 grid((unsigned)blocks), block(256);
   if (act_dtype == FMSA_BF16)
-    DISPATCH(bf16_t);
+    hipLaunchKernelGGL(lora_pack_kernel<bf16_t>, grid, block, 0, st, a);
   else
-    DISPATCH(f16_t);
-#undef DISPATCH
-#undef LAUNCH
+    hipLaunchKernelGGL(lora_pack_kernel<f16_t>, grid, block, 0, st, a);
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }

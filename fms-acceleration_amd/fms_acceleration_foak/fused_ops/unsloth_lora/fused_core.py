@@ -76,8 +76,7 @@ class _Proj:
         self.A = self.At = self.B = self.Bt = None
 
     def pack(self, A16_out=None):
-        if self.r:
-            self.A, self.At, self.B, self.Bt = fmsa_hip.lora_pack(self.A_param, self.B_param, self.dtype, A16_out)
+        _pack_projs([(self, A16_out)])
 
     # the kernels walk K in the repacked order for act-order weights
     def to_kernel_order(self, X2):
@@ -108,32 +107,42 @@ class _Proj:
         return dA, dB
 
 
+def _pack_projs(items):
+    """items: (projection, A16_out or None).  One launch packs the adapters of all of them."""
+    live = [(p, out) for p, out in items if p.r]
+    if live:
+        packed = fmsa_hip.lora_pack_batch([(p.A_param, p.B_param, out) for p, out in live], live[0][0].dtype)
+        for (p, _), quad in zip(live, packed):
+            p.A, p.At, p.B, p.Bt = quad
+
+
 class _Stack:
     """Adapters of projections that read the same (post-dropout) input, stacked: one pass over the
     input gives all their U = Xd A^T (forward) and, with equal scalings, all their dA = s T^T Xd
     (backward).  `cols[i]` is the column range of projection i inside the stacked [M, R] matrices."""
 
-    def __init__(self, projs, dtype, device):
+    def __init__(self, projs, dtype, device, also=()):
         self.R = sum(p.r for p in projs)
         self.K = projs[0].w.K
         self.A_cat = torch.empty((self.R, self.K), dtype=dtype, device=device)
-        self.cols, o = [], 0
+        self.cols, o, items = [], 0, []
         for p in projs:
             self.cols.append((o, o + p.r))
-            p.pack(self.A_cat[o : o + p.r])
+            items.append((p, self.A_cat[o : o + p.r]))
             o += p.r
+        _pack_projs(items + [(p, None) for p in also])
         self.same_s = all(p.s == projs[0].s for p in projs)
 
 
-def _pack_group(projs, Xds, dtype):
-    """Packs the adapters of a group of projections; returns a _Stack when they can share passes
-    over the input (all adapted, one post-dropout input, none act-order, total rank <= 128)."""
+def _pack_group(projs, Xds, dtype, also=()):
+    """Packs the adapters of a group of projections (and of the projections in `also`, in the same
+    launch); returns a _Stack when the group can share passes over the input (all adapted, one
+    post-dropout input, none act-order, total rank <= 128)."""
     live = [p for p in projs if p.r]
     if (len(live) == len(projs) and len(projs) > 1 and all(_same(Xd, Xds[0]) for Xd in Xds)
             and all(p.w.perm is None for p in projs) and sum(p.r for p in projs) <= 128):
-        return _Stack(projs, dtype, Xds[0].device)
-    for p in projs:
-        p.pack()
+        return _Stack(projs, dtype, Xds[0].device, also)
+    _pack_projs([(p, None) for p in list(projs) + list(also)])
     return None
 
 
@@ -266,8 +275,7 @@ def mlp_forward(ctx, X, gate, up, down, dropouts, dtype):
     dropout_gate, dropout_up, dropout_down = dropouts
     X2 = _as2d(X, dtype)
     Xg, Xu = _dropped_inputs(X2, (gate, up), (dropout_gate, dropout_up))
-    stack = _pack_group([gate, up], [Xg, Xu], dtype)
-    down.pack()
+    stack = _pack_group([gate, up], [Xg, Xu], dtype, also=(down,))
     fused = gate.w.perm is None and up.w.perm is None
     if fused:
         Ug, Uu = _lora_down_all([gate, up], [Xg, Xu], stack)

@@ -41,6 +41,7 @@ EXPORTED_SYMBOLS = (
     "fmsa_nf4_dequant",
     "fmsa_nf4_prepare",
     "fmsa_lora_pack",
+    "fmsa_lora_pack_batch",
     "fmsa_rms_layernorm_fwd",
     "fmsa_rms_layernorm_bwd",
     "fmsa_rope_embedding",
@@ -100,6 +101,23 @@ class LoraGradJob(Structure):
         ("transpose_out", c_int32),
         ("out_dtype", c_int32),
         ("reserved", c_int32),
+    ]
+
+
+class LoraPackJob(Structure):
+    """fmsa_lora_pack_job: one adapter of a batched pack."""
+
+    _fields_ = [
+        ("A", c_void_p),
+        ("B", c_void_p),
+        ("A16", c_void_p),
+        ("At16", c_void_p),
+        ("B16", c_void_p),
+        ("Bt16", c_void_p),
+        ("r", c_int32),
+        ("K", c_int32),
+        ("N", c_int32),
+        ("param_dtype", c_int32),
     ]
 
 
@@ -172,6 +190,7 @@ def lib() -> ctypes.CDLL:
     L.fmsa_nf4_prepare.argtypes = [POINTER(Nf4Weight), c_void_p, c_void_p, c_void_p]
     L.fmsa_lora_pack.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p]
+    L.fmsa_lora_pack_batch.argtypes = [POINTER(LoraPackJob), c_int, c_int, c_void_p]
     L.fmsa_rms_layernorm_fwd.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p,
                                          c_int64, c_void_p, c_void_p]
     L.fmsa_rms_layernorm_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
@@ -439,31 +458,47 @@ def nf4_prepare(packed, absmax_q, absmax2, code2, offset: float, shape, blocksiz
     return qweight, block_scale
 
 
+LORA_PACK_MAX_JOBS = 4
+
+
+def lora_pack_batch(adapters, act_dtype):
+    """adapters: (lora_A.weight [r, K], lora_B.weight [N, r], A16_out or None) triples (fp32 / bf16 / fp16
+    parameters).  Returns one (A16 [r, K], At16 [K, r], B16 [N, r], Bt16 [r, N]) per adapter in `act_dtype`,
+    from one launch per LORA_PACK_MAX_JOBS adapters.  `A16_out` (contiguous [r, K]) lets the caller place A16
+    inside a larger stacked matrix."""
+    outs, jobs = [], []
+    for A, B, A16_out in adapters:
+        if not (A.is_cuda and B.is_cuda):
+            raise RuntimeError("fmsa_hip needs GPU tensors")
+        A, B = A.detach(), B.detach()
+        if A.dtype != B.dtype:
+            B = B.to(A.dtype)
+        A = A if A.is_contiguous() else A.contiguous()
+        B = B if B.is_contiguous() else B.contiguous()
+        r, K = A.shape
+        N = B.shape[0]
+        own_a = A16_out is None
+        buf = torch.empty(r * K * (2 if own_a else 1) + 2 * r * N, dtype=act_dtype, device=A.device)
+        o = 0
+        if own_a:
+            A16_out, o = buf[: r * K].view(r, K), r * K
+        assert A16_out.shape == (r, K) and A16_out.is_contiguous() and A16_out.dtype == act_dtype
+        At16 = buf[o : o + r * K].view(K, r)
+        B16 = buf[o + r * K : o + r * K + N * r].view(N, r)
+        Bt16 = buf[o + r * K + N * r :].view(r, N)
+        outs.append((A16_out, At16, B16, Bt16))
+        jobs.append((A, B, LoraPackJob(_ptr(A), _ptr(B), _ptr(A16_out), _ptr(At16), _ptr(B16), _ptr(Bt16), r, K, N,
+                                       _DTYPE_ENUM[A.dtype])))
+    for i in range(0, len(jobs), LORA_PACK_MAX_JOBS):
+        chunk = jobs[i : i + LORA_PACK_MAX_JOBS]
+        arr = (LoraPackJob * len(chunk))(*[j for _, _, j in chunk])
+        _check("fmsa_lora_pack_batch", lib().fmsa_lora_pack_batch(arr, len(chunk), act_enum(act_dtype), _stream(chunk[0][0])))
+    return outs
+
+
 def lora_pack(A, B, act_dtype, A16_out=None):
-    """(A16 [r, K], At16 [K, r], B16 [N, r], Bt16 [r, N]) in `act_dtype` from lora_A.weight [r, K] and
-    lora_B.weight [N, r] (fp32 / bf16 / fp16), one launch.  `A16_out` (contiguous [r, K]) lets the
-    caller place A16 inside a larger stacked matrix."""
-    if not (A.is_cuda and B.is_cuda):
-        raise RuntimeError("fmsa_hip needs GPU tensors")
-    A, B = A.detach(), B.detach()
-    if A.dtype != B.dtype:
-        B = B.to(A.dtype)
-    A = A if A.is_contiguous() else A.contiguous()
-    B = B if B.is_contiguous() else B.contiguous()
-    r, K = A.shape
-    N = B.shape[0]
-    own_a = A16_out is None
-    buf = torch.empty(r * K * (2 if own_a else 1) + 2 * r * N, dtype=act_dtype, device=A.device)
-    o = 0
-    if own_a:
-        A16_out, o = buf[: r * K].view(r, K), r * K
-    assert A16_out.shape == (r, K) and A16_out.is_contiguous() and A16_out.dtype == act_dtype
-    At16 = buf[o : o + r * K].view(K, r)
-    B16 = buf[o + r * K : o + r * K + N * r].view(N, r)
-    Bt16 = buf[o + r * K + N * r :].view(r, N)
-    _check("fmsa_lora_pack", lib().fmsa_lora_pack(_ptr(A), _ptr(B), r, K, N, _DTYPE_ENUM[A.dtype], act_enum(act_dtype),
-                                                  _ptr(A16_out), _ptr(At16), _ptr(B16), _ptr(Bt16), _stream(A)))
-    return A16_out, At16, B16, Bt16
+    """lora_pack_batch for one adapter."""
+    return lora_pack_batch([(A, B, A16_out)], act_dtype)[0]
 
 
 def rms_layernorm_fwd(x2d, weight, eps: float, gemma: bool = False):

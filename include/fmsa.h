@@ -149,6 +149,21 @@ int fmsa_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int 
 int fmsa_lora_pack(const void* A, const void* B, int r, int K, int N, int param_dtype, int act_dtype,
                    void* A16, void* At16, void* B16, void* Bt16, void* stream);
 
+/* The same for up to FMSA_LORA_PACK_MAX_JOBS adapters in one launch (q, k, v; gate, up, down): job q is
+ * fmsa_lora_pack with its fields. */
+#define FMSA_LORA_PACK_MAX_JOBS 4
+typedef struct fmsa_lora_pack_job {
+  const void* A; /* lora_A.weight [r, K] */
+  const void* B; /* lora_B.weight [N, r] */
+  void* A16;     /* [r, K]   (each output may be NULL) */
+  void* At16;    /* [K, r] */
+  void* B16;     /* [N, r] */
+  void* Bt16;    /* [r, N] */
+  int32_t r, K, N;
+  int32_t param_dtype; /* FMSA_F32, FMSA_BF16 or FMSA_F16 */
+} fmsa_lora_pack_job;
+int fmsa_lora_pack_batch(const fmsa_lora_pack_job* jobs, int n_jobs, int act_dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Fused forward:  Y_p = X * deq(W_p) + s_p * U_p * B_p^T (+ bias_p)   for 1..3 projections
  * sharing X (LoRA_W / LoRA_QKV forward, UL/gptq/fast_lora.py:770-805, 497-589), or the

@@ -32,6 +32,7 @@ def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(fmsa_hip.FwdProj) == 128
     assert ctypes.sizeof(fmsa_hip.BwdProj) == 144
     assert ctypes.sizeof(fmsa_hip.LoraGradJob) == 64
+    assert ctypes.sizeof(fmsa_hip.LoraPackJob) == 64
 
 
 def _w(K=64, N=64, gs=64, q=0x1000, s=0x2000, z=0x3000, g=None, zo=0):
@@ -148,6 +149,14 @@ def test_bwd_and_skinny_validation():
     assert gb(two, 2, 8, 1, None, 1 << 20, None) == -6
     assert lib.fmsa_lora_pack(None, 0x1000, 16, 64, 64, 2, 1, None, None, None, None, None) == -1
     assert lib.fmsa_lora_pack(0x1000, 0x2000, 16, 64, 64, 2, 2, None, None, None, None, None) == -4
+    P = fmsa_hip.LoraPackJob
+    pj = lambda **kw: P(**{**dict(A=0x1000, B=0x2000, A16=0x3000, At16=None, B16=None, Bt16=None, r=16, K=64, N=64, param_dtype=2), **kw})
+    pb = lib.fmsa_lora_pack_batch
+    assert pb(None, 1, 1, None) == -1 and pb((P * 1)(pj()), 0, 1, None) == -2 and pb((P * 1)(pj()), 5, 1, None) == -2
+    assert pb((P * 2)(pj(), pj(B=None)), 2, 1, None) == -1
+    assert pb((P * 2)(pj(), pj(N=0)), 2, 1, None) == -2
+    assert pb((P * 2)(pj(), pj(param_dtype=5)), 2, 1, None) == -4
+    assert pb((P * 2)(pj(), pj()), 2, 2, None) == -4          # fp32 is no activation dtype
     assert lib.fmsa_swiglu_fwd(0x1000, 0x2000, 0x3000, 8, 60, 64, 1, None) == -2
     assert lib.fmsa_gptq_permute_rows(0x1000, 0x2000, 64, 64, 0x1000, None) == -5  # in place
 

@@ -119,6 +119,32 @@ def test_lora_grad_batch_equals_separate_calls(dtype):
         assert torch.equal(out, single)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_lora_pack_batch(dtype):
+    """Five adapters of different shapes and parameter types in one call (two launches): every copy is
+    the parameter rounded once to the activation type, A16 of the first three lands inside a stacked
+    matrix."""
+    import fmsa_hip
+
+    shapes = [(16, 2048, 4096, torch.float32), (8, 2048, 1024, torch.float32), (24, 2048, 1024, torch.bfloat16),
+              (64, 1056, 96, torch.float16), (16, 96, 14336, torch.float32)]
+    A_cat = torch.zeros((48, 2048), dtype=dtype, device="cuda")
+    adapters, o = [], 0
+    for i, (r, K, N, pd) in enumerate(shapes):
+        A = dev(randn((r, K), 30 + i, torch.float32)).to(pd)
+        B = dev(randn((N, r), 40 + i, torch.float32)).to(pd)
+        adapters.append((A, B, A_cat[o : o + r] if i < 3 else None))
+        o += r if i < 3 else 0
+    outs = fmsa_hip.lora_pack_batch(adapters, dtype)
+    for (A, B, slot), (A16, At16, B16, Bt16) in zip(adapters, outs):
+        assert torch.equal(A16, A.to(dtype)) and torch.equal(At16, A.to(dtype).t())
+        assert torch.equal(B16, B.to(dtype)) and torch.equal(Bt16, B.to(dtype).t())
+        assert slot is None or A16.data_ptr() == slot.data_ptr()
+        single = fmsa_hip.lora_pack(A, B, dtype)
+        assert all(torch.equal(x, y) for x, y in zip(single, (A16, At16, B16, Bt16)))
+    assert torch.equal(A_cat, torch.cat([a[0].to(dtype) for a in adapters[:3]]))
+
+
 def _fwd_case(M, K, N, gs, r, dtype, s=2.0, bias=False, seed=0):
     w = make_gptq(K, N, gs, seed=seed)
     x = randn((M, K), 2 + seed, dtype)
