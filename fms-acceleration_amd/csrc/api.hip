@@ -91,7 +91,7 @@ const char* fmsa_strerror(int code) {
   }
 }
 
-int fmsa_abi_version(void) { return 3; }
+int fmsa_abi_version(void) { return 4; }
 
 int fmsa_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, void* stream) {
   if (!w || !out) return FMSA_ERR_NULL;
@@ -146,6 +146,8 @@ int fmsa_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int 
   if (!jobs) return FMSA_ERR_NULL;
   if (n_jobs < 1 || n_jobs > FMSA_LORA_GRAD_MAX_JOBS || M <= 0) return FMSA_ERR_SHAPE;
   if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  bool any_t = false;
+  int r_max = 0;
   for (int q = 0; q < n_jobs; ++q) {
     const fmsa_lora_grad_job& j = jobs[q];
     if (!j.L || !j.R || !j.out) return FMSA_ERR_NULL;
@@ -153,7 +155,15 @@ int fmsa_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int 
     if (j.C % 8 != 0 || j.ldr % 8 != 0 || j.ldl % 8 != 0 || j.r % 8 != 0 || j.r > 128) return FMSA_ERR_SHAPE;
     if (j.out_dtype != FMSA_F16 && j.out_dtype != FMSA_BF16 && j.out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
     if (!aligned16(j.R) || !aligned16(j.L)) return FMSA_ERR_ALIGN;
+    if (j.Wt) {
+      if (!j.T) return FMSA_ERR_NULL;
+      if (j.ldt < j.r) return FMSA_ERR_SHAPE;
+      if (!aligned16(j.Wt) || j.ldt % 4 != 0 || (reinterpret_cast<uintptr_t>(j.T) & 7u)) return FMSA_ERR_ALIGN;
+      any_t = true;
+    }
+    r_max = j.r > r_max ? j.r : r_max;
   }
+  if (any_t && r_max > 32) return FMSA_ERR_UNSUPPORTED;
   if (!workspace || workspace_bytes < lora_grad_batch_workspace(jobs, n_jobs, M)) return FMSA_ERR_WORKSPACE;
   if (!aligned16(workspace)) return FMSA_ERR_ALIGN;
   return launch_lora_grad_batch(jobs, n_jobs, M, act_dtype, workspace, (hipStream_t)stream);
@@ -161,7 +171,7 @@ int fmsa_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int 
 
 int fmsa_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale, int transpose_out,
                    int act_dtype, int out_dtype, void* out, void* workspace, size_t workspace_bytes, void* stream) {
-  const fmsa_lora_grad_job job = {L, R, out, ldl, ldr, C, r, scale, transpose_out, out_dtype, 0};
+  const fmsa_lora_grad_job job = {L, R, out, ldl, ldr, C, r, scale, transpose_out, out_dtype, 0, nullptr, nullptr, 0};
   return fmsa_lora_grad_batch(&job, 1, M, act_dtype, workspace, workspace_bytes, stream);
 }
 

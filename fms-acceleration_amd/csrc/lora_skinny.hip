@@ -251,8 +251,8 @@ __global__ __launch_bounds__(512) void lora_down_staged_kernel(const uint16_t* _
 // 32w .. 32w+31 (two 16-wide MFMA tiles) and all r ranks.  Partial sums go to partial[split][r][C]
 // (fp32).  Pass 2 adds the splits in index order, so the result does not depend on scheduling.
 constexpr int LG_TM = 32;               // tokens per tile
-constexpr int LG_TC = 128;              // columns of R per workgroup
-constexpr int LG_RSTRIDE = LG_TC + 16;  // elements: 256 B + 32 B pad
+constexpr int LG_TC = 128;     // columns of R per workgroup (4 waves x 32)
+constexpr int LG_TC_T = 256;   // ... of the flavour that also produces T (8 waves): half as many partial T's
 
 // Several gradients over the same M tokens go out as ONE launch of each pass (the dA of stacked
 // adapters and their dB's; a launch of a small gradient alone neither fills the chip nor hides its
@@ -268,10 +268,15 @@ struct LoraGradJobDev {
   int rblock_start;  // ... in pass 2
   int transpose_out, out_dtype;
   float scale;
+  // optional second product of the same pass over R: T[M, r] = R * Wt^T (see below)
+  const uint16_t* Wt;  // [r, C]
+  float* tpart;        // [column blocks][M][r]
+  uint16_t* T;
+  int64_t ldt;
 };
 struct LoraGradArgs {
   LoraGradJobDev j[FMSA_LORA_GRAD_MAX_JOBS];
-  int n_jobs, M;
+  int n_jobs, M, act_dtype;
 };
 // the job that owns workgroup `block` (wave-uniform), copied field by field: indexing the
 // kernel-argument struct with a runtime value would force a copy of it into scratch memory
@@ -284,11 +289,23 @@ FMSA_DEVI LoraGradJobDev select_job(const LoraGradArgs& a, int block) {
   return J;
 }
 
-template <typename T, int RT>
-__global__ __launch_bounds__(256) void lora_grad_partial_kernel(const LoraGradArgs a) {
+// WITH_T: a job with Wt set also produces T = R * Wt^T (the `dY @ B` every backward needs next to
+// dB = s * dY^T U: both read dY, which is the whole cost of either).  The R tile is in LDS anyway, and
+// row-major, which is the natural MFMA layout for a contraction over columns: wave w multiplies the
+// tile's 32 tokens by its own 32 columns (2 * rt MFMAs per tile), the four waves' partial tiles meet in
+// LDS and are summed in wave order by the whole workgroup one iteration later (behind the barrier the
+// loop has anyway), and leave as the column block's partial T[column block][token][rank] (fp32).  The
+// reduce pass adds the column blocks in index order and rounds once: deterministic like the rest.
+template <typename T, int RT, bool WITH_T>
+__global__ __launch_bounds__(WITH_T ? 512 : 256) void lora_grad_partial_kernel(const LoraGradArgs a) {
+  constexpr int NWV = WITH_T ? 8 : 4;       // waves
+  constexpr int NTH = 64 * NWV;             // threads
+  constexpr int TC = 32 * NWV;              // columns of R per workgroup
+  constexpr int LG_RSTRIDE = TC + 16;       // elements: row + 32 B pad
   constexpr int LSTRIDE = (RT == 1) ? 16 : RT * 16 + 16;  // elements; row pitch = 8 banks mod 32
   __shared__ __attribute__((aligned(16))) uint16_t r_lds[2][LG_TM * LG_RSTRIDE];
   __shared__ __attribute__((aligned(16))) uint16_t l_lds[2][LG_TM * LSTRIDE];
+  __shared__ __attribute__((aligned(16))) float t_lds[WITH_T ? 2 : 1][WITH_T ? NWV : 1][2][WITH_T ? RT : 1][64][WITH_T ? 4 : 1];
   const LoraGradJobDev J = select_job<false>(a, blockIdx.x);
   const uint16_t* __restrict__ L = J.L;
   const uint16_t* __restrict__ R = J.R;
@@ -296,28 +313,28 @@ __global__ __launch_bounds__(256) void lora_grad_partial_kernel(const LoraGradAr
   const int64_t ldl = J.ldl, ldr = J.ldr;
   const int M = a.M, C = J.C, r = J.r, rows_per_split = J.rows_per_split;
   const int rt = (r + 15) / 16;  // 16-rank tiles this job uses of the RT the launch is built for
-  const int ncb = (C + LG_TC - 1) / LG_TC;
+  const int ncb = (C + TC - 1) / TC;
   const int local = blockIdx.x - J.block_start;
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int l16 = lane & 15, kg = lane >> 4;
   const int split = local / ncb;
-  const int c0 = (local % ncb) * LG_TC;
+  const int c0 = (local % ncb) * TC;
   const int m_begin = split * rows_per_split;
   const int m_end = min(M, m_begin + rows_per_split);
   const int n_tiles = (m_end - m_begin + LG_TM - 1) / LG_TM;
 
-  // global -> LDS assignment: R tile = 32 rows x 16 chunks of 16 B -> 2 chunks per thread;
-  // L tile = 32 rows x (RT*2) chunks = 64*RT chunks -> LP per thread (chunk tid + 256*p), threads
+  // global -> LDS assignment: R tile = 32 rows x TC/8 chunks of 16 B -> 2 chunks per thread (16 rows per pass);
+  // L tile = 32 rows x (RT*2) chunks = 64*RT chunks -> LP per thread (chunk tid + NTH*p), threads
   // past the last chunk idle
-  const int r_row = tid >> 4, r_chunk = tid & 15;
+  const int r_row = tid / (TC / 8), r_chunk = tid % (TC / 8);
   const bool r_col_ok = (c0 + 8 * r_chunk) < C;  // C % 8 == 0
-  constexpr int LP = (64 * RT + 255) / 256;
+  constexpr int LP = (64 * RT + NTH - 1) / NTH;
   int l_row[LP], l_chunk[LP];
   bool l_thread[LP], l_col_ok[LP];
 #pragma unroll
   for (int p = 0; p < LP; ++p) {
-    const int ci = tid + 256 * p;
+    const int ci = tid + NTH * p;
     l_row[p] = ci / (2 * RT);
     l_chunk[p] = ci % (2 * RT);
     l_thread[p] = ci < 64 * RT;
@@ -366,6 +383,35 @@ __global__ __launch_bounds__(256) void lora_grad_partial_kernel(const LoraGradAr
 #pragma unroll
     for (int t = 0; t < RT; ++t) acc[g][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // T product: this lane's Wt fragments (rank 16t + l16, columns c0 + 32*wave + 8*kg ..), fixed for the workgroup
+  const bool with_t = WITH_T && J.Wt != nullptr;
+  u32x4 wtf[RT];
+  if constexpr (WITH_T) {
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      wtf[t] = u32x4{0u, 0u, 0u, 0u};
+      const int j = 16 * t + l16, c = c0 + 32 * wave + 8 * kg;
+      if (with_t && j < r && c < C) wtf[t] = *reinterpret_cast<const u32x4*>(J.Wt + (size_t)j * C + c);
+    }
+  }
+  // sums the four waves' partial T tiles of token tile `tile` (parked in t_lds[tile & 1]) and stores them
+  auto flush_t = [&](int tile) {
+    if constexpr (WITH_T) {
+      if (!with_t) return;
+      const int tb = tile & 1;
+      const int m0 = m_begin + tile * LG_TM;
+      float* dst = J.tpart + ((size_t)(local % ncb) * M) * r;
+      for (int v = tid; v < LG_TM * 16 * RT; v += NTH) {
+        const int j = v % (16 * RT), m = v / (16 * RT);
+        const int u = m >> 4, ln = ((m & 15) >> 2) * 16 + (j & 15), i = m & 3, t = j >> 4;
+        float sum = t_lds[tb][0][u][t][ln][i];
+#pragma unroll
+        for (int w = 1; w < NWV; ++w) sum += t_lds[tb][w][u][t][ln][i];
+        if (m0 + m < m_end && j < r) dst[(size_t)(m0 + m) * r + j] = sum;
+      }
+    }
+  };
+
   if (n_tiles > 0) {
     load_tile(0);
     commit_tile(0);
@@ -374,6 +420,19 @@ __global__ __launch_bounds__(256) void lora_grad_partial_kernel(const LoraGradAr
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int buf = tile & 1;
     if (tile + 1 < n_tiles) load_tile(tile + 1);
+    if (tile > 0) flush_t(tile - 1);
+    if constexpr (WITH_T) {
+      if (with_t) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const u32x4 yf = *reinterpret_cast<const u32x4*>(&r_lds[buf][(16 * u + l16) * LG_RSTRIDE + 32 * wave + 8 * kg]);
+#pragma unroll
+          for (int t = 0; t < RT; ++t)
+            if (t < rt)
+              *reinterpret_cast<f32x4*>(t_lds[buf][wave][u][t][lane]) = mfma16<T>(yf, wtf[t], f32x4{0.f, 0.f, 0.f, 0.f});  // D[token][rank]
+        }
+      }
+    }
     u32x4 lf[RT], rf[2];
 #pragma unroll
     for (int t = 0; t < RT; ++t)
@@ -389,6 +448,7 @@ __global__ __launch_bounds__(256) void lora_grad_partial_kernel(const LoraGradAr
     if (tile + 1 < n_tiles) commit_tile(buf ^ 1);
     __syncthreads();
   }
+  if (n_tiles > 0) flush_t(n_tiles - 1);
   // lane holds D[c = 4*kg + i][j = l16]: four consecutive columns -> one 16-byte store
 #pragma unroll
   for (int g = 0; g < 2; ++g) {
@@ -412,7 +472,22 @@ __global__ __launch_bounds__(256) void lora_grad_partial_kernel(const LoraGradAr
 __global__ __launch_bounds__(256) void lora_grad_reduce_kernel(const LoraGradArgs a) {
   const LoraGradJobDev J = select_job<true>(a, blockIdx.x);
   const int r = J.r, C = J.C;
-  const int idx = (blockIdx.x - J.rblock_start) * 256 + threadIdx.x;  // over r*C, c fastest
+  const int nb_grad = (r * C + 255) / 256;
+  const int lb = blockIdx.x - J.rblock_start;
+  if (lb >= nb_grad) {  // the job's T: column blocks added in index order, one rounding; four ranks per thread
+    const int64_t ti = ((int64_t)(lb - nb_grad) * 256 + threadIdx.x) * 4;
+    if (ti >= (int64_t)a.M * r) return;  // r % 8 == 0: the four stay inside one token's row
+    const int m = (int)(ti / r), j = (int)(ti % r);
+    const int ncb = (C + LG_TC_T - 1) / LG_TC_T;
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    for (int cb = 0; cb < ncb; ++cb) v += *reinterpret_cast<const f32x4*>(J.tpart + ((size_t)cb * a.M + m) * r + j);
+    u32x2 pk;
+    pk[0] = a.act_dtype == FMSA_BF16 ? pack2<bf16_t>(v[0], v[1]) : pack2<f16_t>(v[0], v[1]);
+    pk[1] = a.act_dtype == FMSA_BF16 ? pack2<bf16_t>(v[2], v[3]) : pack2<f16_t>(v[2], v[3]);
+    *reinterpret_cast<u32x2*>(J.T + (size_t)m * J.ldt + j) = pk;
+    return;
+  }
+  const int idx = lb * 256 + threadIdx.x;  // over r*C, c fastest
   if (idx >= r * C) return;
   const int j = idx / C, c = idx % C;
   float v = 0.f;
@@ -497,10 +572,18 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
   return FMSA_OK;
 }
 
+namespace {
+size_t job_partial_bytes(const fmsa_lora_grad_job& s, int M) {
+  return (size_t)lora_grad_splits(M, s.C) * (size_t)s.r * (size_t)s.C * sizeof(float);
+}
+size_t job_tpart_bytes(const fmsa_lora_grad_job& s, int M) {
+  return s.Wt ? (size_t)((s.C + LG_TC_T - 1) / LG_TC_T) * (size_t)M * (size_t)s.r * sizeof(float) : 0;
+}
+}  // namespace
+
 size_t lora_grad_batch_workspace(const fmsa_lora_grad_job* jobs, int n_jobs, int M) {
   size_t bytes = 0;
-  for (int q = 0; q < n_jobs; ++q)
-    bytes += (size_t)lora_grad_splits(M, jobs[q].C) * (size_t)jobs[q].r * (size_t)jobs[q].C * sizeof(float);
+  for (int q = 0; q < n_jobs; ++q) bytes += job_partial_bytes(jobs[q], M) + job_tpart_bytes(jobs[q], M);
   return bytes;
 }
 
@@ -508,6 +591,10 @@ int launch_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, in
   LoraGradArgs a{};
   a.n_jobs = n_jobs;
   a.M = M;
+  a.act_dtype = act_dtype;
+  bool any_t = false;
+  for (int q = 0; q < n_jobs; ++q) any_t = any_t || jobs[q].Wt != nullptr;
+  const int tc = any_t ? LG_TC_T : LG_TC;  // the launch's flavour decides the column-block width of all its jobs
   int blocks = 0, rblocks = 0, r_max = 0;
   size_t ws_off = 0;
   for (int q = 0; q < n_jobs; ++q) {
@@ -529,20 +616,28 @@ int launch_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, in
     d.transpose_out = s.transpose_out;
     d.out_dtype = s.out_dtype;
     d.scale = s.scale;
-    blocks += ((s.C + LG_TC - 1) / LG_TC) * d.splits;
+    blocks += ((s.C + tc - 1) / tc) * d.splits;
     rblocks += (s.r * s.C + 255) / 256;
-    ws_off += (size_t)d.splits * s.r * s.C * sizeof(float);
+    ws_off += job_partial_bytes(s, M);
+    if (s.Wt) {
+      d.Wt = (const uint16_t*)s.Wt;
+      d.T = (uint16_t*)s.T;
+      d.ldt = s.ldt;
+      d.tpart = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + ws_off);
+      ws_off += job_tpart_bytes(s, M);
+      rblocks += (int)(((int64_t)M * s.r / 4 + 255) / 256);
+    }
     r_max = s.r > r_max ? s.r : r_max;
   }
-  dim3 grid1(blocks), grid2(rblocks), block(256);
+  dim3 grid1(blocks), grid2(rblocks), block(256), block1(any_t ? 512 : 256);
   const int rt = (r_max + 15) / 16;
-#define LAUNCH(TT, RT) hipLaunchKernelGGL((lora_grad_partial_kernel<TT, RT>), grid1, block, 0, st, a)
-#define DISPATCH(TT)                      \
-  switch (rt) {                           \
-    case 1: LAUNCH(TT, 1); break;         \
-    case 2: LAUNCH(TT, 2); break;         \
-    case 3: case 4: LAUNCH(TT, 4); break; \
-    default: LAUNCH(TT, 8); break;        \
+#define LAUNCH(TT, RT, WT) hipLaunchKernelGGL((lora_grad_partial_kernel<TT, RT, WT>), grid1, block1, 0, st, a)
+#define DISPATCH(TT)                                                  \
+  switch (rt) {                                                       \
+    case 1: if (any_t) LAUNCH(TT, 1, true); else LAUNCH(TT, 1, false); break; \
+    case 2: if (any_t) LAUNCH(TT, 2, true); else LAUNCH(TT, 2, false); break; \
+    case 3: case 4: LAUNCH(TT, 4, false); break;                      \
+    default: LAUNCH(TT, 8, false); break;                             \
   }
   if (act_dtype == FMSA_BF16) {
     DISPATCH(bf16_t)

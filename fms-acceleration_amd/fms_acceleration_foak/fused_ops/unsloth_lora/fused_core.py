@@ -106,6 +106,32 @@ class _Proj:
                                            (U, dY2, self.s, True, self.B_param.dtype)])
         return dA, dB
 
+    def t_and_grads(self, Xd, U, dY2):
+        """(T = dY B, dA, dB).  Where it pays, T and dB come from one pass over dY and dA from a second launch
+        that reads T; otherwise T from its own pass and both gradients from one launch."""
+        if not self.r:
+            return None, None, None
+        if not _fuse_t([self], [dY2]):
+            T = fmsa_hip.lora_down(dY2, self.Bt)
+            return (T,) + self.lora_grads(T, Xd, U, dY2)
+        T = torch.empty((dY2.shape[0], self.r), dtype=dY2.dtype, device=dY2.device)
+        (dB,) = fmsa_hip.lora_grad_batch([(U, dY2, self.s, True, self.B_param.dtype, self.Bt, T)])
+        (dA,) = fmsa_hip.lora_grad_batch([(T, Xd, self.s, False, self.A_param.dtype)])
+        return T, dA, dB
+
+
+FUSE_T_MIN_BYTES = 96 << 20
+
+
+def _fuse_t(projs, dYs):
+    """Whether T_p = dY_p B_p should come out of the dB launch (one pass over dY_p instead of two).  The
+    dependent dA launch then cannot share the dB launch any more, which costs about 15 us of launch ramp
+    and tail: measured to pay from about 100 MB of dY (q, k, v together; gate and up), not for one
+    4096-wide projection."""
+    if any(p.r > fmsa_hip.LORA_GRAD_T_MAX_RANK for p in projs):
+        return False
+    return sum(dY.numel() * dY.element_size() for dY in dYs) >= FUSE_T_MIN_BYTES
+
 
 def _pack_projs(items):
     """items: (projection, A16_out or None).  One launch packs the adapters of all of them."""
@@ -171,23 +197,28 @@ def _adapter_grads(projs, dYs, Xds, Us, stack):
     if stack is not None:
         M = dYs[0].shape[0]
         T_cat = torch.empty((M, stack.R), dtype=dYs[0].dtype, device=dYs[0].device)
-        Ts = [fmsa_hip.lora_down(dY, p.Bt, out=T_cat[:, a:b]) for p, dY, (a, b) in zip(projs, dYs, stack.cols)]
-        # every gradient of the group in one launch of each pass
+        Ts = [T_cat[:, a:b] for a, b in stack.cols]
+        # one launch: every dB, and with it (same pass over dY) every T; a second one: every dA, which reads the T's
         stacked_dA = stack.same_s and all(p.A_param.dtype == projs[0].A_param.dtype for p in projs)
-        if stacked_dA:
-            jobs = [(T_cat, Xds[0], projs[0].s, False, projs[0].A_param.dtype)]
+        dA_jobs = ([(T_cat, Xds[0], projs[0].s, False, projs[0].A_param.dtype)] if stacked_dA else
+                   [(T, Xds[0], p.s, False, p.A_param.dtype) for p, T in zip(projs, Ts)])
+        if _fuse_t(projs, dYs):
+            dBs = fmsa_hip.lora_grad_batch([(U, dY, p.s, True, p.B_param.dtype, p.Bt, T)
+                                            for p, dY, U, T in zip(projs, dYs, Us, Ts)])
+            dAs = fmsa_hip.lora_grad_batch(dA_jobs)
         else:
-            jobs = [(T, Xds[0], p.s, False, p.A_param.dtype) for p, T in zip(projs, Ts)]
-        n_dA = len(jobs)
-        jobs += [(U, dY, p.s, True, p.B_param.dtype) for p, dY, U in zip(projs, dYs, Us)]
-        outs = fmsa_hip.lora_grad_batch(jobs)
-        dAs = [outs[0][a:b] for a, b in stack.cols] if stacked_dA else outs[:n_dA]
-        return Ts, list(zip(dAs, outs[n_dA:]))
+            for p, dY, T in zip(projs, dYs, Ts):
+                fmsa_hip.lora_down(dY, p.Bt, out=T)
+            outs = fmsa_hip.lora_grad_batch(dA_jobs + [(U, dY, p.s, True, p.B_param.dtype) for p, dY, U in zip(projs, dYs, Us)])
+            dAs, dBs = outs[: len(dA_jobs)], outs[len(dA_jobs) :]
+        if stacked_dA:
+            dAs = [dAs[0][a:b] for a, b in stack.cols]
+        return Ts, list(zip(dAs, dBs))
     Ts, grads = [], []
     for p, dY, Xd, U in zip(projs, dYs, Xds, Us):
-        T = fmsa_hip.lora_down(dY, p.Bt) if p.r else None
+        T, dA, dB = p.t_and_grads(Xd, U, dY)
         Ts.append(T)
-        grads.append(p.lora_grads(T, Xd, U, dY))
+        grads.append((dA, dB))
     return Ts, grads
 
 
@@ -230,8 +261,7 @@ def w_backward(ctx, dY):
     T = Xd = None
     if p.r:
         Xd, U = ctx.saved_tensors
-        T = fmsa_hip.lora_down(dY2, p.Bt)
-        dA, dB = p.lora_grads(T, Xd, U, dY2)
+        T, dA, dB = p.t_and_grads(Xd, U, dY2)
     dX = _linear_backward_dx([p], [dY2], [T], [Xd], M, K)
     return dX.view(ctx.x_shape).to(ctx.x_dtype), dA, dB
 
@@ -302,7 +332,15 @@ def mlp_backward(ctx, dY):
     M, H, I = dY2.shape[0], gate.w.K, down.w.K
 
     # ---- down projection: dh, then SwiGLU backward in place (e <- d_g, g <- d_e) -----------
-    Td = fmsa_hip.lora_down(dY2, down.Bt) if down.r else None
+    # T_d = dY B_d is needed by the dh launch; dB_d = s dY^T U_d shares its pass over dY unless U_d has to be
+    # re-formed from the recomputed h (dropout on h), which exists only after that launch
+    Td = dAd = dBd = None
+    if down.r:
+        if ctx.down_dropped or not _fuse_t([down], [dY2]):
+            Td = fmsa_hip.lora_down(dY2, down.Bt)
+        else:
+            Td = torch.empty((M, down.r), dtype=dY2.dtype, device=dY2.device)
+            (dBd,) = fmsa_hip.lora_grad_batch([(Ud, dY2, down.s, True, down.B_param.dtype, down.Bt, Td)])
     mask_h = hd if ctx.down_dropped else None
     if down.w.perm is None:
         h = fmsa_hip.gptq_lora_bwd_dx([down.bwd_dict(dY2, Td, mask_h)], M, I, fmsa_hip.BWD_SWIGLU, e=e, g=g)
@@ -314,11 +352,13 @@ def mlp_backward(ctx, dY):
             fmsa_hip.gptq_lora_bwd_dx([down.bwd_dict(dY2, Td, mask_h if mask_h is not None else h_now)], M, I))
         h = fmsa_hip.swiglu_bwd(dh, e, g)
     d_g, d_e = e, g
-    dAd = dBd = None
     if down.r:
         # the reference forms both down-projection grads from the recomputed h (gptq/fast_lora.py:369-370)
-        Ud_b = fmsa_hip.lora_down(h, down.A) if ctx.down_dropped else Ud
-        dAd, dBd = down.lora_grads(Td, h, Ud_b, dY2)
+        if dBd is None:
+            Ud_b = fmsa_hip.lora_down(h, down.A) if ctx.down_dropped else Ud
+            dAd, dBd = down.lora_grads(Td, h, Ud_b, dY2)
+        else:
+            (dAd,) = fmsa_hip.lora_grad_batch([(Td, h, down.s, False, down.A_param.dtype)])
 
     # ---- up / gate: adapter grads, then dX over the concatenated contraction ---------------
     (Tg, Tu), ((dAg, dBg), (dAu, dBu)) = _adapter_grads([gate, up], [d_e, d_g], [Xg, Xu], [Ug, Uu], ctx.stack)

@@ -101,6 +101,9 @@ class LoraGradJob(Structure):
         ("transpose_out", c_int32),
         ("out_dtype", c_int32),
         ("reserved", c_int32),
+        ("Wt", c_void_p),
+        ("T", c_void_p),
+        ("ldt", c_int64),
     ]
 
 
@@ -340,23 +343,32 @@ def lora_grad(L, R, scale: float, transpose_out: bool, out_dtype=torch.float32):
 LORA_GRAD_MAX_JOBS = 8
 
 
+LORA_GRAD_T_MAX_RANK = 32  # fmsa_lora_grad_batch computes T next to the gradient only up to this rank
+
+
 def lora_grad_batch(jobs):
-    """jobs: (L, R, scale, transpose_out, out_dtype) tuples over the same M tokens; returns the list of
-    scale * L^T @ R, each as lora_grad would give it, from one launch of each pass per
-    LORA_GRAD_MAX_JOBS jobs."""
+    """jobs: (L, R, scale, transpose_out, out_dtype[, Wt, T_out]) tuples over the same M tokens; returns
+    the list of scale * L^T @ R, each as lora_grad would give it, from one launch of each pass per
+    LORA_GRAD_MAX_JOBS jobs.  A job with Wt [r, C] and T_out [M, r] (may be a column slice) also gets
+    T_out = R @ Wt^T from the same pass over R (all ranks of such a call <= LORA_GRAD_T_MAX_RANK)."""
     outs = []
     for i in range(0, len(jobs), LORA_GRAD_MAX_JOBS):
         chunk = jobs[i : i + LORA_GRAD_MAX_JOBS]
         M = chunk[0][0].shape[0]
         arr = (LoraGradJob * len(chunk))()
-        for q, (L, R, scale, tr, out_dtype) in enumerate(chunk):
+        for q, job in enumerate(chunk):
+            L, R, scale, tr, out_dtype = job[:5]
+            Wt, T_out = job[5:7] if len(job) > 5 else (None, None)
             r, C = L.shape[1], R.shape[1]
             assert L.shape[0] == M and R.shape[0] == M and L.stride(1) == 1 and R.stride(1) == 1
             assert L.dtype == R.dtype == chunk[0][1].dtype
+            if Wt is not None:
+                assert Wt.shape == (r, C) and Wt.is_contiguous() and Wt.dtype == R.dtype
+                assert T_out.shape == (M, r) and T_out.stride(1) == 1 and T_out.dtype == R.dtype
             out = torch.empty((C, r) if tr else (r, C), dtype=out_dtype, device=R.device)
             outs.append(out)
             arr[q] = LoraGradJob(_ptr(L), _ptr(R), _ptr(out), L.stride(0), R.stride(0), C, r, float(scale), int(tr),
-                                 _DTYPE_ENUM[out_dtype], 0)
+                                 _DTYPE_ENUM[out_dtype], 0, _ptr(Wt), _ptr(T_out), 0 if T_out is None else T_out.stride(0))
         R0 = chunk[0][1]
         ws = _workspace(lib().fmsa_lora_grad_batch_workspace(arr, len(chunk), M), R0.device)
         _check("fmsa_lora_grad_batch",

@@ -136,6 +136,15 @@ typedef struct fmsa_lora_grad_job {
   int32_t transpose_out;
   int32_t out_dtype; /* FMSA_F32, FMSA_BF16 or FMSA_F16 */
   int32_t reserved;
+  /* Optional second product of the same pass over R:  T[M, r] = R * Wt^T  in act_dtype, row stride ldt
+   * (what fmsa_lora_down(R, Wt) gives, up to the order of the fp32 sums).  A backward needs both
+   * dB = s * dY^T U (this job: L = U, R = dY) and T = dY B (Wt = lora_B.weight^T [r, C]),
+   * UL/gptq/fast_lora.py:822-823, and reading dY is the whole cost of either.  Wt == NULL: no T.
+   * With Wt set every job of the call needs r <= 32; T 8-byte aligned, ldt % 4 == 0.  Worth it when the pass
+   * over R it saves (2 * M * C bytes) outweighs the second launch the dependent dA then needs. */
+  const void* Wt;
+  void* T;
+  int64_t ldt;
 } fmsa_lora_grad_job;
 size_t fmsa_lora_grad_batch_workspace(const fmsa_lora_grad_job* jobs, int n_jobs, int M);
 int fmsa_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int act_dtype, void* workspace,

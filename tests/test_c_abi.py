@@ -31,7 +31,7 @@ def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(fmsa_hip.GptqWeight) == 72
     assert ctypes.sizeof(fmsa_hip.FwdProj) == 128
     assert ctypes.sizeof(fmsa_hip.BwdProj) == 144
-    assert ctypes.sizeof(fmsa_hip.LoraGradJob) == 64
+    assert ctypes.sizeof(fmsa_hip.LoraGradJob) == 88
     assert ctypes.sizeof(fmsa_hip.LoraPackJob) == 64
 
 
@@ -132,7 +132,7 @@ def test_bwd_and_skinny_validation():
     assert lib.fmsa_lora_grad(0x1000, 16, 0x2000, 64, 8, 64, 16, 1.0, 0, 1, 2, 0x3000, None, 0, None) == -6
     J = fmsa_hip.LoraGradJob
     job = lambda **kw: J(**{**dict(L=0x1000, R=0x2000, out=0x3000, ldl=16, ldr=64, C=64, r=16, scale=1.0, transpose_out=0,
-                                   out_dtype=2, reserved=0), **kw})
+                                   out_dtype=2, reserved=0, Wt=None, T=None, ldt=0), **kw})
     gb, gw = lib.fmsa_lora_grad_batch, lib.fmsa_lora_grad_batch_workspace
     two = (J * 2)(job(), job(C=128, ldr=128, r=8))
     assert gw(two, 2, 8) == lib.fmsa_lora_grad_workspace(8, 64, 16) + lib.fmsa_lora_grad_workspace(8, 128, 8)
@@ -146,6 +146,12 @@ def test_bwd_and_skinny_validation():
     assert gb((J * 2)(job(), job(out_dtype=7)), 2, 8, 1, 0x4000, 1 << 20, None) == -4
     assert gb((J * 2)(job(), job(L=0x1004)), 2, 8, 1, 0x4000, 1 << 20, None) == -3
     assert gb(two, 2, 8, 1, 0x4000, gw(two, 2, 8) - 1, None) == -6             # workspace one byte short
+    with_t = (J * 1)(job(Wt=0x5000, T=0x6000, ldt=16))
+    assert gw(with_t, 1, 8) == lib.fmsa_lora_grad_workspace(8, 64, 16) + 1 * 8 * 16 * 4   # + one column block of partial T
+    assert gb((J * 1)(job(Wt=0x5000, T=None, ldt=16)), 1, 8, 1, 0x4000, 1 << 20, None) == -1
+    assert gb((J * 1)(job(Wt=0x5000, T=0x6000, ldt=8)), 1, 8, 1, 0x4000, 1 << 20, None) == -2
+    assert gb((J * 1)(job(Wt=0x5004, T=0x6000, ldt=16)), 1, 8, 1, 0x4000, 1 << 20, None) == -3
+    assert gb((J * 2)(job(Wt=0x5000, T=0x6000, ldt=16), job(r=64, ldl=64)), 2, 8, 1, 0x4000, 1 << 20, None) == -5  # T only up to rank 32
     assert gb(two, 2, 8, 1, None, 1 << 20, None) == -6
     assert lib.fmsa_lora_pack(None, 0x1000, 16, 64, 64, 2, 1, None, None, None, None, None) == -1
     assert lib.fmsa_lora_pack(0x1000, 0x2000, 16, 64, 64, 2, 2, None, None, None, None, None) == -4

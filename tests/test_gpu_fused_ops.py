@@ -16,6 +16,17 @@ def _q(t, dtype):
     return t.to(dtype).float()
 
 
+@pytest.fixture(params=["own_pass", "with_dB"], autouse=True)
+def t_product_route(request, monkeypatch):
+    """The backward forms T = dY B either in its own pass over dY or inside the dB launch (the route large
+    shapes take): every test of this file runs both ways."""
+    from fms_acceleration_foak.fused_ops.unsloth_lora import fused_core
+
+    if request.param == "with_dB":
+        monkeypatch.setattr(fused_core, "FUSE_T_MIN_BYTES", 0)
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("act_order", [False, True])
 @pytest.mark.parametrize("B_,S_,K,N,r", [(1, 128, 2048, 2048, 8), (2, 256, 512, 1024, 16), (3, 50, 256, 96, 32)])

@@ -120,6 +120,38 @@ def test_lora_grad_batch_equals_separate_calls(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_lora_grad_batch_with_T(dtype):
+    """Jobs that also produce T = R @ Wt^T from the same pass over R: ragged token / column counts (last
+    token tile of 23 rows, last column block of 8 columns), T written as a column slice of a stacked
+    matrix, ranks 8 / 16 / 32, next to a job without T.  T against the fp32 product and against
+    lora_down (same rounding point, other order of the sums); the gradients bit for bit as without T."""
+    import fmsa_hip
+
+    M = 2327
+    shapes = [(4104, 16, True), (1056, 8, False), (136, 32, True), (2048, 16, True)]
+    T_cat = torch.full((M, 80), 3.0, dtype=dtype, device="cuda")
+    jobs, o = [], 0
+    for i, (C, r, tr) in enumerate(shapes):
+        L, R, Wt = dev(randn((M, r), 110 + i, dtype)), dev(randn((M, C), 120 + i, dtype)), dev(randn((r, C), 130 + i, dtype, 0.05))
+        with_t = i != 1
+        jobs.append((L, R, 0.5, tr, torch.float32) + ((Wt, T_cat[:, o : o + r]) if with_t else ()))
+        o += r if with_t else 0
+    outs = fmsa_hip.lora_grad_batch(jobs)
+    assert torch.all(T_cat[:, o:] == 3.0)
+    for job, out in zip(jobs, outs):
+        L, R, scale, tr, od = job[:5]
+        assert torch.equal(out, fmsa_hip.lora_grad(L, R, scale, tr, od))
+        if len(job) > 5:
+            Wt, T = job[5:]
+            ref = R.float() @ Wt.float().t()
+            assert olora.max_rel_err(T.float().cpu(), ref.cpu()) < 5e-3
+            assert olora.max_rel_err(T.float().cpu(), fmsa_hip.lora_down(R, Wt).float().cpu()) < 5e-3
+    T_first = T_cat.clone()
+    fmsa_hip.lora_grad_batch(jobs)
+    assert torch.equal(T_cat, T_first)  # run-to-run bit-stable
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_lora_pack_batch(dtype):
     """Five adapters of different shapes and parameter types in one call (two launches): every copy is
     the parameter rounded once to the activation type, A16 of the first three lands inside a stacked
