@@ -479,8 +479,20 @@ __global__ __launch_bounds__(256) void lora_grad_reduce_kernel(const LoraGradArg
     if (ti >= (int64_t)a.M * r) return;  // r % 8 == 0: the four stay inside one token's row
     const int m = (int)(ti / r), j = (int)(ti % r);
     const int ncb = (C + LG_TC_T - 1) / LG_TC_T;
+    // eight loads in flight per thread (a plain loop waits for each load before it issues the next); the sum
+    // itself stays in index order
+    const float* src = J.tpart + (size_t)m * r + j;
+    const size_t step = (size_t)a.M * r;
     f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    for (int cb = 0; cb < ncb; ++cb) v += *reinterpret_cast<const f32x4*>(J.tpart + ((size_t)cb * a.M + m) * r + j);
+    int cb = 0;
+    for (; cb + 8 <= ncb; cb += 8) {
+      f32x4 p[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) p[k] = *reinterpret_cast<const f32x4*>(src + (size_t)(cb + k) * step);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v += p[k];
+    }
+    for (; cb < ncb; ++cb) v += *reinterpret_cast<const f32x4*>(src + (size_t)cb * step);
     u32x2 pk;
     pk[0] = a.act_dtype == FMSA_BF16 ? pack2<bf16_t>(v[0], v[1]) : pack2<f16_t>(v[0], v[1]);
     pk[1] = a.act_dtype == FMSA_BF16 ? pack2<bf16_t>(v[2], v[3]) : pack2<f16_t>(v[2], v[3]);
@@ -490,8 +502,18 @@ __global__ __launch_bounds__(256) void lora_grad_reduce_kernel(const LoraGradArg
   const int idx = lb * 256 + threadIdx.x;  // over r*C, c fastest
   if (idx >= r * C) return;
   const int j = idx / C, c = idx % C;
+  const float* src = J.partial + (size_t)j * C + c;
+  const size_t step = (size_t)r * C;
   float v = 0.f;
-  for (int sp = 0; sp < J.splits; ++sp) v += J.partial[((size_t)sp * r + j) * C + c];
+  int sp = 0;
+  for (; sp + 8 <= J.splits; sp += 8) {  // eight loads in flight, summed in index order
+    float p[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) p[k] = src[(size_t)(sp + k) * step];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v += p[k];
+  }
+  for (; sp < J.splits; ++sp) v += src[(size_t)sp * step];
   v *= J.scale;
   const size_t o = J.transpose_out ? ((size_t)c * r + j) : (size_t)idx;
   if (J.out_dtype == FMSA_F32)
