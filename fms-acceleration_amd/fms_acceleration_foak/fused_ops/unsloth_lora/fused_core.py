@@ -88,13 +88,23 @@ class _Proj:
     def fwd_dict(self, U):
         return {"w": self.w.struct, "U": U, "B": self.B, "bias": self.bias, "r": self.r, "s": self.s}
 
-    def bwd_dict(self, dY2, T, mask_src):
+    def bwd_dict(self, dY2, T, mask_src, permuted=None):
+        """`permuted`: dict shared by the projections of one launch, so that a mask source they have in common
+        is brought into kernel order once."""
         At = None
         if self.r:
             At = self.At  # [K, r]
             if self.w.perm is not None:
                 At = At[self.w.perm.long()].contiguous()
-                mask_src = None if mask_src is None else fmsa_hip.permute_cols(mask_src, self.w.perm, gather=True)
+                if mask_src is not None:
+                    key = (id(mask_src), self.w.perm_key)
+                    if permuted is not None and key in permuted:
+                        mask_src = permuted[key][1]
+                    else:
+                        pm = fmsa_hip.permute_cols(mask_src, self.w.perm, gather=True)
+                        if permuted is not None:
+                            permuted[key] = (mask_src, pm)  # holds the source too: its id stays taken
+                        mask_src = pm
         return {"w": self.w.struct, "nsz": self.w.nsz, "dY": dY2, "T": T, "At": At, "mask_src": mask_src if self.r else None,
                 "r": self.r, "s": self.s}
 
@@ -160,13 +170,20 @@ class _Stack:
         self.same_s = all(p.s == projs[0].s for p in projs)
 
 
+def _one_order(projs):
+    """All projections walk K in the same order (none act-order, or act-order with one shared permutation, which
+    is what GPTQ gives projections quantised on the same input): they can share launches."""
+    return all(p.w.perm_key == projs[0].w.perm_key for p in projs)
+
+
 def _pack_group(projs, Xds, dtype, also=()):
     """Packs the adapters of a group of projections (and of the projections in `also`, in the same
     launch); returns a _Stack when the group can share passes over the input (all adapted, one
-    post-dropout input, none act-order, total rank <= 128)."""
+    post-dropout input, total rank <= 128; the rank-r kernels work in the model's own K order, so act-order
+    weights do not matter here)."""
     live = [p for p in projs if p.r]
     if (len(live) == len(projs) and len(projs) > 1 and all(_same(Xd, Xds[0]) for Xd in Xds)
-            and all(p.w.perm is None for p in projs) and sum(p.r for p in projs) <= 128):
+            and sum(p.r for p in projs) <= 128):
         return _Stack(projs, dtype, Xds[0].device, also)
     _pack_projs([(p, None) for p in list(projs) + list(also)])
     return None
@@ -180,11 +197,11 @@ def _lora_down_all(projs, Xds, stack):
 
 
 def _linear_forward(projs, X2, Xds, stack=None):
-    """Y_p = X deq(W_p) + s U_p B_p^T for projections sharing X2.  One launch when no weight is
-    act-order; otherwise one launch per projection on its own column-permuted copy of X."""
+    """Y_p = X deq(W_p) + s U_p B_p^T for projections sharing X2.  One launch when the weights walk K in one
+    order (on X in that order); otherwise one launch per projection on its own column-permuted copy of X."""
     Us = _lora_down_all(projs, Xds, stack)
-    if all(p.w.perm is None for p in projs):
-        outs = fmsa_hip.gptq_lora_fwd(X2, [p.fwd_dict(U) for p, U in zip(projs, Us)])
+    if _one_order(projs):
+        outs = fmsa_hip.gptq_lora_fwd(projs[0].to_kernel_order(X2), [p.fwd_dict(U) for p, U in zip(projs, Us)])
     else:
         outs = [fmsa_hip.gptq_lora_fwd(p.to_kernel_order(X2), [p.fwd_dict(U)])[0] for p, U in zip(projs, Us)]
     return outs, Us
@@ -224,12 +241,14 @@ def _adapter_grads(projs, dYs, Xds, Us, stack):
 
 def _linear_backward_dx(projs, dYs, Ts, Xds, M, K):
     """dX = sum_p dY_p deq(W_p)^T + mask (.) sum_p s_p T_p A_p.  One launch when the projections share
-    one mask source (no dropout, or one dropout module applied once) and none is act-order; otherwise
+    one mask source (no dropout, or one dropout module applied once) and one K order; otherwise
     one launch per projection (each with its own mask / column order) and a sum."""
     masks = [Xd for p, Xd in zip(projs, Xds) if p.r]
     one_mask = all(_same(m, masks[0]) for m in masks)
-    if one_mask and all(p.w.perm is None for p in projs):
-        return fmsa_hip.gptq_lora_bwd_dx([p.bwd_dict(dY, T, Xd) for p, dY, T, Xd in zip(projs, dYs, Ts, Xds)], M, K)
+    if one_mask and _one_order(projs):
+        permuted = {}
+        dXk = fmsa_hip.gptq_lora_bwd_dx([p.bwd_dict(dY, T, Xd, permuted) for p, dY, T, Xd in zip(projs, dYs, Ts, Xds)], M, K)
+        return projs[0].from_kernel_order(dXk)
     dX = None
     for p, dY, T, Xd in zip(projs, dYs, Ts, Xds):
         part = p.from_kernel_order(fmsa_hip.gptq_lora_bwd_dx([p.bwd_dict(dY, T, Xd)], M, K))
@@ -306,10 +325,10 @@ def mlp_forward(ctx, X, gate, up, down, dropouts, dtype):
     X2 = _as2d(X, dtype)
     Xg, Xu = _dropped_inputs(X2, (gate, up), (dropout_gate, dropout_up))
     stack = _pack_group([gate, up], [Xg, Xu], dtype, also=(down,))
-    fused = gate.w.perm is None and up.w.perm is None
+    fused = _one_order([gate, up])
     if fused:
         Ug, Uu = _lora_down_all([gate, up], [Xg, Xu], stack)
-        e, g, h = fmsa_hip.gptq_lora_fwd(X2, [gate.fwd_dict(Ug), up.fwd_dict(Uu)], fmsa_hip.FWD_SWIGLU)
+        e, g, h = fmsa_hip.gptq_lora_fwd(gate.to_kernel_order(X2), [gate.fwd_dict(Ug), up.fwd_dict(Uu)], fmsa_hip.FWD_SWIGLU)
     else:
         (e, g), (Ug, Uu) = _linear_forward([gate, up], X2, [Xg, Xu], stack)
         h = fmsa_hip.swiglu_fwd(e, g)

@@ -12,9 +12,11 @@ class PreparedWeight:
     """The C-ABI view of one QuantLinear.  For an act-order g_idx the packed rows are re-ordered
     once (fmsa_gptq_permute_rows) so that the group of row k' is k' // group_size; `perm` then
     maps the kernels' row order back to the model's: row k' of the repacked weight is row
-    perm[k'] of the original."""
+    perm[k'] of the original.  Projections quantised on the same input (q, k, v; gate, up) get the
+    same order from act-order GPTQ (it sorts by the diagonal of the input's Hessian): `perm_key`
+    lets their callers see that and keep them in one launch."""
 
-    __slots__ = ("struct", "K", "N", "group_size", "perm", "nsz", "_keep")
+    __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep")
 
     def __init__(self, qweight, scales, qzeros, g_idx, bits):
         if bits != 4:
@@ -31,11 +33,13 @@ class PreparedWeight:
         g64 = g_idx.to(torch.int64)
         g64 = torch.where(g64 < 0, g64 + G, g64)
         perm = None
+        self.perm_key = None  # hashable identity of the row order: weights with equal keys can share one launch
         if not torch.equal(g64, ident):
             perm64 = torch.argsort(g64, stable=True)
             if not torch.equal(g64[perm64], ident):
                 raise NotImplementedError("act-order g_idx with groups of unequal size is not supported")
             perm = perm64.to(torch.int32).contiguous()
+            self.perm_key = hash(perm.cpu().numpy().tobytes())
             qweight = fmsa_hip.gptq_permute_rows(qweight, perm)
         self.K, self.N, self.group_size, self.perm = K, N, gs, perm
         self._keep = (qweight, scales, qzeros)

@@ -12,7 +12,7 @@ import fmsa_hip
 class PreparedNf4Weight:
     """The C-ABI view (`struct`, code-book format) of one NF4 linear of shape [N, K]."""
 
-    __slots__ = ("struct", "K", "N", "group_size", "perm", "nsz", "_keep")
+    __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep")
 
     def __init__(self, W, quant_state):
         if isinstance(quant_state, list):
@@ -33,7 +33,7 @@ class PreparedNf4Weight:
                                                     float(quant_state.offset), (N, K), bs, int(state2.blocksize))
         code = quant_state.code.to(device=data.device, dtype=torch.float32).contiguous()
         self.K, self.N, self.group_size = K, N, bs
-        self.perm = None  # no act-order for NF4
+        self.perm = self.perm_key = None  # no act-order for NF4
         self.nsz = None   # the input-gradient kernel reads block_scale through the struct
         self._keep = (qweight, block_scale, code)
         self.struct = fmsa_hip.make_codebook_weight(qweight, code, block_scale, bs)

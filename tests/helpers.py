@@ -8,11 +8,13 @@ import torch
 from oracle import gptq as ogptq
 
 
-def make_gptq(K, N, group_size=128, seed=0, act_order=False, sym=False, v1=False):
-    """Returns dict with numpy QuantLinear buffers, torch CPU tensors, and the fp32 dense weight."""
+def make_gptq(K, N, group_size=128, seed=0, act_order=False, sym=False, v1=False, order_seed=None):
+    """Returns dict with numpy QuantLinear buffers, torch CPU tensors, and the fp32 dense weight.
+    `order_seed` fixes the act-order permutation independently of the weights, so that several
+    projections can share one (as projections quantised on the same input do)."""
     gen = torch.Generator().manual_seed(seed)
     W = (torch.randn(N, K, generator=gen) * 0.02).numpy()
-    g_idx = ogptq.act_order_g_idx(K, group_size, seed=seed + 4) if act_order else None
+    g_idx = ogptq.act_order_g_idx(K, group_size, seed=seed + 4 if order_seed is None else order_seed) if act_order else None
     buf = ogptq.quantize_and_pack(W, group_size, sym=sym, g_idx=g_idx)
     zero_offset = 0
     if v1:

@@ -22,11 +22,11 @@ class MaskDropout(nn.Module):
 
 
 def make_lora_gptq_linear(K, N, r, alpha, seed, group_size=128, act_order=False, bias=False, device="cpu",
-                          lora_dtype=torch.float32, dropout=None):
+                          lora_dtype=torch.float32, dropout=None, order_seed=None):
     """LoraLinear(QuantLinear) with seeded weights.  Returns (module, dense fp32 W [K, N], A, B)."""
     from fms_acceleration_peft import LoraLinear, QuantLinear
 
-    w = make_gptq(K, N, group_size, seed=seed, act_order=act_order)
+    w = make_gptq(K, N, group_size, seed=seed, act_order=bool(act_order), order_seed=order_seed)
     ql = QuantLinear(4, w["group_size"], K, N, bias)
     ql.load_packed(w["np"]["qweight"], w["np"]["qzeros"], w["np"]["scales"], w["np"]["g_idx"])
     if bias:

@@ -22,7 +22,7 @@ DT = torch.bfloat16
 N_ROWS = 96
 
 
-def _gptq_lora(K, N, r, alpha, seed, act_order=False, group=128):
+def _gptq_lora(K, N, r, alpha, seed, act_order=False, group=128, order_seed=None):
     """LoraLinear(QuantLinear) quantised on the GPU; returns (module, fp32 dense W [K, N] on the CPU
     from the oracle's dequantisation of the packed buffers, A, B rounded to the activation dtype)."""
     from fms_acceleration_peft import LoraLinear
@@ -32,7 +32,7 @@ def _gptq_lora(K, N, r, alpha, seed, act_order=False, group=128):
     W = torch.randn(N, K, generator=gen, device="cuda") * 0.02
     g_idx = None
     if act_order:
-        perm = torch.randperm(K, generator=torch.Generator().manual_seed(seed + 4))
+        perm = torch.randperm(K, generator=torch.Generator().manual_seed(seed + 4 if order_seed is None else order_seed))
         g_idx = (torch.arange(K) // group)[perm].to(torch.int32).cuda()
     ql = quantize_linear(W, group, g_idx=g_idx).cuda()
     del W

@@ -54,8 +54,10 @@ def test_lora_w(B_, S_, K, N, r, dtype, act_order):
     assert all(not b.requires_grad for b in lin.base_layer.buffers())
 
 
+# act_order "shared": one permutation for the projections that read the same input (what act-order GPTQ produces,
+# since it sorts by the input's Hessian diagonal): they stay in one launch; True: one permutation per projection
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("act_order", [False, True])
+@pytest.mark.parametrize("act_order", [False, True, "shared"])
 def test_lora_qkv(dtype, act_order):
     from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_qkv
 
@@ -64,7 +66,8 @@ def test_lora_qkv(dtype, act_order):
     attn = torch.nn.Module()
     refs = {}
     for i, (name, N) in enumerate(Ns.items()):
-        lin, W, A, B = make_lora_gptq_linear(K, N, r, alpha, seed=10 + i, act_order=act_order, device="cuda")
+        lin, W, A, B = make_lora_gptq_linear(K, N, r, alpha, seed=10 + i, act_order=act_order, device="cuda",
+                                             order_seed=99 if act_order == "shared" else None)
         setattr(attn, name, lin)
         refs[name] = (W, _q(A, dtype), _q(B, dtype), alpha / r)
     x = randn((Bz, S, K), 2, dtype)
@@ -84,19 +87,41 @@ def test_lora_qkv(dtype, act_order):
         assert olora.max_rel_err(lin.lora_B["default"].weight.grad, dB_ref) < TOL
 
 
+@pytest.mark.parametrize("act_order,fwd_launches,bwd_launches", [(False, 1, 1), ("shared", 1, 1), (True, 3, 3)])
+def test_qkv_launch_count(monkeypatch, act_order, fwd_launches, bwd_launches):
+    """q, k, v go out as one fused-GEMM launch per direction unless their act-order permutations differ."""
+    import fmsa_hip
+    from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_qkv
+
+    calls = {"fwd": 0, "bwd": 0}
+    real_fwd, real_bwd = fmsa_hip.gptq_lora_fwd, fmsa_hip.gptq_lora_bwd_dx
+    monkeypatch.setattr(fmsa_hip, "gptq_lora_fwd", lambda *a, **k: (calls.__setitem__("fwd", calls["fwd"] + 1), real_fwd(*a, **k))[1])
+    monkeypatch.setattr(fmsa_hip, "gptq_lora_bwd_dx", lambda *a, **k: (calls.__setitem__("bwd", calls["bwd"] + 1), real_bwd(*a, **k))[1])
+    attn = torch.nn.Module()
+    for i, (name, N) in enumerate({"q_proj": 512, "k_proj": 128, "v_proj": 128}.items()):
+        lin, *_ = make_lora_gptq_linear(512, N, 8, 16.0, seed=40 + i, act_order=act_order, device="cuda",
+                                        order_seed=97 if act_order == "shared" else None)
+        setattr(attn, name, lin)
+    xg = randn((1, 64, 512), 5, torch.bfloat16).cuda().requires_grad_(True)
+    Q, Kt, V = apply_lora_qkv(attn, xg)
+    (Q.float().sum() + Kt.float().sum() + V.float().sum()).backward()
+    assert calls == {"fwd": fwd_launches, "bwd": bwd_launches}
+
+
 def _mlp(H, I, r, alpha, act_order, seed=20):
     mlp = torch.nn.Module()
     refs = {}
     for i, (name, (K, N)) in enumerate({"gate_proj": (H, I), "up_proj": (H, I), "down_proj": (I, H)}.items()):
         gs = 128 if K % 128 == 0 else 32
-        lin, W, A, B = make_lora_gptq_linear(K, N, r, alpha, seed=seed + i, act_order=act_order, device="cuda", group_size=gs)
+        lin, W, A, B = make_lora_gptq_linear(K, N, r, alpha, seed=seed + i, act_order=act_order, device="cuda", group_size=gs,
+                                             order_seed=98 if act_order == "shared" else None)
         setattr(mlp, name, lin)
         refs[name] = (W, A, B, alpha / r)
     return mlp, refs
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("act_order", [False, True])
+@pytest.mark.parametrize("act_order", [False, True, "shared"])
 @pytest.mark.parametrize("Bz,S,H,I", [(2, 128, 512, 1024), (1, 100, 256, 352)])
 def test_lora_mlp(Bz, S, H, I, dtype, act_order):
     from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_mlp
