@@ -74,16 +74,48 @@ class _Proj:
         # activation-type copies of the adapter in the four layouts the kernels read (one launch,
         # see pack): A [r, K], A^T [K, r], B [N, r], B^T [r, N]
         self.A = self.At = self.B = self.Bt = None
+        # An MLP whose down projection is act-order runs its intermediate dimension in that projection's
+        # kernel order: gate / up get re-ordered output columns (col_perm: column n' is the model's column
+        # col_perm[n']), down takes its input as it comes (input_ordered).
+        self.col_perm = None
+        self.input_ordered = False
+
+    def with_columns(self, col_perm, key):
+        """This projection producing its output columns in the order col_perm (before pack)."""
+        q = _Proj(self.w.with_columns(col_perm, key), None, self.A_param, self.B_param, self.s if self.r else None, self.dtype)
+        q.bias = None if self.bias is None else self.bias.index_select(0, col_perm)
+        q.col_perm = col_perm
+        return q
+
+    def with_ordered_input(self):
+        """This projection reading an input whose columns are already in its kernel order (before pack)."""
+        q = _Proj(self.w, None, self.A_param, self.B_param, self.s if self.r else None, self.dtype)
+        q.bias, q.input_ordered = self.bias, True
+        return q
+
+    def after_pack(self):
+        if self.r and self.col_perm is not None:
+            self.B, self.Bt = self.B.index_select(0, self.col_perm), self.Bt.index_select(1, self.col_perm)
+        if self.r and self.input_ordered:
+            self.A = self.A.index_select(1, self.w.perm.long())  # U = h' A'^T on the ordered input
+
+    def natural_grads(self, dA, dB):
+        """Adapter gradients back in the layouts of the parameters."""
+        if dB is not None and self.col_perm is not None:
+            dB = dB.index_select(0, self.w.col_inv)
+        if dA is not None and self.input_ordered:
+            dA = dA.index_select(1, torch.argsort(self.w.perm.long()))
+        return dA, dB
 
     def pack(self, A16_out=None):
         _pack_projs([(self, A16_out)])
 
     # the kernels walk K in the repacked order for act-order weights
     def to_kernel_order(self, X2):
-        return X2 if self.w.perm is None else fmsa_hip.permute_cols(X2, self.w.perm, gather=True)
+        return X2 if self.w.perm is None or self.input_ordered else fmsa_hip.permute_cols(X2, self.w.perm, gather=True)
 
     def from_kernel_order(self, dXp):
-        return dXp if self.w.perm is None else fmsa_hip.permute_cols(dXp, self.w.perm, gather=False)
+        return dXp if self.w.perm is None or self.input_ordered else fmsa_hip.permute_cols(dXp, self.w.perm, gather=False)
 
     def fwd_dict(self, U):
         return {"w": self.w.struct, "U": U, "B": self.B, "bias": self.bias, "r": self.r, "s": self.s}
@@ -96,7 +128,7 @@ class _Proj:
             At = self.At  # [K, r]
             if self.w.perm is not None:
                 At = At[self.w.perm.long()].contiguous()
-                if mask_src is not None:
+                if mask_src is not None and not self.input_ordered:
                     key = (id(mask_src), self.w.perm_key)
                     if permuted is not None and key in permuted:
                         mask_src = permuted[key][1]
@@ -150,6 +182,7 @@ def _pack_projs(items):
         packed = fmsa_hip.lora_pack_batch([(p.A_param, p.B_param, out) for p, out in live], live[0][0].dtype)
         for (p, _), quad in zip(live, packed):
             p.A, p.At, p.B, p.Bt = quad
+            p.after_pack()
 
 
 class _Stack:
@@ -324,6 +357,15 @@ def mlp_forward(ctx, X, gate, up, down, dropouts, dtype):
     dropout_gate, dropout_up, dropout_down = dropouts
     X2 = _as2d(X, dtype)
     Xg, Xu = _dropped_inputs(X2, (gate, up), (dropout_gate, dropout_up))
+    # act-order down projection: let gate / up write e, g, h in its kernel order, so that nothing between the two
+    # GEMM stages is permuted and both SwiGLU epilogues stay fused (not with a dropout on h: its mask is tied to
+    # the model's column order)
+    no_down_dropout = dropout_down is None or isinstance(dropout_down, torch.nn.Identity) or not down.r
+    if (down.w.perm is not None and no_down_dropout and hasattr(gate.w, "with_columns")
+            and gate.w.N == down.w.K and up.w.N == down.w.K):
+        order = down.w.perm.long()
+        gate, up = gate.with_columns(order, down.w.perm_key), up.with_columns(order, down.w.perm_key)
+        down = down.with_ordered_input()
     stack = _pack_group([gate, up], [Xg, Xu], dtype, also=(down,))
     fused = _one_order([gate, up])
     if fused:
@@ -361,7 +403,7 @@ def mlp_backward(ctx, dY):
             Td = torch.empty((M, down.r), dtype=dY2.dtype, device=dY2.device)
             (dBd,) = fmsa_hip.lora_grad_batch([(Ud, dY2, down.s, True, down.B_param.dtype, down.Bt, Td)])
     mask_h = hd if ctx.down_dropped else None
-    if down.w.perm is None:
+    if down.w.perm is None or down.input_ordered:
         h = fmsa_hip.gptq_lora_bwd_dx([down.bwd_dict(dY2, Td, mask_h)], M, I, fmsa_hip.BWD_SWIGLU, e=e, g=g)
     else:
         # un-fused epilogue for a repacked (act-order) weight: dh in kernel order, scatter back,
@@ -382,4 +424,5 @@ def mlp_backward(ctx, dY):
     # ---- up / gate: adapter grads, then dX over the concatenated contraction ---------------
     (Tg, Tu), ((dAg, dBg), (dAu, dBu)) = _adapter_grads([gate, up], [d_e, d_g], [Xg, Xu], [Ug, Uu], ctx.stack)
     dX = _linear_backward_dx([up, gate], [d_g, d_e], [Tu, Tg], [Xu, Xg], M, H)
-    return dX.view(ctx.x_shape).to(ctx.x_dtype), (dAg, dBg), (dAu, dBu), (dAd, dBd)
+    return (dX.view(ctx.x_shape).to(ctx.x_dtype), gate.natural_grads(dAg, dBg), up.natural_grads(dAu, dBu),
+            down.natural_grads(dAd, dBd))

@@ -16,7 +16,7 @@ class PreparedWeight:
     same order from act-order GPTQ (it sorts by the diagonal of the input's Hessian): `perm_key`
     lets their callers see that and keep them in one launch."""
 
-    __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep")
+    __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep", "_zero_offset", "_columns", "col_inv")
 
     def __init__(self, qweight, scales, qzeros, g_idx, bits):
         if bits != 4:
@@ -42,11 +42,37 @@ class PreparedWeight:
             self.perm_key = hash(perm.cpu().numpy().tobytes())
             qweight = fmsa_hip.gptq_permute_rows(qweight, perm)
         self.K, self.N, self.group_size, self.perm = K, N, gs, perm
+        self._zero_offset = zero_offset
+        self._columns = {}    # column-permuted twins, by the key of the permutation
+        self.col_inv = None   # set on such a twin: natural column n is column col_inv[n] of the twin
+        self._finish(qweight, scales, qzeros)
+
+    def _finish(self, qweight, scales, qzeros):
         self._keep = (qweight, scales, qzeros)
-        self.struct = fmsa_hip.make_weight(qweight, scales, qzeros, None, gs, zero_offset)
+        self.struct = fmsa_hip.make_weight(qweight, scales, qzeros, None, self.group_size, self._zero_offset)
         # -scale * zero per (group, column), fp32: read by the input-gradient kernel (frozen weight,
         # so it is built once)
         self.nsz = fmsa_hip.gptq_make_nsz(self.struct, qweight.device)
+
+    def with_columns(self, col_perm, key):
+        """The same weight with its output columns re-ordered: column n' of the twin is column col_perm[n'] of
+        this one (built once per permutation).  An MLP whose down projection is act-order lets gate and up
+        produce e, g and h directly in the row order the down projection's repacked weight wants."""
+        twin = self._columns.get(key)
+        if twin is None:
+            qweight, scales, qzeros = self._keep
+            idx = col_perm.long()
+            shifts = torch.arange(0, 32, 4, device=qzeros.device, dtype=torch.int64)
+            z = ((qzeros.to(torch.int64).unsqueeze(-1) >> shifts) & 0xF).reshape(qzeros.shape[0], -1)[:, idx]
+            zw = (z.reshape(qzeros.shape[0], -1, 8) << shifts).sum(-1)
+            zw = torch.where(zw >= 2**31, zw - 2**32, zw).to(torch.int32)
+            twin = object.__new__(PreparedWeight)
+            twin.K, twin.N, twin.group_size, twin.perm, twin.perm_key = self.K, self.N, self.group_size, self.perm, self.perm_key
+            twin._zero_offset, twin._columns = self._zero_offset, {}
+            twin.col_inv = torch.argsort(idx)
+            twin._finish(qweight[:, idx].contiguous(), scales[:, idx].contiguous(), zw.contiguous())
+            self._columns[key] = twin
+        return twin
 
 
 def prepare(qweight, scales, qzeros, g_idx, bits) -> PreparedWeight:
