@@ -100,12 +100,12 @@ __global__ __launch_bounds__(64 * NW) void lora_down_kernel(const uint16_t* __re
 // direct load writes lane p's 16 bytes to slot p), which spreads the 16 rows a fragment read touches
 // over all banks.  Wave w multiplies columns 64w .. 64w+63 of every stage; its Wd fragments come
 // straight from global (L2) one stage ahead.  Partial sums of the 8 waves are added as above.
-template <typename T, int RT>
+template <typename T, int RT, int MTL>
 __global__ __launch_bounds__(512) void lora_down_staged_kernel(const uint16_t* __restrict__ X, int64_t ldx,
                                                                const uint16_t* __restrict__ Wd, int M, int C, int r,
                                                                uint16_t* __restrict__ out, int64_t ldo) {
-  constexpr int NW = 8, NH = 4, MTL = 2, ROWS = 32, SC = 512;
-  static_assert(RT <= 4, "the reduction buffer overlays one stage buffer");
+  constexpr int NW = 8, NH = 4, ROWS = 16 * MTL, SC = 512;  // a wave moves 2 * MTL rows per stage
+  static_assert(RT <= 4 && (MTL == 1 || MTL == 2), "the reduction buffer overlays one stage buffer");
   // four separate arrays: every access names its buffer statically, so the compiler's wait counts
   // can tell reads of one buffer from direct loads in flight into the others
   __shared__ __attribute__((aligned(1024))) uint16_t s0[ROWS * SC];
@@ -130,19 +130,21 @@ __global__ __launch_bounds__(512) void lora_down_staged_kernel(const uint16_t* _
   const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(X + (size_t)m_base * ldx, (size_t)rows_valid * ldx * 2);
   const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(Wd, (size_t)r * C * 2);
 
-  // direct loads: wave w moves rows 4w .. 4w+3 of a stage
+  // direct loads: wave w moves rows RPW * w .. of a stage
+  // (arrays of fixed size and the template parameter itself in the loops: a local constant that depends on MTL,
+  // used inside the generic lambdas below, makes the host pass drop the kernel's stub without a diagnostic)
   uint32_t d_off[4], d_col[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = 4 * wave + i;
+  for (int i = 0; i < 2 * MTL; ++i) {
+    const int row = 2 * MTL * wave + i;
     d_col[i] = 8 * (lane ^ (row & 15));
     d_off[i] = (uint32_t)((row * ldx + d_col[i]) * 2);
   }
   auto dma = [&](int st, auto b_c) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 2 * MTL; ++i) {
       const uint32_t dead = (st * SC + (int)d_col[i]) < C ? 0u : 0x80000000u;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (__attribute__((address_space(3))) void*)(buf(b_c) + (4 * uwave + i) * (SC * 2)),
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (__attribute__((address_space(3))) void*)(buf(b_c) + (2 * MTL * uwave + i) * (SC * 2)),
                                                16, d_off[i] | dead, (uint32_t)st * (SC * 2), 0, 0);
     }
   };
@@ -177,9 +179,9 @@ __global__ __launch_bounds__(512) void lora_down_staged_kernel(const uint16_t* _
     }
   };
   // s_waitcnt vmcnt(n) only (expcnt / lgkmcnt fields left at their maxima)
-  constexpr int YOUNGER = 8 + 4 * RT;  // loads a wave issues after the direct loads of a stage and before that stage's turn
+  constexpr int YOUNGER = 4 * MTL + 4 * RT;  // loads a wave issues after the direct loads of a stage and before that stage's turn
   constexpr int WAIT_STEADY = (YOUNGER & 0xF) | ((YOUNGER >> 4) << 14) | 0x0F70;
-  constexpr int YOUNGER0 = 8 + 2 * RT;  // ... for stage 0 (prologue order)
+  constexpr int YOUNGER0 = 4 * MTL + 2 * RT;  // ... for stage 0 (prologue order)
   constexpr int WAIT_FIRST = (YOUNGER0 & 0xF) | ((YOUNGER0 >> 4) << 14) | 0x0F70;
   // one stage: its own direct loads have landed -> barrier (all waves' parts are there, and everybody has
   // left the buffer that is re-filled next) -> requests two and three stages ahead -> multiply
@@ -542,15 +544,23 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
   constexpr int NW = 8;  // waves per workgroup: measured best of 4 / 8 / 16 at 8192 tokens
   dim3 grid((M + 16 * mtl - 1) / (16 * mtl)), block(64 * NW);
   const int rt = (r + 15) / 16;
-  // staged kernel: 32 tokens per workgroup, worth it once that gives every CU a workgroup and the rows are long
-  // enough to amortise its pipeline fill (measured at 8192 tokens: 59 -> 48 us at C = 14336, r = 16; 32 -> 28 us
-  // at C = 4096, r = 48; 20 -> 21 us at C = 4096, r = 16)
-  const bool staged = M >= 32 * 256 && rt <= 4 && (C >= 8192 || (rt >= 2 && C >= 2048));
+  // staged kernel: 32 (from 8192 tokens) or 16 (from 4096) tokens per workgroup, worth it once that gives every CU a
+  // workgroup and the rows are long enough to amortise its pipeline fill (measured at 8192 tokens: 59 -> 48 us at
+  // C = 14336, r = 16; 32 -> 28 us at C = 4096, r = 48; 20 -> 21 us at C = 4096, r = 16; at 4096 tokens, C = 28672,
+  // r = 64: 205 us with the fragment loads above)
+  const bool staged = M >= 16 * 256 && rt <= 4 && (C >= 8192 || (rt >= 2 && C >= 2048));
   if (staged) {
-    dim3 sgrid((M + 31) / 32), sblock(512);
-#define SLAUNCH(TT, RT)                                                                                                        \
-  hipLaunchKernelGGL((lora_down_staged_kernel<TT, RT>), sgrid, sblock, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, M, C, \
-                     r, (uint16_t*)out, ldo)
+    const int smtl = M >= 32 * 256 ? 2 : 1;
+    dim3 sgrid((M + 16 * smtl - 1) / (16 * smtl)), sblock(512);
+#define SLAUNCH(TT, RT)                                                                                                           \
+  do {                                                                                                                            \
+    if (smtl == 2)                                                                                                                \
+      hipLaunchKernelGGL((lora_down_staged_kernel<TT, RT, 2>), sgrid, sblock, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, \
+                         M, C, r, (uint16_t*)out, ldo);                                                                           \
+    else                                                                                                                          \
+      hipLaunchKernelGGL((lora_down_staged_kernel<TT, RT, 1>), sgrid, sblock, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, \
+                         M, C, r, (uint16_t*)out, ldo);                                                                           \
+  } while (0)
 #define SDISPATCH(TT)                \
   switch (rt) {                      \
     case 1: SLAUNCH(TT, 1); break;   \

@@ -104,7 +104,7 @@ class _Proj:
         if dB is not None and self.col_perm is not None:
             dB = dB.index_select(0, self.w.col_inv)
         if dA is not None and self.input_ordered:
-            dA = dA.index_select(1, torch.argsort(self.w.perm.long()))
+            dA = dA.index_select(1, self.w.row_inv)
         return dA, dB
 
     def pack(self, A16_out=None):

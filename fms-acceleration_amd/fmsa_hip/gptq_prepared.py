@@ -16,7 +16,7 @@ class PreparedWeight:
     same order from act-order GPTQ (it sorts by the diagonal of the input's Hessian): `perm_key`
     lets their callers see that and keep them in one launch."""
 
-    __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep", "_zero_offset", "_columns", "col_inv")
+    __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep", "_zero_offset", "_columns", "col_inv", "_row_inv")
 
     def __init__(self, qweight, scales, qzeros, g_idx, bits):
         if bits != 4:
@@ -43,6 +43,7 @@ class PreparedWeight:
             qweight = fmsa_hip.gptq_permute_rows(qweight, perm)
         self.K, self.N, self.group_size, self.perm = K, N, gs, perm
         self._zero_offset = zero_offset
+        self._row_inv = None
         self._columns = {}    # column-permuted twins, by the key of the permutation
         self.col_inv = None   # set on such a twin: natural column n is column col_inv[n] of the twin
         self._finish(qweight, scales, qzeros)
@@ -53,6 +54,13 @@ class PreparedWeight:
         # -scale * zero per (group, column), fp32: read by the input-gradient kernel (frozen weight,
         # so it is built once)
         self.nsz = fmsa_hip.gptq_make_nsz(self.struct, qweight.device)
+
+    @property
+    def row_inv(self):
+        """Inverse of `perm` (int64): the model's row k is row row_inv[k] of the repacked weight."""
+        if self._row_inv is None:
+            self._row_inv = torch.argsort(self.perm.long())
+        return self._row_inv
 
     def with_columns(self, col_perm, key):
         """The same weight with its output columns re-ordered: column n' of the twin is column col_perm[n'] of
@@ -68,7 +76,7 @@ class PreparedWeight:
             zw = torch.where(zw >= 2**31, zw - 2**32, zw).to(torch.int32)
             twin = object.__new__(PreparedWeight)
             twin.K, twin.N, twin.group_size, twin.perm, twin.perm_key = self.K, self.N, self.group_size, self.perm, self.perm_key
-            twin._zero_offset, twin._columns = self._zero_offset, {}
+            twin._zero_offset, twin._columns, twin._row_inv = self._zero_offset, {}, None
             twin.col_inv = torch.argsort(idx)
             twin._finish(qweight[:, idx].contiguous(), scales[:, idx].contiguous(), zw.contiguous())
             self._columns[key] = twin
