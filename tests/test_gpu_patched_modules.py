@@ -29,11 +29,13 @@ def _llama_cfg(hidden):
     return cfg
 
 
-def _wrap(mod, names, seed, dropout_p=0.0, tokens=None):
+def _wrap(mod, names, seed, dropout_p=0.0, tokens=None, act_order=False, dropout_on=None):
     for i, name in enumerate(names):
         lin = getattr(mod, name)
-        drop = MaskDropout(dropout_p, (tokens, lin.in_features), seed=seed + 50 + i) if dropout_p else None
-        wrapped, _, _, _ = make_lora_gptq_linear(lin.in_features, lin.out_features, R, ALPHA, seed=seed + i, dropout=drop)
+        dropped = dropout_p is not None and (dropout_on is None or name in dropout_on) and (dropout_p or dropout_on)
+        drop = MaskDropout(dropout_p, (tokens, lin.in_features), seed=seed + 50 + i) if dropped else None
+        wrapped, _, _, _ = make_lora_gptq_linear(lin.in_features, lin.out_features, R, ALPHA, seed=seed + i, dropout=drop,
+                                                 act_order=act_order)
         setattr(mod, name, wrapped)
 
 
@@ -99,16 +101,46 @@ def test_attention_qkvo(bsz, seq, hidden, dropout_p, dtype):
     _compare(attn, fused, run, x, dtype)
 
 
+# Dropout on gate / up only: with a dropout on h the fused function forms the down-projection gradients from the
+# recomputed h like the reference does (UL/gptq/fast_lora.py:369-370), which the unfused module does not.
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("act_order,dropout_p", [(False, 0.0), (True, 0.0), (True, 0.5), (False, 0.5)])
 @pytest.mark.parametrize("bsz,seq,hidden", SIZES)
-def test_mlp(bsz, seq, hidden, dtype):
+def test_mlp(bsz, seq, hidden, dtype, act_order, dropout_p):
     from transformers.models.llama.modeling_llama import LlamaMLP
 
     cfg = _llama_cfg(hidden)
     mlp = LlamaMLP(cfg)
-    _wrap(mlp, ("gate_proj", "up_proj", "down_proj"), seed=9)
+    _wrap(mlp, ("gate_proj", "up_proj", "down_proj"), seed=9, dropout_p=dropout_p, tokens=bsz * seq, act_order=act_order,
+          dropout_on=("gate_proj", "up_proj") if dropout_p else None)
     mlp = mlp.cuda()
     fused, n_patched = _patched_copy(mlp, cfg)
     assert n_patched == 1
     x = randn((bsz, seq, hidden), 2, dtype).cuda()
     _compare(mlp, fused, lambda mod, xi: mod(xi), x, dtype)
+
+
+def test_mlp_act_order_routes_agree():
+    """An act-order down projection normally takes its input in kernel order straight from gate / up (checked
+    against the unfused module above); a dropout module on h switches that off and h is permuted instead.  With
+    a dropout that keeps everything the two routes compute the same function."""
+    from transformers.models.llama.modeling_llama import LlamaMLP
+
+    bsz, seq, hidden, dtype = 2, 128, 2048, torch.bfloat16
+    cfg = _llama_cfg(hidden)
+    results = []
+    for keep_all_dropout in (False, True):
+        mlp = LlamaMLP(cfg)
+        _wrap(mlp, ("gate_proj", "up_proj", "down_proj"), seed=9, dropout_p=0.0, tokens=bsz * seq, act_order=True,
+              dropout_on=("down_proj",) if keep_all_dropout else None)
+        fused, _ = _patched_copy(mlp.cuda(), cfg)
+        xi = randn((bsz, seq, hidden), 2, dtype).cuda().requires_grad_(True)
+        with torch.autocast(device_type="cuda", dtype=dtype):
+            out = fused(xi)
+        out.float().norm().backward()
+        results.append((out.float().detach().cpu(), xi.grad.float().cpu(), _lora_grads(fused)))
+    (o0, dx0, g0), (o1, dx1, g1) = results
+    assert torch.equal(o0, o1)
+    assert torch.allclose(dx0, dx1, rtol=1e-2, atol=1e-3 * dx0.abs().max().item())
+    for name in g0:
+        assert torch.allclose(g0[name], g1[name], rtol=1e-2, atol=1e-3 * g0[name].abs().max().item()), name
