@@ -105,7 +105,7 @@ __global__ __launch_bounds__(512) void lora_down_staged_kernel(const uint16_t* _
                                                                const uint16_t* __restrict__ Wd, int M, int C, int r,
                                                                uint16_t* __restrict__ out, int64_t ldo) {
   constexpr int NW = 8, NH = 4, ROWS = 16 * MTL, SC = 512;  // a wave moves 2 * MTL rows per stage
-  static_assert(RT <= 4 && (MTL == 1 || MTL == 2), "the reduction buffer overlays one stage buffer");
+  static_assert(RT <= 8 && (MTL == 1 || MTL == 2), "rank tiles are reduced four at a time through one stage buffer");
   // four separate arrays: every access names its buffer statically, so the compiler's wait counts
   // can tell reads of one buffer from direct loads in flight into the others
   __shared__ __attribute__((aligned(1024))) uint16_t s0[ROWS * SC];
@@ -213,33 +213,39 @@ __global__ __launch_bounds__(512) void lora_down_staged_kernel(const uint16_t* _
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the surplus direct loads (all lanes out of range) have landed too
   __syncthreads();
 
-  float(*red)[MTL][RT][64][4] = reinterpret_cast<float(*)[MTL][RT][64][4]>(s0);  // [NH]: 8 * RT KB <= one stage buffer
-  if (wave >= NH) {
+  // the waves' partial tiles are added through stage buffer 0, RC rank tiles at a time ([NH][MTL][RC] KB <= its size)
+  constexpr int RC = RT < 4 ? RT : 4;
+  float(*red)[MTL][RC][64][4] = reinterpret_cast<float(*)[MTL][RC][64][4]>(s0);
+  static_for<0, RT / RC>([&](auto c_c) {
+    constexpr int t0 = decltype(c_c)::value * RC;
+    if (wave >= NH) {
 #pragma unroll
-    for (int u = 0; u < MTL; ++u)
+      for (int u = 0; u < MTL; ++u)
 #pragma unroll
-      for (int t = 0; t < RT; ++t) *reinterpret_cast<f32x4*>(red[wave - NH][u][t][lane]) = acc[u][t];
-  }
-  __syncthreads();
-  if (wave < NH) {
+        for (int t = 0; t < RC; ++t) *reinterpret_cast<f32x4*>(red[wave - NH][u][t][lane]) = acc[u][t0 + t];
+    }
+    __syncthreads();
+    if (wave < NH) {
 #pragma unroll
-    for (int u = 0; u < MTL; ++u)
+      for (int u = 0; u < MTL; ++u)
 #pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        const f32x4 o = *reinterpret_cast<const f32x4*>(red[wave][u][t][lane]);
-        *reinterpret_cast<f32x4*>(red[wave][u][t][lane]) = acc[u][t] + o;
-      }
-  }
-  __syncthreads();
-  for (int o = tid; o < MTL * RT * 256; o += 64 * NW) {
-    const int u = o / (RT * 256), t = (o >> 8) % RT, ln = (o >> 2) & 63, i = o & 3;
-    float v = red[0][u][t][ln][i];
+        for (int t = 0; t < RC; ++t) {
+          const f32x4 o = *reinterpret_cast<const f32x4*>(red[wave][u][t][lane]);
+          *reinterpret_cast<f32x4*>(red[wave][u][t][lane]) = acc[u][t0 + t] + o;
+        }
+    }
+    __syncthreads();
+    for (int o = tid; o < MTL * RC * 256; o += 64 * NW) {
+      const int u = o / (RC * 256), t = (o >> 8) % RC, ln = (o >> 2) & 63, i = o & 3;
+      float v = red[0][u][t][ln][i];
 #pragma unroll
-    for (int w = 1; w < NH; ++w) v += red[w][u][t][ln][i];
-    const int row = m_base + 16 * u + 4 * (ln >> 4) + i;
-    const int j = 16 * t + (ln & 15);
-    if (row < M && j < r) out[(size_t)row * ldo + j] = pack1<T>(v);
-  }
+      for (int w = 1; w < NH; ++w) v += red[w][u][t][ln][i];
+      const int row = m_base + 16 * u + 4 * (ln >> 4) + i;
+      const int j = 16 * (t0 + t) + (ln & 15);
+      if (row < M && j < r) out[(size_t)row * ldo + j] = pack1<T>(v);
+    }
+    if constexpr (t0 + RC < RT) __syncthreads();  // the next four rank tiles reuse the buffer
+  });
 }
 
 // ---- lora_grad ----------------------------------------------------------------------------------
@@ -548,7 +554,7 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
   // workgroup and the rows are long enough to amortise its pipeline fill (measured at 8192 tokens: 59 -> 48 us at
   // C = 14336, r = 16; 32 -> 28 us at C = 4096, r = 48; 20 -> 21 us at C = 4096, r = 16; at 4096 tokens, C = 28672,
   // r = 64: 205 us with the fragment loads above)
-  const bool staged = M >= 16 * 256 && rt <= 4 && (C >= 8192 || (rt >= 2 && C >= 2048));
+  const bool staged = M >= 16 * 256 && rt <= 8 && (C >= 8192 || (rt >= 2 && C >= 2048));
   if (staged) {
     const int smtl = M >= 32 * 256 ? 2 : 1;
     dim3 sgrid((M + 16 * smtl - 1) / (16 * smtl)), sblock(512);
@@ -561,11 +567,12 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
       hipLaunchKernelGGL((lora_down_staged_kernel<TT, RT, 1>), sgrid, sblock, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, \
                          M, C, r, (uint16_t*)out, ldo);                                                                           \
   } while (0)
-#define SDISPATCH(TT)                \
-  switch (rt) {                      \
-    case 1: SLAUNCH(TT, 1); break;   \
-    case 2: SLAUNCH(TT, 2); break;   \
-    default: SLAUNCH(TT, 4); break;  \
+#define SDISPATCH(TT)                        \
+  switch (rt) {                              \
+    case 1: SLAUNCH(TT, 1); break;           \
+    case 2: SLAUNCH(TT, 2); break;           \
+    case 3: case 4: SLAUNCH(TT, 4); break;   \
+    default: SLAUNCH(TT, 8); break;          \
   }
     if (act_dtype == FMSA_BF16) {
       SDISPATCH(bf16_t)

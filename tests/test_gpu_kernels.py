@@ -77,7 +77,7 @@ def test_permute_cols(M, C):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,C,r", [(4096, 28672, 64), (4100, 8192, 32), (8192, 8200, 16), (8200, 14336, 32), (8192, 2048, 48), (8222, 9000, 64), (8192, 4096, 24)])
+@pytest.mark.parametrize("M,C,r", [(4096, 28672, 64), (4100, 8192, 32), (8192, 4096, 96), (8200, 2048, 128), (4096, 8200, 120), (8192, 8200, 16), (8200, 14336, 32), (8192, 2048, 48), (8222, 9000, 64), (8192, 4096, 24)])
 def test_lora_down_many_tokens(M, C, r, dtype):
     """From 8192 tokens on, long rows / stacked ranks take the kernel that stages X through LDS: ragged
     token and column counts (last workgroup of 8 or 30 rows, last 512-column stage of 8 or 296 columns),
