@@ -1,5 +1,7 @@
 """Plugin registry / framework behaviours (mirrors plugins/framework/tests/test_framework.py of
 the reference): AND / OR configuration paths, activation order, errors."""
+import os
+
 import pytest
 import torch
 
@@ -146,3 +148,51 @@ def test_shipped_plugins_are_registered_and_configurable():
     with instantiate_framework(alt) as fw:
         plugin = fw.active_plugins[0][1]
         assert plugin.configurations["base_layer"] == "auto_gptq" and plugin.configurations["fast_loss"] is False
+
+
+def test_shipped_sample_configurations(monkeypatch):
+    """The YAML files under fms-acceleration_amd/configs (the reference's plugin configuration keys under
+    the framework's `plugins:` body, cf. plugins/accelerated-peft/tests/test_peft_plugins.py:47-120 and
+    plugins/fused-ops-and-kernels/tests/test_foak_plugins.py:39-85): read from the path and through the
+    ACCELERATION_FRAMEWORK_CONFIG_FILE route, each activates the plugins it names with the values it sets."""
+    import glob
+
+    import yaml
+
+    from fms_acceleration.constants import KEY_PLUGINS
+    from fms_acceleration.framework import AccelerationFramework, read_configuration_file
+
+    cfg_dir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "fms-acceleration_amd", "configs")
+    expected = {
+        "accelerated-peft-autogptq-foak.yaml": (["AutoGPTQAccelerationPlugin", "FastKernelsAccelerationPlugin"], "auto_gptq", True),
+        "accelerated-peft-autogptq-foak-liger.yaml": (["AutoGPTQAccelerationPlugin", "FastKernelsAccelerationPlugin"], "auto_gptq", "fused_ce_liger"),
+        "accelerated-peft-bnb-nf4-foak.yaml": (["BNBAccelerationPlugin", "FastKernelsAccelerationPlugin"], "bitsandbytes", True),
+        "foak-fast-kernels.yaml": (["FastKernelsAccelerationPlugin"], "auto_gptq", True),
+    }
+    files = sorted(glob.glob(os.path.join(cfg_dir, "*.yaml")))
+    assert sorted(os.path.basename(f) for f in files) == sorted(expected)
+    for path in files:
+        names, base_layer, fast_loss = expected[os.path.basename(path)]
+        body = read_configuration_file(path)
+        for via_env in (False, True):
+            # the framework keeps its activation lists on the class: a fresh pair per instantiation
+            monkeypatch.setattr(AccelerationFramework, "active_plugins", [])
+            monkeypatch.setattr(AccelerationFramework, "plugins_require_custom_loading", [])
+            if via_env:
+                monkeypatch.setenv("ACCELERATION_FRAMEWORK_CONFIG_FILE", path)
+                fw = AccelerationFramework(None, require_packages_check=False)
+            else:
+                monkeypatch.delenv("ACCELERATION_FRAMEWORK_CONFIG_FILE", raising=False)
+                fw = AccelerationFramework(path, require_packages_check=False)
+            assert [n for n, _ in fw.active_plugins] == names
+            foak = dict(fw.active_plugins)["FastKernelsAccelerationPlugin"]
+            assert foak.configurations["base_layer"] == base_layer and foak.configurations["fast_loss"] == fast_loss
+            assert fw.requires_augmentation and fw.requires_custom_loading == (len(names) == 2)
+        monkeypatch.delenv("ACCELERATION_FRAMEWORK_CONFIG_FILE", raising=False)
+        # a value outside the allowed set is refused with the plugin's name in the message
+        section = body["peft"]["quantization"] if "peft" in body else body["training"]
+        section["fused_ops_and_kernels"]["fast_loss"] = "something_else"
+        with pytest.raises(AccelerationPluginConfigError, match="FastKernelsAccelerationPlugin"):
+            with instantiate_framework(body, require_packages_check=False):
+                pass
+    assert yaml.safe_load(open(files[0], encoding="utf-8"))[KEY_PLUGINS]
