@@ -120,9 +120,12 @@ def _mlp(H, I, r, alpha, act_order, seed=20):
     return mlp, refs
 
 
+# two fixed shapes and six odd ones (H, I any multiple of 32: every tile cut in M, N, K; at least 33 tokens, fewer leave
+# the 16-bit roundings of single products unaveraged and above the tolerance)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("act_order", [False, True, "shared"])
-@pytest.mark.parametrize("Bz,S,H,I", [(2, 128, 512, 1024), (1, 100, 256, 352)])
+@pytest.mark.parametrize("Bz,S,H,I", [(2, 128, 512, 1024), (1, 100, 256, 352), (1, 33, 96, 160), (3, 37, 160, 608),
+                                      (1, 257, 672, 96), (2, 150, 32, 1312), (1, 513, 416, 288), (1, 64, 1184, 736)])
 def test_lora_mlp(Bz, S, H, I, dtype, act_order):
     from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_mlp
 

@@ -316,6 +316,56 @@ def test_bwd_dx_linear(M, K, N, gs, r, dtype):
     assert olora.max_rel_err(dx2.cpu(), ref2) < TOL
 
 
+def _random_shapes(n, seed):
+    """Seeded shapes that respect the kernels' contract (K, N multiples of 32; group size a multiple of 32
+    dividing K; rank a multiple of 8) and otherwise hit every tail: token counts from 1, tiles cut in M, N and K."""
+    import random
+
+    rng = random.Random(seed)
+    cases = []
+    for _ in range(n):
+        K = 32 * rng.randint(1, 40)
+        gs = rng.choice([g for g in (32, 64, 96, 128, 256, K) if K % g == 0])
+        cases.append((rng.choice([1, 7, 31, 64, 100, 255, 256, 257, 300, 513]), K, 32 * rng.randint(1, 40), gs,
+                      rng.choice([0, 8, 16, 24, 40]), rng.random() < 0.4, rng.choice([torch.bfloat16, torch.float16])))
+    return cases
+
+
+@pytest.mark.parametrize("M,K,N,gs,r,bias,dtype", _random_shapes(20, 1234))
+def test_fwd_and_bwd_random_shapes(M, K, N, gs, r, bias, dtype):
+    import fmsa_hip
+
+    s = 0.5
+    w = make_gptq(K, N, gs, seed=K + N)
+    gw = gweight(w)
+    x = randn((M, K), 2, dtype)
+    x[::3, ::4] = 0
+    A, B = olora.make_lora(K, N, r, 5) if r else (None, None)
+    Aq, Bq = (A.to(dtype).float(), B.to(dtype).float()) if r else (None, None)
+    b = randn((N,), 9, dtype, 0.1) if bias else None
+    xd = dev(x)
+    p = {"w": gw, "r": r, "s": s, "bias": None if b is None else dev(b)}
+    if r:
+        p["U"] = fmsa_hip.lora_down(xd, dev(A.to(dtype)))
+        p["B"] = dev(B.to(dtype))
+    (y,) = fmsa_hip.gptq_lora_fwd(xd, [p])
+    ref = olora.lora_linear(x.float(), w["dense"], Aq, Bq, s, None if b is None else b.float())
+    assert olora.max_rel_err(y.cpu(), ref) < TOL
+    dy = randn((M, N), 3, dtype)
+    dyd = dev(dy)
+    if r:
+        dx = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(w, dyd, A, B, s, dtype, mask_src=xd)], M, K)
+        dx_ref, dA_ref, dB_ref = olora.lora_w_manual(x.float(), w["dense"], Aq, Bq, s, dy.float())
+        T = fmsa_hip.lora_down(dyd, dev(B.to(dtype).t().contiguous()))
+        dA, dB = fmsa_hip.lora_grad_batch([(T, xd, s, False, torch.float32), (p["U"], dyd, s, True, torch.float32)])
+        assert olora.max_rel_err(dA.cpu(), dA_ref) < TOL and olora.max_rel_err(dB.cpu(), dB_ref) < TOL
+    else:
+        dx = fmsa_hip.gptq_lora_bwd_dx([{"w": gw, "nsz": fmsa_hip.gptq_make_nsz(gw, dyd.device), "dY": dyd, "T": None, "At": None,
+                                         "mask_src": None, "r": 0, "s": 0.0}], M, K)
+        dx_ref = dy.float() @ w["dense"].t()
+    assert olora.max_rel_err(dx.cpu(), dx_ref) < TOL
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16])
 def test_bwd_dx_three_projections(dtype):
     import fmsa_hip
