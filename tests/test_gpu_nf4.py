@@ -185,7 +185,9 @@ def test_nf4_prepare_bit_exact(N, K, blocksize, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,K,N,r,blocksize", [(200, 256, 96, 16, 64), (512, 1024, 512, 8, 64), (64, 1056, 288, 32, 32), (300, 512, 256, 16, 128)])
+@pytest.mark.parametrize("M,K,N,r,blocksize", [(200, 256, 96, 16, 64), (512, 1024, 512, 8, 64), (64, 1056, 288, 32, 32), (300, 512, 256, 16, 128),
+                                               (1, 64, 32, 8, 64), (257, 1344, 608, 24, 64), (31, 96, 1184, 40, 32), (513, 640, 160, 8, 128),
+                                               (100, 1152, 896, 16, 64), (7, 2048, 96, 64, 64)])
 def test_codebook_kernels(M, K, N, r, blocksize, dtype):
     """Forward (LoRA + bias) and input gradient (LoRA with a mask) of the code-book kernel flavour."""
     import fmsa_hip
