@@ -4,30 +4,36 @@ kernels/unsloth/rope_embedding.py of the reference: `Fast_RoPE_Embedding` :68-12
 
 Like the reference the rotation is applied in place on the [batch, seq, heads, head_dim] view of the
 projection output and ignores `position_ids` (:131): row m of the flattened tokens takes position
-m % seq_len of a 2-D cos / sin; a 3-D cos / sin [batch, seq, head_dim] (what recent transformers
-pass) is used row by row, which is the same thing for the default positions."""
+m % seq_len (:60-63, with seq_len <= cos.shape[0] allowed) of a 2-D cos / sin cache, however many
+positions that cache holds; a 3-D cos / sin [batch, seq, head_dim] (what recent transformers pass)
+is used row by row, which is the same thing for the default positions."""
 import torch
 
 import fmsa_hip
 
 
-def _rows(t):
-    """cos / sin as [rows, head_dim]: [seq, d], [1, seq, d] -> [seq, d]; [batch, seq, d] -> [batch*seq, d]."""
-    t = t.squeeze()
-    if t.dim() == 3:
-        t = t.reshape(-1, t.shape[-1])
-    if t.dim() != 2:
-        raise ValueError(f"cos / sin must be [seq, head_dim] or [batch, seq, head_dim], got {tuple(t.shape)}")
+def _rows(t, batch, seq_len):
+    """cos / sin as the [rows, head_dim] table the kernel indexes with (token row % rows):
+    [P, d] or [1, P, d] with P >= seq_len -> its first seq_len rows (every batch entry starts again at
+    position 0); [batch, seq_len, d] -> [batch * seq_len, d]."""
+    while t.dim() > 2 and t.shape[0] == 1:
+        t = t[0]
+    if t.dim() == 2:
+        if t.shape[0] < seq_len:
+            raise ValueError("cos / sin cover fewer positions than the sequence")
+        t = t[:seq_len]
+    elif t.dim() == 3 and t.shape[0] == batch and t.shape[1] == seq_len:
+        t = t.reshape(batch * seq_len, t.shape[-1])
+    else:
+        raise ValueError(f"cos / sin must be [positions, head_dim] or [batch, seq, head_dim], got {tuple(t.shape)}")
     return t if t.stride(1) == 1 else t.contiguous()
 
 
 class Fast_RoPE_Embedding(torch.autograd.Function):
     @staticmethod
     def forward(ctx, Q, cos, sin):
-        cos, sin = _rows(cos), _rows(sin)
         batch, seq_len, n_heads, head_dim = Q.shape
-        if seq_len > cos.shape[0]:
-            raise ValueError("cos / sin cover fewer positions than the sequence")
+        cos, sin = _rows(cos, batch, seq_len), _rows(sin, batch, seq_len)
         Q2 = Q.view(batch * seq_len, n_heads * head_dim)
         fmsa_hip.rope_embedding_(Q2, cos, sin, n_heads, head_dim, backward=False)
         ctx.cos, ctx.sin = cos, sin

@@ -90,7 +90,7 @@ def test_fast_rms_layernorm_vs_transformers(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("cos_3d", [False, True])
+@pytest.mark.parametrize("cos_3d", [False, True, "long_cache"])
 def test_fast_rope_embedding_vs_transformers(dtype, cos_3d):
     from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
 
@@ -98,8 +98,14 @@ def test_fast_rope_embedding_vs_transformers(dtype, cos_3d):
 
     b, s, h, hk, d = 2, 48, 8, 2, 64
     cos, sin = _cos_sin(s, d, dtype)
-    cos_b = cos[None].expand(b, s, d).contiguous().cuda() if cos_3d else cos[None].cuda()
-    sin_b = sin[None].expand(b, s, d).contiguous().cuda() if cos_3d else sin[None].cuda()
+    cos_b = cos[None].expand(b, s, d).contiguous().cuda() if cos_3d is True else cos[None].cuda()
+    sin_b = sin[None].expand(b, s, d).contiguous().cuda() if cos_3d is True else sin[None].cuda()
+    cos_f, sin_f = cos_b, sin_b
+    if cos_3d == "long_cache":
+        # a 2-D cache that holds more positions than the sequence (rope_embedding.py:60-63 of the reference
+        # allows seq_len <= cos.shape[0]): every batch entry still starts at position 0
+        cos_l, sin_l = _cos_sin(s + 16, d, dtype)
+        cos_f, sin_f = cos_l.cuda(), sin_l.cuda()
     xq = randn((b, s, h * d), 8, dtype).cuda()
     xk = randn((b, s, hk * d), 9, dtype).cuda()
     dq = randn((b, h, s, d), 10, dtype).cuda()
@@ -111,7 +117,8 @@ def test_fast_rope_embedding_vs_transformers(dtype, cos_3d):
         # projection outputs viewed the way the attention module views them (a non-leaf, as in the model)
         q = (pq * 1.0).view(b, s, h, d).transpose(1, 2)
         k = (pk * 1.0).view(b, s, hk, d).transpose(1, 2)
-        qo, ko = fn(q, k, cos_b, sin_b)
+        cs = (cos_f, sin_f) if fn is fast_rope_embedding else (cos_b, sin_b)
+        qo, ko = fn(q, k, *cs)
         torch.autograd.backward([qo, ko], [dq, dk])
         return qo.detach(), ko.detach(), pq.grad, pk.grad
 

@@ -79,3 +79,30 @@ def test_rope_backward_is_the_vjp():
     dy = torch.randn(s, h * d, dtype=torch.float64)
     out.backward(dy)
     assert torch.allclose(onr.rope(dy.float(), cos.float(), sin.float(), h, d, backward=True).double(), q.grad, atol=1e-5)
+
+
+def test_rope_table_rows_of_the_host_wrapper():
+    """The table the kernel indexes with (token row % rows): a 2-D cache longer than the sequence is cut to
+    seq_len rows, so batch entry b restarts at position 0 (reference rope_embedding.py:60-63: row % seq_len
+    with seq_len <= cos.shape[0]); a per-batch 3-D table is flattened row by row."""
+    import pytest
+
+    from fms_acceleration_foak.kernels.unsloth.rope_embedding import _rows
+
+    b, s, h, d = 2, 5, 2, 16
+    ang = torch.outer(torch.arange(s + 3).float(), 1.0 / (10000 ** (torch.arange(0, d, 2).float() / d)))
+    cache = torch.cat([ang, ang], -1).cos()
+    for form in (cache, cache[None]):
+        t = _rows(form, b, s)
+        assert t.shape == (s, d) and torch.equal(t, cache[:s])
+    per_batch = torch.stack([cache[:s], cache[3:3 + s]])
+    assert torch.equal(_rows(per_batch, b, s), per_batch.reshape(b * s, d))
+    with pytest.raises(ValueError):
+        _rows(cache[: s - 1], b, s)
+    with pytest.raises(ValueError):
+        _rows(per_batch[:, : s - 1], b, s)
+    # with that table the oracle's row % rows lookup gives batch 1 the positions 0 .. s-1 again
+    q = torch.randn(b * s, h * d, generator=torch.Generator().manual_seed(3))
+    sin = torch.cat([ang, ang], -1).sin()
+    out = onr.rope(q, _rows(cache, b, s), _rows(sin, b, s), h, d)
+    assert torch.allclose(out[s:], onr.rope(q[s:], cache[:s], sin[:s], h, d))
