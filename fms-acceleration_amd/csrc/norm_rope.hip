@@ -365,9 +365,11 @@ constexpr float kLog2e = 1.44269504088896341f;
 constexpr float kLn2 = 0.69314718055994531f;
 
 // (m, s) <- (m, s) (+) (x): running maximum and sum of exp(. - m)
+// While everything seen so far is -inf (a masked vocabulary span) the pair stays (-inf, 0): the update
+// would form (-inf) - (-inf) = NaN, which no later finite logit could remove from s.
 FMSA_DEVI void online_add(float& m, float& s, float x) {
   const float mn = fmaxf(m, x);
-  s = s * __builtin_amdgcn_exp2f((m - mn) * kLog2e) + __builtin_amdgcn_exp2f((x - mn) * kLog2e);
+  if (mn != -INFINITY) s = s * __builtin_amdgcn_exp2f((m - mn) * kLog2e) + __builtin_amdgcn_exp2f((x - mn) * kLog2e);
   m = mn;
 }
 
@@ -386,6 +388,7 @@ __global__ __launch_bounds__(256) void ce_fwd_kernel(const void* __restrict__ lo
 #pragma unroll
       for (int k = 1; k < 8; ++k) mx = fmaxf(mx, x[k]);
       const float mn = fmaxf(m, mx);
+      if (mn == -INFINITY) continue;  // nothing finite yet: (m, s) stays (-inf, 0), see online_add
       float acc = 0.f;
 #pragma unroll
       for (int k = 0; k < 8; ++k) acc += __builtin_amdgcn_exp2f((x[k] - mn) * kLog2e);
@@ -426,7 +429,8 @@ __global__ __launch_bounds__(256) void ce_bwd_kernel(void* __restrict__ logits, 
   const int row = blockIdx.x;
   const int64_t base = (int64_t)row * ld;
   const int64_t label = labels[row];
-  const float dl = label == -100 ? 0.f : dloss[(int64_t)row * dloss_stride];
+  // -100 and any other label outside [0, V) are ignored rows, as in the forward kernel: loss 0, gradient 0
+  const float dl = (label < 0 || label >= V) ? 0.f : dloss[(int64_t)row * dloss_stride];
   const float l = lse[row];
   if (VEC) {
     const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
@@ -487,12 +491,12 @@ __global__ __launch_bounds__(256) void ce_fused_kernel(void* __restrict__ logits
 #pragma unroll
       for (int k = 1; k < 8; ++k) mx = fmaxf(mx, x[k]);
       const float mn = fmaxf(m, mx);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) sx += x[k];
+      if (mn == -INFINITY) continue;  // nothing finite yet: (m, s) stays (-inf, 0), see online_add
       float acc = 0.f;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        acc += __builtin_amdgcn_exp2f((x[k] - mn) * kLog2e);
-        sx += x[k];
-      }
+      for (int k = 0; k < 8; ++k) acc += __builtin_amdgcn_exp2f((x[k] - mn) * kLog2e);
       s = s * __builtin_amdgcn_exp2f((m - mn) * kLog2e) + acc;
       m = mn;
     }
@@ -521,7 +525,9 @@ __global__ __launch_bounds__(256) void ce_fused_kernel(void* __restrict__ logits
   }
   const float lse = red_m[0] + __builtin_amdgcn_logf(red_s[0]) * kLn2;
   const float eps = smoothing / (float)V;
-  if (tid == 0) losses[row] = scale * ((1.0f - smoothing) * (lse - x_label) + (smoothing * lse - eps * red_x[0]));
+  // without smoothing the sum of the logits is not used (it is -inf for a row with masked logits, and 0 * inf is NaN)
+  const float smooth_term = smoothing != 0.f ? smoothing * lse - eps * red_x[0] : 0.f;
+  if (tid == 0) losses[row] = scale * ((1.0f - smoothing) * (lse - x_label) + smooth_term);
   const float hit = 1.0f - smoothing;
   if (VEC) {
     for (int c = 8 * tid; c < V; c += 2048) {
