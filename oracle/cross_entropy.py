@@ -20,8 +20,8 @@ def ce_fwd(logits: torch.Tensor, labels: torch.Tensor):
     x = logits.double()
     c = x.max(dim=-1, keepdim=True).values
     lse = (c + torch.log(torch.exp(x - c).sum(dim=-1, keepdim=True))).squeeze(-1)
-    keep = labels != -100
-    picked = x.gather(1, labels.clamp(min=0).unsqueeze(1)).squeeze(1)
+    keep = (labels >= 0) & (labels < x.shape[1])  # -100 and any other label outside the vocabulary: ignored row
+    picked = x.gather(1, torch.where(keep, labels, torch.zeros_like(labels)).unsqueeze(1)).squeeze(1)
     loss = torch.where(keep, lse - picked, torch.zeros_like(lse))
     return loss.float(), lse.float()
 
@@ -29,7 +29,7 @@ def ce_fwd(logits: torch.Tensor, labels: torch.Tensor):
 def ce_bwd(logits: torch.Tensor, labels: torch.Tensor, lse: torch.Tensor, dloss: torch.Tensor):
     x = logits.double()
     y = torch.exp(x - lse.double().unsqueeze(1))
-    keep = labels != -100
+    keep = (labels >= 0) & (labels < x.shape[1])
     onehot = torch.zeros_like(y)
     onehot[keep, labels[keep]] = 1.0
     dl = torch.where(keep, dloss.double(), torch.zeros_like(dloss.double())).unsqueeze(1)

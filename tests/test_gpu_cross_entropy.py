@@ -37,6 +37,39 @@ def test_cross_entropy_kernels(M, V, dtype):
         assert torch.all(g[M // 2] == 0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("V", [4096, 1003])
+def test_cross_entropy_masked_logits_and_bad_labels(V, dtype):
+    """Rows with a masked (-inf) span of the vocabulary -- at the start of the row, where a thread's first
+    elements are all -inf, and in the middle -- keep a finite loss and gradient (V = 1003 takes the scalar
+    path, V = 4096 the 8-wide one); a label outside [0, V) other than -100 is an ignored row in both passes."""
+    import fmsa_hip
+
+    M = 6
+    x = randn((M, V), 11, dtype, scale=2.0)
+    x[0, :600] = float("-inf")
+    x[1, 300:900] = float("-inf")
+    x[2, V - 200:] = float("-inf")
+    y = torch.tensor([700, 10, 5, V + 3, -7, 2])
+    loss, lse = fmsa_hip.cross_entropy_fwd(x.cuda(), y.cuda())
+    loss_ref, lse_ref = oce.ce_fwd(x, y)
+    assert torch.isfinite(loss).all() and torch.isfinite(lse).all()
+    assert torch.allclose(loss.cpu(), loss_ref, rtol=2e-5, atol=2e-5) and torch.allclose(lse.cpu(), lse_ref, rtol=2e-5, atol=2e-5)
+    assert loss[3].item() == 0.0 and loss[4].item() == 0.0
+    dloss = torch.full((M,), 0.5)
+    g = fmsa_hip.cross_entropy_bwd_(x.cuda().clone(), dloss.cuda(), lse, y.cuda())
+    g_ref = oce.ce_bwd(x.float(), y, lse_ref, dloss)
+    assert torch.isfinite(g).all()
+    tol = 1e-5 if dtype == torch.float32 else 2.0 ** -7
+    assert (g.float().cpu() - g_ref.float()).abs().max().item() <= tol
+    assert torch.all(g[3] == 0) and torch.all(g[4] == 0) and torch.all(g[0, :600] == 0)
+    # the fused loss + gradient launch on the same rows (no smoothing: the sum of the logits is not used)
+    xf = x.cuda().clone()
+    losses, _ = fmsa_hip.cross_entropy_fused_(xf, y.cuda(), scale=None, label_smoothing=0.0)
+    assert torch.isfinite(losses).all() and torch.isfinite(xf).all()
+    assert torch.allclose(losses.cpu(), loss_ref, rtol=2e-5, atol=2e-5)
+
+
 def test_fast_cross_entropy_loss_vs_torch():
     from fms_acceleration_foak.kernels.unsloth import FastCrossEntropyLoss, fast_cross_entropy_loss
 

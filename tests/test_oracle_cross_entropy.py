@@ -73,3 +73,20 @@ def test_fused_linear_ce_matches_autograd():
     # every label ignored under a mean reduction: zero loss and gradients, not NaN
     loss, dx, dw, _ = oce.fused_linear_ce(torch.randn(3, 8), torch.randn(5, 8), torch.full((3,), -100))
     assert float(loss) == 0 and float(dx.abs().max()) == 0 and float(dw.abs().max()) == 0
+
+
+def test_masked_logits_and_labels_outside_the_vocabulary():
+    """-inf logits (a masked span) give the logsumexp of the rest, as torch's own loss does; a label outside [0, V)
+    is an ignored row (loss 0, zero gradient), like -100."""
+    V = 37
+    x = torch.randn(4, V, generator=torch.Generator().manual_seed(1)) * 2
+    x[0, :10] = float("-inf")
+    x[1, 20:] = float("-inf")
+    y = torch.tensor([12, 3, V + 5, -100])
+    loss, lse = oce.ce_fwd(x, y)
+    ref = F.cross_entropy(x[:2], y[:2], reduction="none")
+    assert torch.allclose(loss[:2], ref, atol=1e-6) and loss[2] == 0 and loss[3] == 0
+    assert torch.allclose(lse, torch.logsumexp(x, dim=-1), atol=1e-6)
+    g = oce.ce_bwd(x, y, lse, torch.ones(4))
+    assert torch.isfinite(g).all() and torch.all(g[2] == 0) and torch.all(g[3] == 0) and torch.all(g[0, :10] == 0)
+    assert torch.allclose(g[:2].sum(dim=-1), torch.zeros(2), atol=1e-6)
