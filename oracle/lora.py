@@ -160,3 +160,15 @@ def max_rel_err(out, ref):
     out = out.detach().double().cpu()
     ref = ref.detach().double().cpu()
     return ((out - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
+
+
+def elementwise_rel_err(out, ref, floor=1e-2):
+    """(max, mean) of |out - ref| / |ref| over the entries with |ref| > floor * max |ref|: the element-wise
+    figure reported next to max_rel_err (entries near zero are left out, where a relative error says nothing)."""
+    out = out.detach().double().cpu()
+    ref = ref.detach().double().cpu()
+    keep = ref.abs() > floor * ref.abs().max()
+    if not bool(keep.any()):
+        return 0.0, 0.0
+    rel = (out[keep] - ref[keep]).abs() / ref[keep].abs()
+    return rel.max().item(), rel.mean().item()

@@ -133,3 +133,16 @@ def test_config1_plumbing_on_cpu():
     assert y.shape == (M, N)
     for a, b in ((dx, dx2), (dA, dA2), (dB, dB2)):
         assert olora.max_rel_err(a, b) < 1e-5
+
+
+def test_error_metrics_known_answers():
+    """max_rel_err is relative to the largest reference entry; elementwise_rel_err leaves out entries below
+    the floor (1e-2 of the largest) and returns (max, mean) of the per-entry relative errors of the rest."""
+    ref = torch.tensor([1.0, 2.0, 0.001, -4.0])
+    out = torch.tensor([1.1, 2.0, 0.002, -4.0])
+    assert abs(olora.max_rel_err(out, ref) - 0.1 / 4.0) < 1e-6
+    mx, mean = olora.elementwise_rel_err(out, ref, 1e-2)
+    assert abs(mx - 0.1) < 1e-6 and abs(mean - 0.1 / 3) < 1e-6   # the 0.001 entry (100 % off) is below the floor
+    mx_all, _ = olora.elementwise_rel_err(out, ref, 0.0)
+    assert abs(mx_all - 1.0) < 1e-6
+    assert olora.elementwise_rel_err(torch.zeros(3), torch.zeros(3)) == (0.0, 0.0)
