@@ -318,7 +318,9 @@ _ws_cache = {}
 
 
 def _workspace(nbytes: int, device) -> torch.Tensor:
-    key = (device.type, device.index)
+    """Partial-sum buffer of the adapter-gradient launches, one per (device, stream): launches on one stream
+    are ordered and may share it, launches on two streams of one device must not."""
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
     ws = _ws_cache.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
