@@ -2,6 +2,8 @@
 // the launchers in the kernel translation units.
 #include "common.h"
 
+#include <atomic>
+
 int launch_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, hipStream_t st);
 int launch_gptq_permute_rows(const int32_t* qweight, const int32_t* perm, int K, int N, int32_t* out, hipStream_t st);
 int launch_permute_cols(const void* in, int64_t ld_in, const int32_t* perm, int M, int C, int gather, void* out,
@@ -71,6 +73,26 @@ int check_rank(int r) {
   if (r < 0) return FMSA_ERR_SHAPE;
   if (r % 8 != 0 || r > 128) return FMSA_ERR_UNSUPPORTED;
   return FMSA_OK;
+}
+
+// Partial sums of fmsa_lora_grad_static: device memory that belongs to the library's code object, so the
+// entry point never allocates.  Every GPU the library runs on holds its own copy at its own address; the
+// name below is only a host-side handle (not a device address), so the address is looked up once per device
+// with that device current, and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[FMSA_LORA_GRAD_STATIC_BYTES];
+constexpr int kMaxDevices = 64;
+std::atomic<void*> scratch_ptr[kMaxDevices];
+
+// Address of the current device's copy of `scratch` (nullptr on failure).  Racing first calls look up the
+// same address twice, which is harmless.
+void* scratch_of_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void* p = scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+  scratch_ptr[dev].store(p, std::memory_order_release);
+  return p;
 }
 
 }  // namespace
@@ -173,6 +195,26 @@ int fmsa_lora_grad(const void* L, int64_t ldl, const void* R, int64_t ldr, int M
                    int act_dtype, int out_dtype, void* out, void* workspace, size_t workspace_bytes, void* stream) {
   const fmsa_lora_grad_job job = {L, R, out, ldl, ldr, C, r, scale, transpose_out, out_dtype, 0, nullptr, nullptr, 0};
   return fmsa_lora_grad_batch(&job, 1, M, act_dtype, workspace, workspace_bytes, stream);
+}
+
+int fmsa_lora_grad_static(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale,
+                          int transpose_out, int act_dtype, int out_dtype, void* out, void* stream) {
+  if (M <= 0 || C <= 0 || r <= 0) return FMSA_ERR_SHAPE;
+  // the size check comes before any HIP call: a request beyond the static buffer is an argument error
+  if (fmsa_lora_grad_workspace(M, C, r) > (size_t)FMSA_LORA_GRAD_STATIC_BYTES) return FMSA_ERR_WORKSPACE;
+  const fmsa_lora_grad_job job = {L, R, out, ldl, ldr, C, r, scale, transpose_out, out_dtype, 0, nullptr, nullptr, 0};
+  // validate with a stand-in workspace pointer (non-null, aligned) so that every argument error is reported
+  // before the device is touched; the launch below gets the real address
+  if (!job.L || !job.R || !job.out) return FMSA_ERR_NULL;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  if (ldr < C || ldl < r) return FMSA_ERR_SHAPE;
+  if (C % 8 != 0 || ldr % 8 != 0 || ldl % 8 != 0 || r % 8 != 0 || r > 128) return FMSA_ERR_SHAPE;
+  if (out_dtype != FMSA_F16 && out_dtype != FMSA_BF16 && out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
+  if (!aligned16(R) || !aligned16(L)) return FMSA_ERR_ALIGN;
+  void* ws = scratch_of_current_device();
+  if (!ws) return FMSA_ERR_LAUNCH;
+  // both passes write every partial sum they later read, so the buffer needs no clearing between calls
+  return launch_lora_grad_batch(&job, 1, M, act_dtype, ws, (hipStream_t)stream);
 }
 
 int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,

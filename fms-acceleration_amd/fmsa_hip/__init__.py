@@ -33,6 +33,7 @@ EXPORTED_SYMBOLS = (
     "fmsa_lora_grad",
     "fmsa_lora_grad_batch_workspace",
     "fmsa_lora_grad_batch",
+    "fmsa_lora_grad_static",
     "fmsa_gptq_lora_fwd",
     "fmsa_gptq_lora_bwd_dx",
     "fmsa_swiglu_fwd",
@@ -182,6 +183,8 @@ def lib() -> ctypes.CDLL:
     L.fmsa_lora_grad_batch_workspace.restype = c_size_t
     L.fmsa_lora_grad_batch_workspace.argtypes = [POINTER(LoraGradJob), c_int, c_int]
     L.fmsa_lora_grad_batch.argtypes = [POINTER(LoraGradJob), c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]
+    L.fmsa_lora_grad_static.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                                        c_void_p, c_void_p]
     L.fmsa_gptq_lora_fwd.argtypes = [POINTER(FwdProj), c_int, c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                                      c_int, c_void_p]
     L.fmsa_gptq_lora_bwd_dx.argtypes = [POINTER(BwdProj), c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p,
@@ -339,6 +342,23 @@ def lora_grad(L, R, scale: float, transpose_out: bool, out_dtype=torch.float32):
     _check("fmsa_lora_grad",
            lib().fmsa_lora_grad(_ptr(L), L.stride(0), _ptr(R), R.stride(0), M, C, r, float(scale), int(transpose_out),
                                 act_enum(R.dtype), _DTYPE_ENUM[out_dtype], _ptr(out), _ptr(ws), ws.numel(), _stream(out)))
+    return out
+
+
+LORA_GRAD_STATIC_BYTES = 16 << 20
+
+
+def lora_grad_static(L, R, scale: float, transpose_out: bool, out):
+    """lora_grad through the entry point that allocates nothing: the partial sums go to a buffer inside the
+    library's device image (LORA_GRAD_STATIC_BYTES; larger requests raise), `out` is the caller's.  Calls that
+    overlap on one GPU share that buffer and race."""
+    M, r = L.shape
+    C = R.shape[1]
+    assert R.shape[0] == M and L.stride(1) == 1 and R.stride(1) == 1 and L.dtype == R.dtype
+    assert out.is_contiguous() and tuple(out.shape) == ((C, r) if transpose_out else (r, C))
+    _check("fmsa_lora_grad_static",
+           lib().fmsa_lora_grad_static(_ptr(L), L.stride(0), _ptr(R), R.stride(0), M, C, r, float(scale), int(transpose_out),
+                                       act_enum(R.dtype), _DTYPE_ENUM[out.dtype], _ptr(out), _stream(out)))
     return out
 
 

@@ -150,6 +150,19 @@ size_t fmsa_lora_grad_batch_workspace(const fmsa_lora_grad_job* jobs, int n_jobs
 int fmsa_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int act_dtype, void* workspace,
                          size_t workspace_bytes, void* stream);
 
+/* fmsa_lora_grad for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc); it has no counterpart in the reference.  Same arguments, same two
+ * kernels and bit-identical results, but the partial sums live in a buffer of FMSA_LORA_GRAD_STATIC_BYTES that
+ * is part of the library's device image (each GPU the library is used on holds its own copy until the process
+ * ends), and the call itself makes no hipMalloc / hipFree or any other allocating call.  Returns
+ * FMSA_ERR_WORKSPACE when fmsa_lora_grad_workspace(M, C, r) exceeds that size (16 MiB covers 8192 tokens x
+ * 14336 columns at rank 16, or 4096 columns at rank 64).  All calls on one GPU share the buffer: calls that
+ * overlap in time on one GPU (two streams, two threads) race on it; calls on one stream are ordered.  The very
+ * first call on a device looks up the buffer's address (not an allocation); make that call outside a capture. */
+#define FMSA_LORA_GRAD_STATIC_BYTES (16u << 20)
+int fmsa_lora_grad_static(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale,
+                          int transpose_out, int act_dtype, int out_dtype, void* out, void* stream);
+
 /* The four activation-type copies of one adapter that the kernels above and below read, in one
  * launch: A16 [r, K], At16 [K, r] from A = lora_A.weight [r, K]; B16 [N, r], Bt16 [r, N] from
  * B = lora_B.weight [N, r].  Each value is the parameter rounded once (RNE) to act_dtype -- the

@@ -130,6 +130,18 @@ def test_bwd_and_skinny_validation():
     assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 64, 16, 1, 0x3000, 8, None) == -2   # ldout < r
     assert lib.fmsa_lora_grad_workspace(8192, 4096, 16) > 0
     assert lib.fmsa_lora_grad(0x1000, 16, 0x2000, 64, 8, 64, 16, 1.0, 0, 1, 2, 0x3000, None, 0, None) == -6
+    # the entry point with the built-in scratch buffer: size and argument errors are reported before any HIP call
+    gs = lib.fmsa_lora_grad_static
+    assert lib.fmsa_lora_grad_workspace(8192, 14336, 16) <= fmsa_hip.LORA_GRAD_STATIC_BYTES
+    assert gs(0x1000, 64, 0x2000, 14336, 8192, 14336, 64, 1.0, 0, 1, 2, 0x3000, None) == -6   # 33 MB of partial sums > 16 MiB
+    assert gs(None, 16, 0x2000, 64, 8, 64, 16, 1.0, 0, 1, 2, 0x3000, None) == -1
+    assert gs(0x1000, 16, 0x2000, 64, 8, 64, 16, 1.0, 0, 1, 2, None, None) == -1
+    assert gs(0x1000, 16, 0x2000, 64, 0, 64, 16, 1.0, 0, 1, 2, 0x3000, None) == -2
+    assert gs(0x1000, 16, 0x2000, 32, 8, 64, 16, 1.0, 0, 1, 2, 0x3000, None) == -2             # rows of R shorter than C
+    assert gs(0x1000, 16, 0x2000, 64, 8, 64, 12, 1.0, 0, 1, 2, 0x3000, None) == -2
+    assert gs(0x1000, 16, 0x2000, 64, 8, 64, 16, 1.0, 0, 2, 2, 0x3000, None) == -4             # fp32 is no activation dtype
+    assert gs(0x1000, 16, 0x2000, 64, 8, 64, 16, 1.0, 0, 1, 7, 0x3000, None) == -4
+    assert gs(0x1004, 16, 0x2000, 64, 8, 64, 16, 1.0, 0, 1, 2, 0x3000, None) == -3
     J = fmsa_hip.LoraGradJob
     job = lambda **kw: J(**{**dict(L=0x1000, R=0x2000, out=0x3000, ldl=16, ldr=64, C=64, r=16, scale=1.0, transpose_out=0,
                                    out_dtype=2, reserved=0, Wt=None, T=None, ldt=0), **kw})
