@@ -41,8 +41,11 @@ class PreparedNf4Weight:
 
 def prepare(W, quant_state) -> PreparedNf4Weight:
     data = W.data if isinstance(W, torch.nn.Parameter) else W
+    # no float(offset) here: reading a device scalar would synchronise on every call of the hot path
+    off = quant_state.offset
+    off_key = (off.data_ptr(), off._version) if isinstance(off, torch.Tensor) else float(off)
     key = (data.data_ptr(), data._version, quant_state.absmax.data_ptr(), quant_state.absmax._version,
-           float(quant_state.offset), tuple(quant_state.shape), int(quant_state.blocksize))
+           off_key, tuple(quant_state.shape), int(quant_state.blocksize))
     cached = getattr(W, "_fmsa_prepared", None)
     if cached is None or cached[0] != key:
         cached = (key, PreparedNf4Weight(W, quant_state))

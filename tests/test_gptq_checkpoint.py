@@ -105,3 +105,52 @@ def test_plugin_model_loader_reads_a_local_directory(tmp_path):
     assert loaded.lm_head.weight.dtype == torch.float16
     with pytest.raises(NotImplementedError):
         plugin.model_loader("TheBloke/Llama-2-7B-GPTQ")
+
+
+def test_augmentation_installs_adapters_and_the_fused_rules_trigger(tmp_path):
+    """model_loader -> AutoGPTQ augmentation (adapters from a duck-typed peft_config) -> fast-kernels augmentation
+    -> ModelPatcher: the qkvo and mlp rules fire on the adapted modules (reference: the LoRA layers come from
+    get_gptq_peft_model, framework_plugin_autogptq.py:250-330, and the triggers look for lora_A / lora_B / base_layer,
+    fused-ops-and-kernels models/utils.py:46-49,195-204)."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from fms_acceleration.model_patcher import ModelPatcher, patch_model
+    from fms_acceleration.utils.test_utils import instantiate_model_patcher
+    from fms_acceleration_foak import FastKernelsAccelerationPlugin
+    from fms_acceleration_peft import AutoGPTQAccelerationPlugin, LoraLinear, QuantizeConfig, QuantLinear, save_quantized
+    from fms_acceleration_peft.quantizer import quantize_linear
+
+    cfg = LlamaConfig(hidden_size=64, intermediate_size=128, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=2, vocab_size=64)
+    cfg.architectures = ["LlamaForCausalLM"]
+    model = LlamaForCausalLM(cfg)
+    for name, mod in list(model.named_modules()):
+        if isinstance(mod, torch.nn.Linear) and "lm_head" not in name:
+            setattr(model.get_submodule(name.rsplit(".", 1)[0]), name.rsplit(".", 1)[1], quantize_linear(mod.weight.data, 32))
+    save_quantized(model, str(tmp_path), QuantizeConfig(bits=4, group_size=32, desc_act=False, sym=False))
+    cfg.save_pretrained(str(tmp_path))
+    plugin = AutoGPTQAccelerationPlugin({"peft": {"quantization": {"auto_gptq": {"kernel": "triton_v2", "from_quantized": True}}}})
+    loaded = plugin.model_loader(str(tmp_path), torch_dtype=torch.float16, device="cpu")
+    train_args = type("T", (), {"bf16": False, "fp16": True, "gradient_checkpointing": False})()
+
+    with pytest.raises(AssertionError, match="peft_config"):
+        plugin.augmentation(loaded, train_args, (None,))
+    with pytest.raises(ValueError, match="no QuantLinear module matches"):
+        plugin.augmentation(loaded, train_args, ({"r": 8, "lora_alpha": 16, "target_modules": ["no_such_proj"]},))
+
+    peft_config = type("LoraConfig", (), {"r": 8, "lora_alpha": 16, "lora_dropout": 0.0,
+                                          "target_modules": ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]})()
+    out, args = plugin.augmentation(loaded, train_args, (peft_config,))
+    assert out is loaded and args == (None,)
+    wrapped = [m for m in loaded.modules() if isinstance(m, LoraLinear)]
+    assert len(wrapped) == 14 and all(isinstance(m.base_layer, QuantLinear) and m.scaling["default"] == 2.0 for m in wrapped)
+    trainable = [n for n, p in loaded.named_parameters() if p.requires_grad]
+    assert len(trainable) == 28 and all("lora_" in n for n in trainable)
+
+    foak = FastKernelsAccelerationPlugin({"training": {"fused_ops_and_kernels": {"fused_lora": True, "base_layer": "auto_gptq"}}})
+    with instantiate_model_patcher():
+        foak.augmentation(loaded, train_args, ())
+        patch_model(loaded)
+        done = {h.rule_id for h in ModelPatcher.history}
+        assert "llama-mlp" in done and any(d.startswith("llama-qkvo") for d in done)
+        assert sum(h.rule_id == "llama-mlp" for h in ModelPatcher.history) == 2   # one per decoder layer
