@@ -36,8 +36,9 @@ def fast_dequantize(W, quant_state=None, out_dtype=None):
     transpose the view when they need [K, N]).  Without a quant state W is returned as is."""
     if quant_state is None:
         return W
-    if isinstance(quant_state, list):
-        raise NotImplementedError("list-style (pre-0.42 bitsandbytes) quant states are not supported")
+    from fmsa_hip.nf4_prepared import normalize_quant_state  # the older list form is accepted too (:100-105)
+
+    quant_state = normalize_quant_state(quant_state)
     state2 = quant_state.state2
     if state2 is None or quant_state.absmax.dtype != torch.uint8:
         raise NotImplementedError("only double-quantised NF4 weights (compress_statistics=True) are supported")

@@ -9,14 +9,37 @@ import torch
 import fmsa_hip
 
 
+class _State:
+    """Attribute view of a quant state."""
+
+    def __init__(self, **kw):
+        self.__dict__.update(kw)
+
+
+def normalize_quant_state(quant_state):
+    """bitsandbytes' QuantState object as it is; the older list form
+    `[absmax, shape, dtype, blocksize, [offset, [absmax2, code2, blocksize2, ...]], quant_type, code]`
+    (what fused_ops/unsloth_lora/utils.py:100-105 of the reference unpacks) as an object with the same
+    attribute names."""
+    if not isinstance(quant_state, (list, tuple)):
+        return quant_state
+    if len(quant_state) < 7 or not isinstance(quant_state[4], (list, tuple)) or len(quant_state[4]) != 2:
+        raise NotImplementedError("list-style quant state without compressed statistics (compress_statistics=False)")
+    absmax, shape, dtype, blocksize, (offset, st2) = quant_state[:5]
+    code = quant_state[6]
+    if not isinstance(st2, (list, tuple)) or len(st2) < 3:
+        raise NotImplementedError("list-style quant state: malformed second-level state")
+    state2 = _State(absmax=st2[0], code=st2[1], blocksize=st2[2])
+    return _State(absmax=absmax, shape=tuple(shape), dtype=dtype, blocksize=blocksize, offset=offset, state2=state2, code=code)
+
+
 class PreparedNf4Weight:
     """The C-ABI view (`struct`, code-book format) of one NF4 linear of shape [N, K]."""
 
     __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep")
 
     def __init__(self, W, quant_state):
-        if isinstance(quant_state, list):
-            raise NotImplementedError("list-style (pre-0.42 bitsandbytes) quant states are not supported")
+        quant_state = normalize_quant_state(quant_state)
         state2 = quant_state.state2
         if state2 is None or quant_state.absmax.dtype != torch.uint8:
             raise NotImplementedError("only double-quantised NF4 weights (compress_statistics=True) are supported")
@@ -41,6 +64,7 @@ class PreparedNf4Weight:
 
 def prepare(W, quant_state) -> PreparedNf4Weight:
     data = W.data if isinstance(W, torch.nn.Parameter) else W
+    quant_state = normalize_quant_state(quant_state)
     # no float(offset) here: reading a device scalar would synchronise on every call of the hot path
     off = quant_state.offset
     off_key = (off.data_ptr(), off._version) if isinstance(off, torch.Tensor) else float(off)

@@ -212,3 +212,22 @@ def test_codebook_kernels(M, K, N, r, blocksize, dtype):
                                      "r": r, "s": s}], M, K)
     dx_ref, _, _ = olora.lora_w_manual(x.float(), W, A16.float(), B16.float(), s, dy.float())
     assert olora.max_rel_err(dx.cpu(), dx_ref) < TOL
+
+
+def test_list_style_quant_state_is_accepted():
+    """The older bitsandbytes quant state, a list of lists (reference fused_ops/unsloth_lora/utils.py:100-105), gives
+    the same dense weight and the same prepared weight as the object form; a list without compressed statistics raises."""
+    import fmsa_hip
+    from fms_acceleration_foak.fused_ops.unsloth_lora.utils import fast_dequantize
+    from fms_acceleration_peft.nf4 import quantize_nf4
+    from fmsa_hip.nf4_prepared import PreparedNf4Weight
+
+    W = randn((64, 128), 21, torch.float32).cuda() * 0.02
+    packed, qs = quantize_nf4(W, 64, 256, torch.bfloat16)
+    as_list = [qs.absmax, qs.shape, qs.dtype, qs.blocksize, [qs.offset, [qs.state2.absmax, qs.state2.code, qs.state2.blocksize, None, None, None, None]],
+               "nf4", qs.code]
+    assert torch.equal(fast_dequantize(packed, as_list), fast_dequantize(packed, qs))
+    a, b = PreparedNf4Weight(packed, as_list), PreparedNf4Weight(packed, qs)
+    assert torch.equal(a._keep[0], b._keep[0]) and torch.equal(a._keep[1], b._keep[1])
+    with pytest.raises(NotImplementedError, match="compress_statistics"):
+        fast_dequantize(packed, [qs.absmax, qs.shape, qs.dtype, qs.blocksize, None, "nf4", qs.code])
