@@ -453,6 +453,45 @@ def other_configs(device, dtype, mlp_layer, steps=10, warmup=3):
     return out
 
 
+def yardsticks(device):
+    """What the machine at hand sustains, next to the fused kernels' figures: the vendor library's plain bf16 GEMM of
+    the gate/up shape (no dequantisation, no LoRA, no SwiGLU), and the register-only MFMA loop of the library with
+    zero operands, random operands, and random operands plus the GEMM kernels' ratio of direct-to-LDS loads."""
+    import torch
+
+    import fmsa_hip
+
+    def ev_time(fn, n, warm):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(n):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / n * 1e-3
+
+    gen = torch.Generator(device=device).manual_seed(0)
+    x = torch.randn(M_TOKENS, HIDDEN, generator=gen, device=device).to(torch.bfloat16)
+    w = (torch.randn(HIDDEN, 2 * INTER, generator=gen, device=device) * 0.02).to(torch.bfloat16)
+    y = torch.empty(M_TOKENS, 2 * INTER, dtype=torch.bfloat16, device=device)
+    t = ev_time(lambda: torch.matmul(x, w, out=y), 30, 10)
+    out = {"library_bf16_gemm": {"shape": f"[{M_TOKENS}, {HIDDEN}] x [{HIDDEN}, {2 * INTER}]", "ms": t * 1e3,
+                                 "tflops": 2.0 * M_TOKENS * HIDDEN * 2 * INTER / t / 1e12}}
+    del x, w, y
+    for mode, name in ((0, "mfma_loop_zero_operands"), (1, "mfma_loop_random_operands"), (2, "mfma_loop_random_operands_with_direct_loads")):
+        flop = [0.0]
+
+        def run():
+            flop[0] = fmsa_hip.probe_mfma(mode, 20000, 1024, device)
+
+        t = ev_time(run, 5, 2)  # 5 x about 40 ms: long enough for the clocks to settle under the power limit
+        out[name] = {"ms": t * 1e3, "tflops": flop[0] / t / 1e12}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -467,6 +506,9 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one device copy of 1 GiB (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--yardsticks", action="store_true",
+                    help="instead of the benchmark: time the vendor library's bf16 GEMM of the gate/up shape and the "
+                         "register-only MFMA loop, and print them as one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the fused-LoRA path is data parallel over tokens and this build "
@@ -479,6 +521,9 @@ def main():
         print("bench.py needs an MI355X: no GPU is visible (there is no CPU fallback for the fused path)", file=sys.stderr)
         sys.exit(3)
     device, dtype, M = torch.device("cuda:0"), torch.bfloat16, args.tokens
+    if args.yardsticks:
+        print(json.dumps({"yardsticks": yardsticks(device), "peak_bf16_tflops": PEAK_BF16_TFLOPS}))
+        return
 
     attn, mlp = build_layer(device)
     io = {}

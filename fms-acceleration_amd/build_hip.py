@@ -20,7 +20,7 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfmsa_hip.so")
 
-SOURCES = ["api.hip", "dequant.hip", "gemm_fwd.hip", "gemm_bwd.hip", "lora_skinny.hip", "elementwise.hip", "nf4.hip", "norm_rope.hip"]
+SOURCES = ["api.hip", "dequant.hip", "gemm_fwd.hip", "gemm_bwd.hip", "lora_skinny.hip", "elementwise.hip", "nf4.hip", "norm_rope.hip", "probe.hip"]
 
 # -packed-fp32-ops is switched off on purpose: the packed fp32 VALU forms are not trusted on the
 # target machines, so fp32 math is emitted as scalar-per-lane instructions.

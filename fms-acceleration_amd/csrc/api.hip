@@ -38,6 +38,8 @@ int launch_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64
 int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, int M, int I, int64_t ld, int act_dtype,
                       hipStream_t st);
 
+int launch_probe_mfma(int mode, int iters, int n_workgroups, float* out, const void* src, hipStream_t st);
+
 namespace {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -113,7 +115,7 @@ const char* fmsa_strerror(int code) {
   }
 }
 
-int fmsa_abi_version(void) { return 4; }
+int fmsa_abi_version(void) { return 5; }
 
 int fmsa_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, void* stream) {
   if (!w || !out) return FMSA_ERR_NULL;
@@ -215,6 +217,12 @@ int fmsa_lora_grad_static(const void* L, int64_t ldl, const void* R, int64_t ldr
   if (!ws) return FMSA_ERR_LAUNCH;
   // both passes write every partial sum they later read, so the buffer needs no clearing between calls
   return launch_lora_grad_batch(&job, 1, M, act_dtype, ws, (hipStream_t)stream);
+}
+
+int fmsa_probe_mfma(int mode, int iters, int n_workgroups, void* out, const void* src, void* stream) {
+  if (!out || (mode == 2 && !src)) return FMSA_ERR_NULL;
+  if (mode < 0 || mode > 2 || iters <= 0 || n_workgroups <= 0 || n_workgroups > 65536) return FMSA_ERR_SHAPE;
+  return launch_probe_mfma(mode, iters, n_workgroups, (float*)out, src, (hipStream_t)stream);
 }
 
 int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,

@@ -1,0 +1,71 @@
+// Measurement support, not part of the hot path: a register-only MFMA loop that shows what the matrix pipe of
+// the machine at hand sustains (all-zero operands: clock-bound; random bf16 operands: what the power limit leaves),
+// and the same loop with the GEMM kernels' ratio of direct-to-LDS loads (one 1 KB load per wave and 8 MFMAs),
+// which shows what those loads cost a wave that has nobody to hide behind.
+#include "common.h"
+
+namespace {
+
+FMSA_DEVI uint32_t probe_hash(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x7feb352dU;
+  x ^= x >> 15;
+  x *= 0x846ca68bU;
+  x ^= x >> 16;
+  return x;
+}
+
+// MODE 0: zero operands; 1: random bf16 in +-[1, 2); 2: as 1, plus one buffer_load_dwordx4 ... lds per 8 MFMAs
+template <int MODE>
+__global__ __launch_bounds__(256) void probe_mfma_kernel(float* out, const uint32_t* src, int iters) {
+  __shared__ __attribute__((aligned(1024))) uint32_t lds[8 * 1024];  // 32 KB: one 1 KB slot per (wave, load)
+  f32x16 acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+  u32x4 a[8], b[8];
+#pragma unroll
+  for (int f = 0; f < 8; ++f)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t ha = probe_hash(threadIdx.x * 64 + f * 8 + j + blockIdx.x * 7919), hb = probe_hash(ha + 12345);
+      if (MODE == 0) ha = hb = 0;
+      else {
+        ha = (ha & 0x807f807fu) | 0x3f803f80u;
+        hb = (hb & 0x807f807fu) | 0x3f803f80u;
+      }
+      a[f][j] = ha;
+      b[f][j] = hb;
+    }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(src, 1u << 20);
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      acc[i] = mfma32<bf16_t>(a[i & 7], b[(i >> 1) & 7], acc[i]);
+      if (MODE == 2 && (i & 7) == 0)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(reinterpret_cast<char*>(lds) + (2 * wave + (i >> 3)) * 1024),
+                                                 16, lane * 16, (uint32_t)((it & 63) * 16384 + (2 * wave + (i >> 3)) * 1024), 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  if (MODE == 2) __builtin_amdgcn_s_waitcnt(0x0F70);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s += acc[i][j];
+  out[blockIdx.x * 256 + threadIdx.x] = s + (MODE == 2 ? (float)lds[threadIdx.x] : 0.f);
+}
+
+}  // namespace
+
+int launch_probe_mfma(int mode, int iters, int n_workgroups, float* out, const void* src, hipStream_t st) {
+  dim3 grid(n_workgroups), block(256);
+  if (mode == 0) hipLaunchKernelGGL(probe_mfma_kernel<0>, grid, block, 0, st, out, (const uint32_t*)src, iters);
+  else if (mode == 1) hipLaunchKernelGGL(probe_mfma_kernel<1>, grid, block, 0, st, out, (const uint32_t*)src, iters);
+  else hipLaunchKernelGGL(probe_mfma_kernel<2>, grid, block, 0, st, out, (const uint32_t*)src, iters);
+  FMSA_CHECK_LAUNCH();
+  return FMSA_OK;
+}

@@ -49,6 +49,7 @@ EXPORTED_SYMBOLS = (
     "fmsa_cross_entropy_fwd",
     "fmsa_cross_entropy_bwd",
     "fmsa_cross_entropy_fused",
+    "fmsa_probe_mfma",
 )
 
 
@@ -205,6 +206,7 @@ def lib() -> ctypes.CDLL:
                                       c_int, c_void_p]
     L.fmsa_cross_entropy_fwd.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.fmsa_cross_entropy_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]
+    L.fmsa_probe_mfma.argtypes = [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.fmsa_cross_entropy_fused.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int64, c_void_p, c_float, c_void_p, c_void_p]
     for name in EXPORTED_SYMBOLS:
         getattr(L, name)  # AttributeError here means the library is stale: rebuild it
@@ -609,3 +611,11 @@ def cross_entropy_fused_(logits2d, labels, scale=None, label_smoothing=0.0, igno
                                           int(ignore_index), _ptr(scale) if scale is not None else None, float(label_smoothing),
                                           _ptr(losses), _stream(logits2d)))
     return losses, logits2d
+
+
+def probe_mfma(mode: int, iters: int = 20000, n_workgroups: int = 1024, device="cuda"):
+    """Launches the register-only MFMA loop (see fmsa_probe_mfma in include/fmsa.h); returns its FLOP count."""
+    out = torch.empty(n_workgroups * 256, dtype=torch.float32, device=device)
+    src = torch.zeros(1 << 18, dtype=torch.int32, device=device)
+    _check("fmsa_probe_mfma", lib().fmsa_probe_mfma(mode, iters, n_workgroups, _ptr(out), _ptr(src), _stream(out)))
+    return float(n_workgroups) * 4 * iters * 16 * 32768.0

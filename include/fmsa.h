@@ -337,6 +337,17 @@ int fmsa_cross_entropy_fused(void* logits, int64_t ld, const int64_t* labels, in
                              int64_t ignore_index, const float* scale, float label_smoothing, float* losses,
                              void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Measurement support (no counterpart in the reference; used by bench.py --yardsticks).
+ * A register-only loop of `iters` x 16 MFMA 32x32x16 bf16 per wave, 4 waves per workgroup:
+ *   mode 0  all-zero operands (what the clock allows),
+ *   mode 1  random bf16 operands (what the power limit leaves),
+ *   mode 2  as 1, plus one 1 KB direct-to-LDS load per wave and 8 MFMAs from `src` (>= 1 MiB), the
+ *           ratio of the GEMM kernels' main loops.
+ * FLOP of a launch = n_workgroups * 4 * iters * 16 * 32768.  `out`: n_workgroups * 256 floats.
+ * ------------------------------------------------------------------------------------------ */
+int fmsa_probe_mfma(int mode, int iters, int n_workgroups, void* out, const void* src, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
