@@ -453,6 +453,41 @@ def other_configs(device, dtype, mlp_layer, steps=10, warmup=3):
     return out
 
 
+def qkv_rope_config(device, dtype, attn, steps=200, warmup=20):
+    """Forward of the Q / K / V projections with the rotary embedding of Q and K: applied in the epilogue of the
+    projection launch (apply_lora_qkv_rope) against the projections followed by the in-place rotary kernel on Q and
+    on K (what the reference's fast_rope_embedding does after its fused projections)."""
+    import torch
+
+    import fmsa_hip
+    from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_qkv, apply_lora_qkv_rope
+
+    attn.head_dim = HEAD_DIM
+    x = torch.randn(1, M_TOKENS, HIDDEN, generator=torch.Generator(device=device).manual_seed(5), device=device).to(dtype)
+    ang = torch.outer(torch.arange(M_TOKENS).float(), 1.0 / (10000 ** (torch.arange(0, HEAD_DIM, 2).float() / HEAD_DIM)))
+    emb = torch.cat([ang, ang], -1)
+    cos, sin = emb.cos().to(dtype).to(device), emb.sin().to(dtype).to(device)
+
+    def plain():
+        with torch.no_grad():
+            apply_lora_qkv(attn, x)
+
+    def separate():
+        with torch.no_grad():
+            Q, K, _ = apply_lora_qkv(attn, x)
+            fmsa_hip.rope_embedding_(Q.view(M_TOKENS, -1), cos, sin, N_HEADS, HEAD_DIM)
+            fmsa_hip.rope_embedding_(K.view(M_TOKENS, -1), cos, sin, N_KV, HEAD_DIM)
+
+    def fused():
+        with torch.no_grad():
+            apply_lora_qkv_rope(attn, x, cos, sin)
+
+    us = {k: time_steps(f, steps, warmup) * 1e6 for k, f in (("projections_only", plain), ("separate_passes", separate), ("in_epilogue", fused))}
+    return {"workload": "LoRA_QKV forward + rotary embedding of Q and K, 8192 tokens, 32 + 8 heads of 128, bf16 tables",
+            "us_projections_only": us["projections_only"], "us_with_separate_rope_passes": us["separate_passes"],
+            "us_with_rope_in_epilogue": us["in_epilogue"]}
+
+
 def yardsticks(device):
     """What the machine at hand sustains, next to the fused kernels' figures: the vendor library's plain bf16 GEMM of
     the gate/up shape (no dequantisation, no LoRA, no SwiGLU), and the register-only MFMA loop of the library with
@@ -626,9 +661,11 @@ def main():
         result["cpu_baseline"] = cpu_base
     if not args.no_other_configs:
         del step
+        rope_cfg = qkv_rope_config(device, dtype, attn)
         attn = None
         torch.cuda.empty_cache()
         result["other_configs"] = other_configs(device, dtype, mlp)
+        result["other_configs"]["qkv_with_rope_llama3_8b"] = rope_cfg
     print(json.dumps(result))
 
 

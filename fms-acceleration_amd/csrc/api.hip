@@ -14,7 +14,7 @@ int lora_grad_splits(int M, int C);
 size_t lora_grad_batch_workspace(const fmsa_lora_grad_job* jobs, int n_jobs, int M);
 int launch_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int act_dtype, void* workspace, hipStream_t st);
 int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,
-                         int64_t ldh, int act_dtype, hipStream_t st);
+                         int64_t ldh, const fmsa_rope* rope, int act_dtype, hipStream_t st);
 int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx, void* e,
                             void* g, void* h_out, int64_t ldeg, int act_dtype, hipStream_t st);
 
@@ -225,8 +225,8 @@ int fmsa_probe_mfma(int mode, int iters, int n_workgroups, void* out, const void
   return launch_probe_mfma(mode, iters, n_workgroups, (float*)out, src, (hipStream_t)stream);
 }
 
-int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,
-                       int64_t ldh, int act_dtype, void* stream) {
+static int check_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, const void* H,
+                     int64_t ldh, int act_dtype) {
   if (!projs || !X) return FMSA_ERR_NULL;
   if (n_proj < 1 || n_proj > 3 || M <= 0) return FMSA_ERR_SHAPE;
   if (mode != FMSA_FWD_LINEAR && mode != FMSA_FWD_SWIGLU) return FMSA_ERR_SHAPE;
@@ -256,7 +256,36 @@ int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, in
     if (ldh < projs[0].w.N) return FMSA_ERR_SHAPE;
     if (!aligned16(H) || ldh % 8 != 0) return FMSA_ERR_ALIGN;
   }
-  return launch_gptq_lora_fwd(projs, n_proj, X, ldx, M, mode, H, ldh, act_dtype, (hipStream_t)stream);
+  return FMSA_OK;
+}
+
+int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,
+                       int64_t ldh, int act_dtype, void* stream) {
+  if (int rc = check_fwd(projs, n_proj, X, ldx, M, mode, H, ldh, act_dtype)) return rc;
+  return launch_gptq_lora_fwd(projs, n_proj, X, ldx, M, mode, H, ldh, nullptr, act_dtype, (hipStream_t)stream);
+}
+
+int fmsa_gptq_lora_fwd_rope(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, const fmsa_rope* rope,
+                            int act_dtype, void* stream) {
+  if (!projs || !X || !rope) return FMSA_ERR_NULL;
+  if (!rope->cos || !rope->sin) return FMSA_ERR_NULL;
+  if (n_proj < 1 || n_proj > 3 || M <= 0) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  if (rope->dtype != act_dtype && rope->dtype != FMSA_F32) return FMSA_ERR_DTYPE;
+  const int hd = rope->head_dim;
+  if (hd <= 0 || rope->rows <= 0 || rope->ld < hd / 2) return FMSA_ERR_SHAPE;
+  if (hd % 16 != 0 || 256 % hd != 0) return FMSA_ERR_UNSUPPORTED;
+  if (rope->proj_mask < 0 || rope->proj_mask >= (1 << n_proj)) return FMSA_ERR_SHAPE;
+  if (!aligned16(rope->cos) || !aligned16(rope->sin) || rope->ld % (rope->dtype == FMSA_F32 ? 4 : 8) != 0) return FMSA_ERR_ALIGN;
+  // the checks of the plain forward (pointers, shapes, alignment), then what the rotating flavour of the kernel adds
+  if (int rc = check_fwd(projs, n_proj, X, ldx, M, FMSA_FWD_LINEAR, nullptr, 0, act_dtype)) return rc;
+  const int K = projs[0].w.K;
+  for (int p = 0; p < n_proj; ++p) {
+    if (((rope->proj_mask >> p) & 1) && projs[p].w.N % hd != 0) return FMSA_ERR_SHAPE;
+    if (projs[p].w.group_size <= 0 || projs[p].w.group_size % 64 != 0) return FMSA_ERR_UNSUPPORTED;
+  }
+  if (K % 64 != 0) return FMSA_ERR_UNSUPPORTED;
+  return launch_gptq_lora_fwd(projs, n_proj, X, ldx, M, FMSA_FWD_LINEAR, nullptr, 0, rope, act_dtype, (hipStream_t)stream);
 }
 
 int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx, void* e,

@@ -54,6 +54,11 @@ struct FwdArgs {
   int M, K, mode, nbm, nbn;
   uint16_t* H;
   int64_t ldh;
+  // rotary embedding in the epilogue (linear mode): projections whose bit is set in rope_mask leave rotated
+  const void* rope_cos;
+  const void* rope_sin;
+  int64_t rope_ld;
+  int rope_rows, rope_head_dim, rope_mask;
 };
 
 // a.p[p] for a runtime (wave-uniform) p without dynamic indexing of the kernel-argument struct,
@@ -63,7 +68,11 @@ FMSA_DEVI FwdProjDev select_proj(const FwdArgs& a, int p) { return p == 0 ? a.p[
 // GPS = scale groups per 64-wide K stage: 1 for group_size % 64 == 0, 2 / 4 for group sizes 32 / 16.
 // CODEBOOK: the nibbles index a 16-entry table and one fp32 scale per (group, column) multiplies the
 // entry (W = code[q] * block_scale); otherwise the affine GPTQ form W = scale * (q - zero).
-template <typename T, int GPS, bool KTAIL, bool CODEBOOK>
+// ROPE (1: cos / sin tables in the activation type, 2: in fp32; 0: none): the Q / K projections of an attention block
+// leave the kernel with the rotary embedding applied
+// (kernels/unsloth/rope_embedding.py:36-65 of the reference: (q1, q2) <- (q1 cos - q2 sin, q2 cos + q1 sin) on the two
+// halves of every head, on the projection output ROUNDED to the storage type, fp32 arithmetic, one more rounding).
+template <typename T, int GPS, bool KTAIL, bool CODEBOOK, int ROPE = 0>
 __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // two separate arrays (not one 2-D array): every access names its buffer statically, which is
   // what lets the compiler see that fragment reads of one buffer do not depend on the direct loads
@@ -571,10 +580,52 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
       }
     }
   }
+  // rotary embedding (ROPE flavour, tiles of a projection named by rope_mask): the thread's pair of half-head chunks
+  bool rope_on = false;
+  int rp_row = 0, rp_c1 = 0, rp_c2 = 0, rp_cw = 0, rp_pos0 = 0;
+  uint32_t rp_voff = 0;
+  u32x4 rp_c[EP_ROWS / 16][2], rp_s[EP_ROWS / 16][2];  // cos / sin of the pair's 8 columns per sweep of the pass, as loaded:
+                                                       // one 16-byte word of 16-bit values or two of fp32
+  if constexpr (ROPE != 0) {
+    rope_on = ((a.rope_mask >> pj[0]) & 1) != 0;
+    const int hd = a.rope_head_dim, hpc = hd >> 4;  // 8-column chunks per half head (a power of two)
+    const int pi = tid & 15;
+    const int head = pi >> (31 - __builtin_clz(hpc)), within = pi & (hpc - 1);
+    rp_row = tid >> 4;
+    rp_c1 = head * (hd >> 3) + within;
+    rp_c2 = rp_c1 + hpc;
+    rp_cw = 8 * within;
+    rp_pos0 = (m0 + rp_row) % a.rope_rows;
+    rp_voff = (uint32_t)((rp_row * ld0 + cb + 8 * rp_c1) * 2) | ((cb + 8 * rp_c1) < n_out ? 0u : 0x80000000u);
+  }
   __syncthreads();  // (the stage buffers are not reused, but all waves are past the main loop)
 
   static_for<0, MT / 2>([&](auto q_c) {
     constexpr int q = decltype(q_c)::value;
+    if constexpr (ROPE != 0) {
+      // cos / sin of this pass's rows, asked for before the accumulators are packed so that they arrive behind that work
+      if (rope_on) {
+        static_for<0, EP_ROWS / 16>([&](auto it_c) {
+          constexpr int it = decltype(it_c)::value;
+          int pos = rp_pos0 + EP_ROWS * q + 16 * it;  // token row m0 + ... takes table row (token row) % rope_rows
+          if (pos >= a.rope_rows) pos %= a.rope_rows;
+          const int64_t cso = (int64_t)pos * a.rope_ld + rp_cw;
+          // kept as loaded and unpacked where they are used: an ALU operation here would make the wave wait for the load
+          // before it goes on to pack its accumulators
+          if constexpr (ROPE == 2) {
+            const u32x4* cp = reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(a.rope_cos) + cso);
+            const u32x4* sp = reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(a.rope_sin) + cso);
+            rp_c[it][0] = cp[0];
+            rp_c[it][1] = cp[1];
+            rp_s[it][0] = sp[0];
+            rp_s[it][1] = sp[1];
+          } else {
+            rp_c[it][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(a.rope_cos) + cso);
+            rp_s[it][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(a.rope_sin) + cso);
+          }
+        });
+      }
+    }
     static_for<0, 2>([&](auto ml_c) {
       constexpr int ml = decltype(ml_c)::value;
       constexpr int mt = 2 * q + ml;
@@ -627,12 +678,46 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
         __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane2 + o), h_rsrc, h_voff, srow * h_row, STORE_NT);
       }
     } else {
+      if (ROPE != 0 && rope_on) {
+        // Two half-head chunks per thread: 8 columns of the first half of a head and the 8 columns half a head
+        // further (heads do not straddle the 256-column tile), so every cos / sin value is loaded and unpacked once
+        // for the two outputs it makes.  16 pairs per row, 16 rows per sweep.
+        static_for<0, EP_ROWS / 16>([&](auto it_c) {
+          constexpr int it = decltype(it_c)::value;
+          const int row = rp_row + 16 * it;
+          const uint32_t srow = (uint32_t)(EP_ROWS * q + 16 * it);
+          u32x4 v1 = *reinterpret_cast<const u32x4*>(plane0 + row * EP_STRIDE_L + 8 * rp_c1);
+          u32x4 v2 = *reinterpret_cast<const u32x4*>(plane0 + row * EP_STRIDE_L + 8 * rp_c2);
+          static_for<0, 4>([&](auto w_c) {
+            constexpr int w = decltype(w_c)::value;  // values 2w and 2w + 1 of the 8 columns
+            float c0, c1, s0, s1;
+            if constexpr (ROPE == 2) {
+              c0 = __uint_as_float(rp_c[it][w >> 1][2 * (w & 1)]);
+              c1 = __uint_as_float(rp_c[it][w >> 1][2 * (w & 1) + 1]);
+              s0 = __uint_as_float(rp_s[it][w >> 1][2 * (w & 1)]);
+              s1 = __uint_as_float(rp_s[it][w >> 1][2 * (w & 1) + 1]);
+            } else {
+              c0 = unpack_lo<T>(rp_c[it][0][w]);
+              c1 = unpack_hi<T>(rp_c[it][0][w]);
+              s0 = unpack_lo<T>(rp_s[it][0][w]);
+              s1 = unpack_hi<T>(rp_s[it][0][w]);
+            }
+            const float a0 = unpack_lo<T>(v1[w]), a1 = unpack_hi<T>(v1[w]);  // first half of the head
+            const float b0 = unpack_lo<T>(v2[w]), b1 = unpack_hi<T>(v2[w]);  // second half
+            v1[w] = pack2<T>(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+            v2[w] = pack2<T>(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+          });
+          __builtin_amdgcn_raw_buffer_store_b128(v1, y0_rsrc, rp_voff, srow * y0_row, STORE_NT);
+          __builtin_amdgcn_raw_buffer_store_b128(v2, y0_rsrc, rp_voff + (uint32_t)(a.rope_head_dim), srow * y0_row, STORE_NT);
+        });
+      } else {
 #pragma unroll
-      for (int it = 0; it < EP_ROWS / 8; ++it) {
-        const int row = crow + 8 * it;
-        const uint32_t srow = (uint32_t)(EP_ROWS * q + 8 * it);
-        __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane0 + row * EP_STRIDE_L + 8 * cchunk), y0_rsrc,
-                                               y0_voff, srow * y0_row, STORE_NT);
+        for (int it = 0; it < EP_ROWS / 8; ++it) {
+          const int row = crow + 8 * it;
+          const uint32_t srow = (uint32_t)(EP_ROWS * q + 8 * it);
+          __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(plane0 + row * EP_STRIDE_L + 8 * cchunk), y0_rsrc,
+                                                 y0_voff, srow * y0_row, STORE_NT);
+        }
       }
     }
     __syncthreads();
@@ -645,8 +730,16 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 }  // namespace
 
 int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode,
-                         void* H, int64_t ldh, int act_dtype, hipStream_t st) {
+                         void* H, int64_t ldh, const fmsa_rope* rope, int act_dtype, hipStream_t st) {
   FwdArgs a{};
+  if (rope) {
+    a.rope_cos = rope->cos;
+    a.rope_sin = rope->sin;
+    a.rope_ld = rope->ld;
+    a.rope_rows = rope->rows;
+    a.rope_head_dim = rope->head_dim;
+    a.rope_mask = rope->proj_mask;
+  }
   a.X = (const uint16_t*)X;
   a.ldx = ldx;
   a.M = M;
@@ -692,7 +785,9 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
   const bool codebook = projs[0].w.format == FMSA_WEIGHT_CODEBOOK;  // api.hip: all projections of a launch share the format
 #define LAUNCH3(TT, KT, CB)                                                                          \
   do {                                                                                               \
-    if (gps == 1) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, KT, CB>), grid, block, 0, st, a);  \
+    if (rope && rope->dtype == FMSA_F32) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, false, CB, 2>), grid, block, 0, st, a); \
+    else if (rope) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, false, CB, 1>), grid, block, 0, st, a); /* api.hip: gps 1, no K tail */ \
+    else if (gps == 1) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, KT, CB>), grid, block, 0, st, a);  \
     else if (gps == 2) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 2, KT, CB>), grid, block, 0, st, a); \
     else hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 4, KT, CB>), grid, block, 0, st, a);           \
   } while (0)

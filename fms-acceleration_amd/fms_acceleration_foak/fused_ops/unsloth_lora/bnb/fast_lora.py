@@ -73,6 +73,35 @@ class LoRA_QKV(torch.autograd.Function):
                 None, None, None)
 
 
+class LoRA_QKV_RoPE(torch.autograd.Function):
+    """LoRA_QKV whose Q and K leave with the rotary position embedding applied in the epilogue of the projection
+    kernel (the NF4 twin of gptq/fast_lora.py's LoRA_QKV_RoPE here; kernels/unsloth/rope_embedding.py:36-65 of the
+    reference is the separate pass it replaces)."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, X, cos, sin, head_dim,
+                QW, QW_quant, Q_bias, QA, QB, QS,
+                KW, KW_quant, K_bias, KA, KB, KS,
+                VW, VW_quant, V_bias, VA, VB, VS,
+                dropout_Q=None, dropout_K=None, dropout_V=None):
+        dtype = _act_dtype(X)
+        projs = [_proj(QW, QW_quant, Q_bias, QA, QB, QS, dtype), _proj(KW, KW_quant, K_bias, KA, KB, KS, dtype),
+                 _proj(VW, VW_quant, V_bias, VA, VB, VS, dtype)]
+        return core.qkv_forward(ctx, X, projs, (dropout_Q, dropout_K, dropout_V), dtype, rope=(cos, sin, int(head_dim)))
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dQ, dK, dV):
+        dX, grads = core.qkv_backward(ctx, dQ, dK, dV)
+        n3 = (None,) * 3
+        return (dX, None, None, None,
+                *n3, grads[0][0], grads[0][1], None,
+                *n3, grads[1][0], grads[1][1], None,
+                *n3, grads[2][0], grads[2][1], None,
+                None, None, None)
+
+
 def swiglu_fg_kernel(e, g):
     """h = silu(e) * g (reference: fused_ops/unsloth_lora/swiglu.py:40-47)."""
     return fmsa_hip.swiglu_fwd(e, g)
@@ -134,6 +163,23 @@ def apply_lora_qkv(self, X):
                           KW, KW_quant, K_bias, KA, KB, KS,
                           VW, VW_quant, V_bias, VA, VB, VS,
                           dropoutQ, dropoutK, dropoutV)
+
+
+def apply_lora_qkv_rope(self, X, cos, sin):
+    """apply_lora_qkv with the rotary embedding of Q and K fused into the projection launch (see the GPTQ twin)."""
+    from ..gptq.fast_lora import rope_tables
+
+    QW, QW_quant, Q_bias, QA, QB, QS, dropoutQ = get_lora_parameters(self.q_proj)
+    KW, KW_quant, K_bias, KA, KB, KS, dropoutK = get_lora_parameters(self.k_proj)
+    VW, VW_quant, V_bias, VA, VB, VS, dropoutV = get_lora_parameters(self.v_proj)
+    batch, seq_len = (X.shape[0], X.shape[1]) if X.dim() == 3 else (1, X.shape[0])
+    cos2d, sin2d = rope_tables(cos, sin, batch, seq_len)
+    head_dim = getattr(self, "head_dim", None) or self.config.head_dim
+    return LoRA_QKV_RoPE.apply(X, cos2d, sin2d, head_dim,
+                               QW, QW_quant, Q_bias, QA, QB, QS,
+                               KW, KW_quant, K_bias, KA, KB, KS,
+                               VW, VW_quant, V_bias, VA, VB, VS,
+                               dropoutQ, dropoutK, dropoutV)
 
 
 def apply_lora_o(self, X):

@@ -229,14 +229,41 @@ def _lora_down_all(projs, Xds, stack):
     return [fmsa_hip.lora_down(Xd, p.A) if p.r else None for p, Xd in zip(projs, Xds)]
 
 
-def _linear_forward(projs, X2, Xds, stack=None):
+def _rope_in_epilogue(projs, rope, dtype):
+    """Whether the forward kernel can apply the rotary embedding itself (fmsa_gptq_lora_fwd_rope): group sizes and
+    K in whole 64-wide stages, heads that do not straddle its 256-column tiles, tables of the activation type or
+    fp32 whose rows start on 16-byte boundaries."""
+    cos2d, sin2d, head_dim, mask = rope
+    K = projs[0].w.K
+    esz = cos2d.element_size()
+    return (K % 64 == 0 and head_dim % 16 == 0 and 256 % head_dim == 0
+            and cos2d.dtype in (dtype, torch.float32) and sin2d.dtype == cos2d.dtype
+            and cos2d.stride() == sin2d.stride() and (cos2d.stride(0) * esz) % 16 == 0
+            and cos2d.data_ptr() % 16 == 0 and sin2d.data_ptr() % 16 == 0
+            and all(p.w.group_size % 64 == 0 for p in projs)
+            and all(p.w.N % head_dim == 0 for i, p in enumerate(projs) if (mask >> i) & 1))
+
+
+def _linear_forward(projs, X2, Xds, stack=None, rope=None):
     """Y_p = X deq(W_p) + s U_p B_p^T for projections sharing X2.  One launch when the weights walk K in one
-    order (on X in that order); otherwise one launch per projection on its own column-permuted copy of X."""
+    order (on X in that order); otherwise one launch per projection on its own column-permuted copy of X.
+    rope = (cos2d, sin2d, head_dim, mask): the projections named by the mask leave with the rotary embedding
+    applied, in the kernel's epilogue where it can, by the in-place kernel otherwise."""
     Us = _lora_down_all(projs, Xds, stack)
+    fused_rope = rope is not None and _rope_in_epilogue(projs, rope, X2.dtype)
     if _one_order(projs):
-        outs = fmsa_hip.gptq_lora_fwd(projs[0].to_kernel_order(X2), [p.fwd_dict(U) for p, U in zip(projs, Us)])
+        outs = fmsa_hip.gptq_lora_fwd(projs[0].to_kernel_order(X2), [p.fwd_dict(U) for p, U in zip(projs, Us)],
+                                      rope=rope if fused_rope else None)
     else:
-        outs = [fmsa_hip.gptq_lora_fwd(p.to_kernel_order(X2), [p.fwd_dict(U)])[0] for p, U in zip(projs, Us)]
+        outs = []
+        for i, (p, U) in enumerate(zip(projs, Us)):
+            r1 = (rope[0], rope[1], rope[2], 1) if fused_rope and (rope[3] >> i) & 1 else None
+            outs.append(fmsa_hip.gptq_lora_fwd(p.to_kernel_order(X2), [p.fwd_dict(U)], rope=r1)[0])
+    if rope is not None and not fused_rope:
+        cos2d, sin2d, head_dim, mask = rope
+        for i, (p, y) in enumerate(zip(projs, outs)):
+            if (mask >> i) & 1:
+                fmsa_hip.rope_embedding_(y, cos2d, sin2d, p.w.N // head_dim, head_dim, backward=False)
     return outs, Us
 
 
@@ -318,11 +345,14 @@ def w_backward(ctx, dY):
     return dX.view(ctx.x_shape).to(ctx.x_dtype), dA, dB
 
 
-def qkv_forward(ctx, X, projs, dropouts, dtype):
+def qkv_forward(ctx, X, projs, dropouts, dtype, rope=None):
+    """rope = (cos2d, sin2d, head_dim): Q and K leave rotated (rows of the [positions, >= head_dim / 2] tables are
+    taken as token row % positions)."""
     X2 = _as2d(X, dtype)
     Xds = _dropped_inputs(X2, projs, dropouts)
     stack = _pack_group(projs, Xds, dtype)
-    outs, Us = _linear_forward(projs, X2, Xds, stack)
+    ctx.rope = None if rope is None else (rope[0], rope[1], rope[2], 0b011)
+    outs, Us = _linear_forward(projs, X2, Xds, stack, ctx.rope)
     ctx.projs, ctx.stack = projs, stack
     ctx.act_dtype = dtype
     ctx.x_shape, ctx.x_dtype = X.shape, X.dtype
@@ -343,6 +373,16 @@ def qkv_backward(ctx, dQ, dK, dV):
     saved = list(ctx.saved_tensors)
     K = projs[0].w.K
     dYs = [_as2d(dY, ctx.act_dtype) for dY in (dQ, dK, dV)]  # dK may arrive non-contiguous (gptq/fast_lora.py:631)
+    if getattr(ctx, "rope", None) is not None:
+        # gradients of the rotated outputs -> gradients of the projections: the inverse rotation (sin negated,
+        # kernels/unsloth/rope_embedding.py:105-128), on copies where autograd handed us its own tensors
+        cos2d, sin2d, head_dim, mask = ctx.rope
+        for i, (dY_in, p) in enumerate(zip((dQ, dK, dV), projs)):
+            if (mask >> i) & 1:
+                d = dYs[i]
+                if d.data_ptr() == dY_in.data_ptr():
+                    d = d.clone()
+                dYs[i] = fmsa_hip.rope_embedding_(d, cos2d, sin2d, p.w.N // head_dim, head_dim, backward=True)
     Xds, Us = [], []
     for has in ctx.layout:
         Xds.append(saved.pop(0) if has else None)

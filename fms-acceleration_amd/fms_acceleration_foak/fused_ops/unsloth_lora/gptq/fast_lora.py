@@ -169,6 +169,43 @@ class LoRA_QKV(torch.autograd.Function):
         )
 
 
+class LoRA_QKV_RoPE(torch.autograd.Function):
+    """LoRA_QKV whose Q and K leave with the rotary position embedding applied (the forward kernel rotates in its
+    epilogue instead of a separate pass of kernels/unsloth/rope_embedding.py over Q and K); V is untouched.  cos / sin:
+    [positions, head_dim] tables (or [batch * seq, head_dim], used row by row); the token at flattened row m takes
+    table row m % positions.  The backward rotates dQ and dK back before the LoRA_QKV backward."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(
+        ctx, X, cos, sin, head_dim,
+        Q_qweight, Q_scales, Q_qzeros, Q_g_idx, Q_bits, Q_bias, QA, QB, QS,
+        K_qweight, K_scales, K_qzeros, K_g_idx, K_bits, K_bias, KA, KB, KS,
+        V_qweight, V_scales, V_qzeros, V_g_idx, V_bits, V_bias, VA, VB, VS,
+        dropout_Q=None, dropout_K=None, dropout_V=None,
+    ):
+        dtype = _act_dtype(X)
+        projs = [
+            _proj((Q_qweight, Q_scales, Q_qzeros, Q_g_idx, Q_bits, Q_bias, QA, QB, QS), dtype),
+            _proj((K_qweight, K_scales, K_qzeros, K_g_idx, K_bits, K_bias, KA, KB, KS), dtype),
+            _proj((V_qweight, V_scales, V_qzeros, V_g_idx, V_bits, V_bias, VA, VB, VS), dtype),
+        ]
+        return core.qkv_forward(ctx, X, projs, (dropout_Q, dropout_K, dropout_V), dtype, rope=(cos, sin, int(head_dim)))
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dQ, dK, dV):
+        dX, grads = core.qkv_backward(ctx, dQ, dK, dV)
+        n6 = (None,) * 6
+        return (
+            dX, None, None, None,
+            *n6, grads[0][0], grads[0][1], None,
+            *n6, grads[1][0], grads[1][1], None,
+            *n6, grads[2][0], grads[2][1], None,
+            None, None, None,
+        )
+
+
 # ----------------------------------------------------------------------------------------------
 # LoRA_MLP  (SwiGLU)
 # ----------------------------------------------------------------------------------------------
@@ -224,6 +261,33 @@ def apply_lora_qkv(self, X):
     Vqstate, V_bias, VA, VB, VS, Vdropout = get_lora_parameters(self.v_proj)
     return LoRA_QKV.apply(
         X,
+        *unpack_gptqstate(Qqstate), Q_bias, QA, QB, QS,
+        *unpack_gptqstate(Kqstate), K_bias, KA, KB, KS,
+        *unpack_gptqstate(Vqstate), V_bias, VA, VB, VS,
+        Qdropout, Kdropout, Vdropout,
+    )
+
+
+def rope_tables(cos, sin, batch, seq_len):
+    """cos / sin as transformers passes them ([1 or batch, seq, head_dim], or a [positions, head_dim] cache) ->
+    contiguous-row 2-D tables for the kernels: a shared table is cut to seq_len rows (every batch entry restarts at
+    position 0), a per-batch table is flattened to [batch * seq, head_dim]."""
+    from ....kernels.unsloth.rope_embedding import _rows
+
+    return _rows(cos, batch, seq_len), _rows(sin, batch, seq_len)
+
+
+def apply_lora_qkv_rope(self, X, cos, sin):
+    """apply_lora_qkv with the rotary embedding of Q and K fused into the projection launch.  X [batch, seq, hidden];
+    returns (Q, K, V) as [batch, seq, N]; `self.head_dim` (or config.head_dim) gives the head size."""
+    Qqstate, Q_bias, QA, QB, QS, Qdropout = get_lora_parameters(self.q_proj)
+    Kqstate, K_bias, KA, KB, KS, Kdropout = get_lora_parameters(self.k_proj)
+    Vqstate, V_bias, VA, VB, VS, Vdropout = get_lora_parameters(self.v_proj)
+    batch, seq_len = (X.shape[0], X.shape[1]) if X.dim() == 3 else (1, X.shape[0])
+    cos2d, sin2d = rope_tables(cos, sin, batch, seq_len)
+    head_dim = getattr(self, "head_dim", None) or self.config.head_dim
+    return LoRA_QKV_RoPE.apply(
+        X, cos2d, sin2d, head_dim,
         *unpack_gptqstate(Qqstate), Q_bias, QA, QB, QS,
         *unpack_gptqstate(Kqstate), K_bias, KA, KB, KS,
         *unpack_gptqstate(Vqstate), V_bias, VA, VB, VS,

@@ -35,6 +35,7 @@ EXPORTED_SYMBOLS = (
     "fmsa_lora_grad_batch",
     "fmsa_lora_grad_static",
     "fmsa_gptq_lora_fwd",
+    "fmsa_gptq_lora_fwd_rope",
     "fmsa_gptq_lora_bwd_dx",
     "fmsa_swiglu_fwd",
     "fmsa_swiglu_bwd",
@@ -71,6 +72,18 @@ class GptqWeight(Structure):
 
 
 WEIGHT_AFFINE, WEIGHT_CODEBOOK = 0, 1
+
+
+class Rope(Structure):
+    _fields_ = [
+        ("cos", c_void_p),
+        ("sin", c_void_p),
+        ("ld", c_int64),
+        ("rows", c_int32),
+        ("head_dim", c_int32),
+        ("dtype", c_int32),
+        ("proj_mask", c_int32),
+    ]
 
 
 class Nf4Weight(Structure):
@@ -188,6 +201,7 @@ def lib() -> ctypes.CDLL:
                                         c_void_p, c_void_p]
     L.fmsa_gptq_lora_fwd.argtypes = [POINTER(FwdProj), c_int, c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                                      c_int, c_void_p]
+    L.fmsa_gptq_lora_fwd_rope.argtypes = [POINTER(FwdProj), c_int, c_void_p, c_int64, c_int, POINTER(Rope), c_int, c_void_p]
     L.fmsa_gptq_lora_bwd_dx.argtypes = [POINTER(BwdProj), c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p,
                                         c_void_p, c_int64, c_int, c_void_p]
     L.fmsa_swiglu_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
@@ -400,9 +414,11 @@ def lora_grad_batch(jobs):
     return outs
 
 
-def gptq_lora_fwd(x2d, projs: Sequence[dict], mode: int = FWD_LINEAR):
+def gptq_lora_fwd(x2d, projs: Sequence[dict], mode: int = FWD_LINEAR, rope=None):
     """projs: dicts with keys w (GptqWeight), U, B, bias (tensors or None), r, s.
-    Returns the list of outputs Y_p [M, N_p]; in SWIGLU mode returns (e, g, h)."""
+    Returns the list of outputs Y_p [M, N_p]; in SWIGLU mode returns (e, g, h).
+    rope = (cos2d, sin2d, head_dim, proj_mask): LINEAR mode only; the projections whose bit is set in proj_mask
+    leave with the rotary embedding applied (token row m takes row m % cos2d.shape[0] of the tables)."""
     M = x2d.shape[0]
     arr = (FwdProj * len(projs))()
     outs = []
@@ -417,6 +433,17 @@ def gptq_lora_fwd(x2d, projs: Sequence[dict], mode: int = FWD_LINEAR):
     h = None
     if mode == FWD_SWIGLU:
         h = torch.empty_like(outs[0])
+    if rope is not None:
+        cos2d, sin2d, head_dim, proj_mask = rope
+        assert mode == FWD_LINEAR and cos2d.shape == sin2d.shape and cos2d.dtype == sin2d.dtype
+        assert cos2d.stride(1) == 1 and sin2d.stride(1) == 1 and cos2d.stride(0) == sin2d.stride(0) and cos2d.is_cuda
+        if cos2d.dim() != 2 or cos2d.shape[1] < int(head_dim) // 2:
+            raise ValueError("cos / sin must be [positions, >= head_dim / 2]")
+        desc = Rope(_ptr(cos2d), _ptr(sin2d), cos2d.stride(0), cos2d.shape[0], int(head_dim), _DTYPE_ENUM[cos2d.dtype], int(proj_mask))
+        _check("fmsa_gptq_lora_fwd_rope",
+               lib().fmsa_gptq_lora_fwd_rope(arr, len(projs), _ptr(x2d), x2d.stride(0), M, ctypes.byref(desc),
+                                             act_enum(x2d.dtype), _stream(x2d)))
+        return outs
     _check("fmsa_gptq_lora_fwd",
            lib().fmsa_gptq_lora_fwd(arr, len(projs), _ptr(x2d), x2d.stride(0), M, mode, _ptr(h),
                                     0 if h is None else h.stride(0), act_enum(x2d.dtype), _stream(x2d)))

@@ -210,6 +210,28 @@ enum fmsa_fwd_mode { FMSA_FWD_LINEAR = 0, FMSA_FWD_SWIGLU = 1 };
 int fmsa_gptq_lora_fwd(const fmsa_fwd_proj* projs /*host*/, int n_proj, const void* X, int64_t ldx,
                        int M, int mode, void* H, int64_t ldh, int act_dtype, void* stream);
 
+/* The same forward (FMSA_FWD_LINEAR) with the rotary position embedding of the attention block applied in the
+ * epilogue of the projections named by `proj_mask` (bit p = projection p; q and k of LoRA_QKV): replaces the
+ * separate in-place pass of kernels/unsloth/rope_embedding.py:36-65, 68-103 over Q and K,
+ *   (y1, y2) <- (y1 cos - y2 sin, y2 cos + y1 sin)   on the two halves of every head,
+ * applied to the projection output rounded to act_dtype (what that pass reads), fp32 arithmetic, one rounding.
+ * cos / sin: [rows, ld] with head_dim / 2 meaningful values per row (the first half of each row of the
+ * [positions, head_dim] tables transformers passes); token row m takes table row m % rows (rope_embedding.py:60-63
+ * with rows = seq_len; a [batch * seq, .] table is used row by row).  dtype: act_dtype or FMSA_F32.
+ * head_dim % 16 == 0, 256 % head_dim == 0, N_p % head_dim == 0 for the rotated projections; every group_size
+ * % 64 == 0 and K % 64 == 0.  The backward takes dQ, dK through fmsa_rope_embedding(backward = 1) first. */
+typedef struct fmsa_rope {
+  const void* cos;
+  const void* sin;
+  int64_t ld;        /* row stride in elements, >= head_dim / 2; % 8 == 0 (16-bit) or % 4 == 0 (fp32) */
+  int32_t rows;      /* > 0 */
+  int32_t head_dim;
+  int32_t dtype;     /* act_dtype or FMSA_F32 */
+  int32_t proj_mask; /* bit p set: projection p leaves rotated */
+} fmsa_rope;
+int fmsa_gptq_lora_fwd_rope(const fmsa_fwd_proj* projs /*host*/, int n_proj, const void* X, int64_t ldx, int M,
+                            const fmsa_rope* rope /*host*/, int act_dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Fused input-gradient:
  *   dX = sum_p [ dY_p * deq(W_p)^T + mask_p (.) ( T_p * (s_p A_p) ) ],  T_p = dY_p * B_p

@@ -111,6 +111,37 @@ def test_fused_forward_validation():
     assert call(proj(), n=1, mode=1) == -2                # SwiGLU needs exactly gate + up
     assert call(proj(), n=2, mode=1, H=None) == -1
 
+    # the flavour that rotates Q / K in its epilogue: the same checks, plus those of the tables and of the head size
+    fr = lib.fmsa_gptq_lora_fwd_rope
+    assert ctypes.sizeof(fmsa_hip.Rope) == 40
+
+    def rope(**kw):
+        d = dict(cos=0xA000, sin=0xB000, ld=64, rows=8, head_dim=64, dtype=1, mask=1)
+        d.update(kw)
+        return fmsa_hip.Rope(d["cos"], d["sin"], d["ld"], d["rows"], d["head_dim"], d["dtype"], d["mask"])
+
+    def rcall(p, rp, n=1, X=0x7000, ldx=64, M=8, dt=1):
+        arr = (fmsa_hip.FwdProj * 3)(*([p] * 3))
+        return fr(arr, n, X, ldx, M, ctypes.byref(rp) if rp is not None else None, dt, None)
+
+    assert rcall(proj(), None) == -1
+    assert rcall(proj(), rope(cos=None)) == -1
+    assert rcall(proj(), rope(), X=None) == -1
+    assert rcall(proj(), rope(dtype=0)) == -4              # tables in the other 16-bit type than the activations
+    assert rcall(proj(), rope(dtype=7)) == -4
+    assert rcall(proj(), rope(head_dim=0)) == -2
+    assert rcall(proj(), rope(rows=0)) == -2
+    assert rcall(proj(), rope(ld=16)) == -2                # rows shorter than half a head
+    assert rcall(proj(), rope(head_dim=96, ld=96)) == -5   # heads would straddle the 256-column tile
+    assert rcall(proj(), rope(head_dim=24)) == -5
+    assert rcall(proj(), rope(mask=2)) == -2               # names a projection the launch does not have
+    assert rcall(proj(), rope(cos=0xA004)) == -3
+    assert rcall(proj(), rope(ld=36)) == -3
+    assert rcall(proj(), rope(dtype=2, ld=34)) == -3       # fp32 rows must start on 16 bytes too
+    assert rcall(proj(), rope(), ldx=32) == -2             # the plain forward's checks still apply
+    assert rcall(proj(w=_w(N=96), ldy=96), rope()) == -2   # N is not whole heads
+    assert rcall(proj(w=_w(gs=32)), rope()) == -5          # group sizes below the 64-wide K stage
+
 
 def test_bwd_and_skinny_validation():
     lib = fmsa_hip.lib()
