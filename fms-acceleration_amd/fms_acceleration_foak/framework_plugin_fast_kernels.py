@@ -4,7 +4,9 @@ ModelPatcher rules (reference: fms_acceleration_foak/framework_plugin_fast_kerne
 Switches with kernels behind them in this build: `fused_lora` (rule suffixes "qkvo", "mlp"),
 `fast_rms_layernorm` ("rms"), `fast_rope_embeddings` ("rope"), `fast_loss: true` ("cross-ent",
 "custom-loss") and `fast_loss: fused_ce_liger` ("fused-lce": llama, mistral and granite, as in the
-reference).
+reference).  One value beyond the reference's: `fast_rope_embeddings: fused_qkv` registers the same "rope" rule and,
+with `fused_lora` on a quantised base, lets the fused Q / K / V projection of llama, mistral and granite apply the
+rotary embedding in its own launch (the separate pass then finds Q and K marked as done and passes them through).
 """
 from __future__ import annotations
 
@@ -15,19 +17,19 @@ from fms_acceleration import AccelerationPlugin, AccelerationPluginConfigError
 from .utils import filter_mp_rules
 
 
-def register_foak_model_patch_rules(base_type: str, filter_endswith: Set[str] = None, config=None):
+def register_foak_model_patch_rules(base_type: str, filter_endswith: Set[str] = None, config=None, qkv_rope: bool = False):
     from fms_acceleration.model_patcher import ModelPatcher  # pylint: disable=import-outside-toplevel
 
     # pylint: disable=import-outside-toplevel
     from .models import granite, granitemoe, granitemoehybrid, granitemoeshared, llama, mistral, mixtral
 
     rules = [
-        *granite.get_mp_rules(base_type, config),
+        *granite.get_mp_rules(base_type, config, qkv_rope),
         *granitemoe.get_mp_rules(base_type),
         *granitemoeshared.get_mp_rules(base_type),
         *granitemoehybrid.get_mp_rules(base_type),
-        *llama.get_mp_rules(base_type, config),
-        *mistral.get_mp_rules(base_type, config),
+        *llama.get_mp_rules(base_type, config, qkv_rope),
+        *mistral.get_mp_rules(base_type, config, qkv_rope),
         *mixtral.get_mp_rules(base_type),
     ]
     if filter_endswith:
@@ -40,7 +42,7 @@ FILTER_MAP = {
     "fused_lora": {"qkvo", "mlp"},
     "fast_loss": {True: {"cross-ent", "custom-loss"}, "fused_ce_liger": "fused-lce"},
     "fast_rms_layernorm": "rms",
-    "fast_rope_embeddings": "rope",
+    "fast_rope_embeddings": {True: "rope", "fused_qkv": "rope"},
 }
 
 
@@ -69,7 +71,7 @@ class FastKernelsAccelerationPlugin(AccelerationPlugin):
             ("fused_lora", [False, True]),
             ("fast_loss", [False, True, "fused_ce_liger"]),
             ("fast_rms_layernorm", [False, True]),
-            ("fast_rope_embeddings", [False, True]),
+            ("fast_rope_embeddings", [False, True, "fused_qkv"]),
         ):
             default = "auto_gptq" if key == "base_layer" else False
             self.configurations[key] = self._check_config_and_maybe_check_values(key=key, values=values, default=default)
@@ -96,7 +98,9 @@ class FastKernelsAccelerationPlugin(AccelerationPlugin):
                 selected = selected[value]
             terms.update({selected} if isinstance(selected, str) else selected)
         register_foak_model_patch_rules(
-            base_type=self.configurations["base_layer"], filter_endswith=terms, config=model.config
+            base_type=self.configurations["base_layer"], filter_endswith=terms, config=model.config,
+            qkv_rope=self.configurations["fast_rope_embeddings"] == "fused_qkv" and "fused_lora" not in omitted
+            and bool(self.configurations["fused_lora"]),
         )
         return model, modifiable_args
 

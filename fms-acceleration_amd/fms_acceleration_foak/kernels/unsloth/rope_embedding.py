@@ -48,7 +48,23 @@ class Fast_RoPE_Embedding(torch.autograd.Function):
         return dY2.view(batch, seq_len, n_heads, head_dim), None, None
 
 
+# Q / K that left a fused projection already rotated (apply_lora_qkv_rope behind the `<arch>-qkvo` rule): keyed by the
+# address of Q's storage, holding both tensors so that the address cannot be reused while the entry waits for the
+# attention's apply_rotary_pos_emb call, which consumes it.
+_ROTATED = {}
+
+
+def mark_rotated(Q, K):
+    _ROTATED[Q.untyped_storage().data_ptr()] = (Q, K)
+
+
 def fast_rope_embedding(Q, K, cos, sin, position_ids=None, unsqueeze_dim=1):
+    if _ROTATED:
+        done = _ROTATED.pop(Q.untyped_storage().data_ptr(), None)
+        if done is not None:
+            if done[1].untyped_storage().data_ptr() != K.untyped_storage().data_ptr():
+                raise RuntimeError("fast_rope_embedding: Q comes rotated from the fused projection, K does not")
+            return Q, K
     Q = Fast_RoPE_Embedding.apply(Q.transpose(1, 2), cos, sin).transpose(1, 2)
     K = Fast_RoPE_Embedding.apply(K.transpose(1, 2), cos, sin).transpose(1, 2)
     return Q, K

@@ -22,7 +22,9 @@ QKV_NAMES = ["q_proj", "k_proj", "v_proj"]
 MLP_NAMES = ["up_proj", "down_proj", "gate_proj"]
 
 
-def fused_lora_rules(arch: str, attn_cls, mlp_cls, base_type: str, config=None, label: str = None):
+def fused_lora_rules(arch: str, attn_cls, mlp_cls, base_type: str, config=None, label: str = None, qkv_rope: bool = False):
+    """qkv_rope: the fused Q / K / V call also applies the rotary embedding (needs the `<arch>-rope` rule, whose
+    fast_rope_embedding passes the marked Q / K through)."""
     rules = [
         ModelPatcherRule(
             rule_id=f"{arch}-qkvo",
@@ -32,7 +34,8 @@ def fused_lora_rules(arch: str, attn_cls, mlp_cls, base_type: str, config=None, 
                 logic="OR",
             ),
             forward_builder=combine_functions(
-                partial(build_lora_fused_ops, submodule_names=QKV_NAMES, fused_op=KEY_QKV, base_type=base_type),
+                partial(build_lora_fused_ops, submodule_names=QKV_NAMES, fused_op=KEY_QKV, base_type=base_type,
+                        qkv_rope=qkv_rope),
                 partial(build_lora_fused_ops, submodule_names=["o_proj"], fused_op=KEY_O, base_type=base_type),
                 logic="APPEND",
             ),

@@ -6,9 +6,9 @@ from transformers.models.mistral.modeling_mistral import MistralAttention, Mistr
 from ._rules import fused_lce_rules, fused_lora_rules, loss_rules, norm_rope_rules
 
 
-def get_mp_rules(base_type: str, config=None):
+def get_mp_rules(base_type: str, config=None, qkv_rope: bool = False):
     return [
-        *fused_lora_rules("mistral", MistralAttention, MistralMLP, base_type, config, label="Mistral"),
+        *fused_lora_rules("mistral", MistralAttention, MistralMLP, base_type, config, label="Mistral", qkv_rope=qkv_rope),
         *fused_lce_rules("mistral", MistralForCausalLM),
         *loss_rules("mistral", MistralForCausalLM, "transformers.models.mistral.modeling_mistral"),
         *norm_rope_rules("mistral", MistralRMSNorm, "transformers.models.mistral.modeling_mistral"),

@@ -20,6 +20,9 @@ from ..fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_mlp as fused_op_m
 from ..fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_o_v2 as fused_op_o_gptq
 from ..fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_qkv as fused_op_qkv_gptq
 
+from ..fused_ops.unsloth_lora.bnb.fast_lora import apply_lora_qkv_rope as fused_op_qkv_rope_bnb
+from ..fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_qkv_rope as fused_op_qkv_rope_gptq
+
 KEY_QKV = "qkv"
 KEY_O = "o"
 KEY_MLP = "mlp"
@@ -32,6 +35,11 @@ FUSED_OPS = {
 }
 
 
+# Q / K / V with the rotary embedding of Q and K applied inside the projection launch (no counterpart in the reference,
+# whose fused projections are followed by the separate fast_rope_embedding pass); chosen by `qkv_rope` below
+FUSED_QKV_ROPE_OPS = {"auto_gptq": fused_op_qkv_rope_gptq, "bitsandbytes": fused_op_qkv_rope_bnb}
+
+
 def register_fused_ops(base_type: str, qkv: Callable, o: Callable, mlp: Callable):
     FUSED_OPS[base_type] = {KEY_QKV: qkv, KEY_O: o, KEY_MLP: mlp}
 
@@ -42,14 +50,34 @@ def _is_loralayer(module: torch.nn.Module, names: List[str] = None):
     return all(hasattr(module, n) for n in names)
 
 
-def _build_fused_forwards(attn: torch.nn.Module, fused_operation: Callable, submodule_names: List[str]):
+def _build_fused_forwards(attn: torch.nn.Module, fused_operation: Callable, submodule_names: List[str],
+                          rope_operation: Callable = None):
     """One closure per sub-module name.  Protocol: each of the named projections is called exactly
-    once per attention forward; the first call computes all outputs.  Not thread-safe."""
+    once per attention forward; the first call computes all outputs.  Not thread-safe.
+
+    rope_operation (apply_lora_qkv_rope): a forward pre-hook of the attention keeps the `position_embeddings` it is
+    called with; the fused call then returns Q and K already rotated and marks them, so that the attention's
+    apply_rotary_pos_emb (fast_rope_embedding of the `<arch>-rope` rule) passes them through.  Without tables
+    (an attention called without `position_embeddings`) the plain fused operation runs."""
     pending = {}
+    tables = {}
+
+    if rope_operation is not None:
+        from ..kernels.unsloth.rope_embedding import mark_rotated  # pylint: disable=import-outside-toplevel
+
+        def _keep_tables(module, args, kwargs):
+            tables["pe"] = kwargs.get("position_embeddings", args[1] if len(args) > 1 else None)
+
+        attn.register_forward_pre_hook(_keep_tables, with_kwargs=True)
 
     def _forward(self, X, name: str):
         if not any(n in pending for n in submodule_names):
-            outs = fused_operation(attn, X)
+            pe = tables.pop("pe", None)
+            if rope_operation is not None and pe is not None and X.dim() == 3:
+                outs = rope_operation(attn, X, pe[0], pe[1])
+                mark_rotated(outs[0], outs[1])
+            else:
+                outs = fused_operation(attn, X)
             outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
             pending.update(zip(submodule_names, outs))
         assert name in pending, "Fused_op needs to be first reset with sequential calls to each of them"
@@ -59,7 +87,7 @@ def _build_fused_forwards(attn: torch.nn.Module, fused_operation: Callable, subm
 
 
 def build_lora_fused_ops(attn: torch.nn.Module, base_type: str = "auto_gptq", submodule_names: List[str] = None,
-                         fused_op: str = KEY_QKV):
+                         fused_op: str = KEY_QKV, qkv_rope: bool = False):
     assert submodule_names is None or len(submodule_names) > 0, \
         "When building lora fused ops requires more than one submodule."
     if submodule_names is None:
@@ -68,7 +96,8 @@ def build_lora_fused_ops(attn: torch.nn.Module, base_type: str = "auto_gptq", su
     if fused_op == KEY_QKV:
         return [
             (ModelPatcherTrigger(check=_is_loralayer, module_name=name), forward)
-            for name, forward in _build_fused_forwards(attn, fused_operation, submodule_names)
+            for name, forward in _build_fused_forwards(attn, fused_operation, submodule_names,
+                                                       FUSED_QKV_ROPE_OPS.get(base_type) if qkv_rope else None)
         ]
     if fused_op == KEY_O:
         return [(ModelPatcherTrigger(check=_is_loralayer, module_name=submodule_names[0]), fused_operation)]

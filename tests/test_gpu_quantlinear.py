@@ -37,7 +37,11 @@ def test_quantlinear_forward_backward(K, N, gs, act_order, dtype):
     assert olora.max_rel_err(xg.grad.reshape(-1, K), dx_ref.reshape(-1, K)) < TOL
 
 
-def test_checkpoint_to_patched_training_step(tmp_path):
+# rope: True = the reference's separate fast_rope_embedding pass after the fused projections; "fused_qkv" = Q and K
+# rotated inside the fused projection launch
+@pytest.mark.parametrize("rope", [True, "fused_qkv"])
+def test_checkpoint_to_patched_training_step(tmp_path, rope, monkeypatch):
+    import fmsa_hip
     from transformers import LlamaConfig, LlamaForCausalLM
 
     from fms_acceleration.model_patcher import ModelPatcher, patch_model
@@ -83,7 +87,20 @@ def test_checkpoint_to_patched_training_step(tmp_path):
 
     loss_ref, grads_ref = step(plain)
     plugin = FastKernelsAccelerationPlugin({"training": {"fused_ops_and_kernels": {
-        "fused_lora": True, "fast_loss": True, "fast_rms_layernorm": True, "fast_rope_embeddings": True}}})
+        "fused_lora": True, "fast_loss": True, "fast_rms_layernorm": True, "fast_rope_embeddings": rope}}})
+    seen = {"fwd_with_rope": 0, "rope_fwd_pass": 0, "rope_bwd_pass": 0}
+    real_fwd, real_rope = fmsa_hip.gptq_lora_fwd, fmsa_hip.rope_embedding_
+
+    def count_fwd(*a, **k):
+        seen["fwd_with_rope"] += k.get("rope") is not None
+        return real_fwd(*a, **k)
+
+    def count_rope(*a, backward=False, **k):
+        seen["rope_bwd_pass" if backward else "rope_fwd_pass"] += 1
+        return real_rope(*a, backward=backward, **k)
+
+    monkeypatch.setattr(fmsa_hip, "gptq_lora_fwd", count_fwd)
+    monkeypatch.setattr(fmsa_hip, "rope_embedding_", count_rope)
     original = ml.apply_rotary_pos_emb
     try:
         with instantiate_model_patcher():
@@ -95,6 +112,9 @@ def test_checkpoint_to_patched_training_step(tmp_path):
             loss, grads = step(model)
     finally:
         ml.apply_rotary_pos_emb = original
+    # per layer: one forward launch that rotates Q and K and no separate forward pass, or two separate passes
+    assert seen == ({"fwd_with_rope": 2, "rope_fwd_pass": 0, "rope_bwd_pass": 4} if rope == "fused_qkv"
+                    else {"fwd_with_rope": 0, "rope_fwd_pass": 4, "rope_bwd_pass": 4})
     assert abs(loss - loss_ref) < 2e-2 * max(1.0, abs(loss_ref))
     assert set(grads) == set(grads_ref) and len(grads) == 2 * 7 * 2  # lora_A and lora_B of 7 projections x 2 layers
     worst = max(olora.max_rel_err(grads[n], grads_ref[n]) for n in grads)

@@ -224,6 +224,58 @@ def test_qkv_wrapper_protocol():
     assert fwd["v_proj"](None, x).item() == 3 and len(calls) == 2  # a new round starts with whoever comes first
 
 
+def test_qkv_wrapper_with_rope_tables():
+    """With a rope operation the wrapper keeps the position_embeddings the attention is called with, hands them to the
+    fused call, and marks Q / K so that fast_rope_embedding passes exactly those tensors through, once."""
+    from fms_acceleration_foak.kernels.unsloth import rope_embedding as re_mod
+    from fms_acceleration_foak.models.utils import _build_fused_forwards
+
+    names = ["q_proj", "k_proj", "v_proj"]
+
+    class Attn(torch.nn.Module):
+        def forward(self, hidden_states, position_embeddings=None):
+            q, k, v = (fwd[n](None, hidden_states) for n in names)
+            q, k = q.view(1, 2, 1, 4).transpose(1, 2), k.view(1, 2, 1, 4).transpose(1, 2)
+            cos, sin = position_embeddings if position_embeddings is not None else (None, None)
+            return re_mod.fast_rope_embedding(q, k, cos, sin), v
+
+    seen = []
+    plain = lambda attn, X: (X + 1, X + 2, X + 3)  # noqa: E731
+
+    def with_rope(attn, X, cos, sin):
+        seen.append((cos, sin))
+        return X + 10, X + 20, X + 30
+
+    attn = Attn()
+    fwd = dict(_build_fused_forwards(attn, plain, names, with_rope))
+    x = torch.zeros(1, 2, 4)
+    (q, k), v = attn(x, position_embeddings=("c", "s"))
+    assert seen == [("c", "s")] and q.flatten()[0] == 10 and k.flatten()[0] == 20 and v.flatten()[0] == 30
+    assert not re_mod._ROTATED  # consumed by the pass-through
+    # a Q the fused call did not produce is not passed through (the kernel is asked for, which a CPU tensor cannot do)
+    with pytest.raises(Exception):
+        re_mod.fast_rope_embedding(q.clone(), k.clone(), torch.ones(2, 4), torch.zeros(2, 4))
+    # Q marked, K from elsewhere: refuses instead of rotating one of them twice
+    re_mod.mark_rotated(q, k)
+    with pytest.raises(RuntimeError, match="K does not"):
+        re_mod.fast_rope_embedding(q, k.clone(), None, None)
+    assert not re_mod._ROTATED
+    # without tables the plain fused operation runs and nothing is marked
+    for n in names:
+        out = fwd[n](None, x)
+    assert out.flatten()[0] == 3 and not re_mod._ROTATED and len(seen) == 1
+
+
+def test_fast_rope_embeddings_fused_qkv_is_accepted():
+    from fms_acceleration_foak import FastKernelsAccelerationPlugin
+
+    plugin = FastKernelsAccelerationPlugin({"training": {"fused_ops_and_kernels": {
+        "fused_lora": True, "fast_rope_embeddings": "fused_qkv"}}})
+    assert plugin.configurations["fast_rope_embeddings"] == "fused_qkv"
+    with pytest.raises(Exception):
+        FastKernelsAccelerationPlugin({"training": {"fused_ops_and_kernels": {"fast_rope_embeddings": "other"}}})
+
+
 def test_filter_mp_rules():
     from fms_acceleration_foak.utils import filter_mp_rules
 
