@@ -12,6 +12,9 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
                      hipStream_t st);
 int lora_grad_splits(int M, int C);
 size_t lora_grad_batch_workspace(const fmsa_lora_grad_job* jobs, int n_jobs, int M);
+size_t lora_down_workspace(int M, int C, int r);
+int launch_lora_down_ws(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out, int64_t ldo,
+                        void* workspace, size_t workspace_bytes, hipStream_t st);
 int launch_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int act_dtype, void* workspace, hipStream_t st);
 int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, void* H,
                          int64_t ldh, const fmsa_rope* rope, int act_dtype, hipStream_t st);
@@ -115,7 +118,7 @@ const char* fmsa_strerror(int code) {
   }
 }
 
-int fmsa_abi_version(void) { return 6; }
+int fmsa_abi_version(void) { return 7; }
 
 int fmsa_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, void* stream) {
   if (!w || !out) return FMSA_ERR_NULL;
@@ -151,6 +154,23 @@ int fmsa_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int
   if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
   if (!aligned16(X) || !aligned16(Wd) || ldx % 8 != 0) return FMSA_ERR_ALIGN;
   return launch_lora_down(X, ldx, Wd, M, C, r, act_dtype, out, ldout, (hipStream_t)stream);
+}
+
+size_t fmsa_lora_down_workspace(int M, int C, int r) {
+  if (M <= 0 || C <= 0 || r <= 0 || r > 128 || r % 8 != 0 || C % 8 != 0) return 0;
+  return lora_down_workspace(M, C, r);
+}
+
+int fmsa_lora_down_ws(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out,
+                      int64_t ldout, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!X || !Wd || !out) return FMSA_ERR_NULL;
+  if (M <= 0 || C <= 0 || r <= 0 || ldx < C || ldout < r) return FMSA_ERR_SHAPE;
+  if (int rc = check_rank(r)) return rc;
+  if (C % 8 != 0) return FMSA_ERR_SHAPE;
+  if (!is_act(act_dtype)) return FMSA_ERR_DTYPE;
+  if (!aligned16(X) || !aligned16(Wd) || ldx % 8 != 0) return FMSA_ERR_ALIGN;
+  if (workspace && !aligned16(workspace)) return FMSA_ERR_ALIGN;
+  return launch_lora_down_ws(X, ldx, Wd, M, C, r, act_dtype, out, ldout, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 size_t fmsa_lora_grad_workspace(int M, int C, int r) {

@@ -4,6 +4,8 @@
 //   lora_grad  out[r, C]  = scale * L[M, r]^T * R[M, C]    (dA, dB: a reduction over tokens)
 #include "common.h"
 
+#include <algorithm>
+
 namespace {
 
 // The big operand is read exactly once: its loads carry the non-temporal hint (`nt`: direct-to-LDS loads through the
@@ -249,6 +251,208 @@ __global__ __launch_bounds__(512) void lora_down_staged_kernel(const uint16_t* _
     }
     if constexpr (t0 + RC < RT) __syncthreads();  // the next four rank tiles reuse the buffer
   });
+}
+
+// ---- lora_down, staged, many tokens per workgroup, columns split over workgroups ----------------------
+// Every workgroup of the kernels above reads all of Wd, which at 16-32 tokens per workgroup is r / 16 .. r / 32 times
+// the bytes of X it consumes: from rank 32 on the L2 traffic of Wd, not HBM, sets the pace.  Here a workgroup owns
+// 32 * G tokens and one of `n_split` contiguous column ranges: the stages of a 512-column chunk are its G row groups one
+// after the other, multiplied by the same Wd fragments (loaded once per chunk), so Wd is read once per 32 * G tokens;
+// the column split gives the chip its workgroups back when M / (32 * G) falls short of the CUs.  With n_split > 1 the
+// fp32 sums of the ranges go to partial[split][M][r] and lora_down_reduce_kernel adds them in index order (same result
+// whatever the scheduling) and rounds once.  Stage buffers, swizzle and the waits are those of the kernel above.
+template <typename T, int RT, int G>
+__global__ __launch_bounds__(512) void lora_down_split_kernel(const uint16_t* __restrict__ X, int64_t ldx,
+                                                              const uint16_t* __restrict__ Wd, int M, int C, int r,
+                                                              uint16_t* __restrict__ out, int64_t ldo,
+                                                              float* __restrict__ partial, int n_tb, int n_split) {
+  constexpr int NW = 8, NH = 4, MTL = 2, ROWS = 32, SC = 512;
+  static_assert(G == 2 || G == 4, "a chunk's row groups fill the four stage buffers a whole number of times");
+  static_assert(G * MTL * RT <= 32, "accumulator registers");
+  __shared__ __attribute__((aligned(1024))) uint16_t s0[ROWS * SC];
+  __shared__ __attribute__((aligned(1024))) uint16_t s1[ROWS * SC];
+  __shared__ __attribute__((aligned(1024))) uint16_t s2[ROWS * SC];
+  __shared__ __attribute__((aligned(1024))) uint16_t s3[ROWS * SC];
+  auto buf = [&](auto b_c) -> char* {
+    constexpr int b = decltype(b_c)::value;
+    return reinterpret_cast<char*>(b == 0 ? s0 : (b == 1 ? s1 : (b == 2 ? s2 : s3)));
+  };
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int uwave = __builtin_amdgcn_readfirstlane(wave);
+  const int l16 = lane & 15, q = lane >> 4;
+  const int tb = blockIdx.x % n_tb, sp = blockIdx.x / n_tb;
+  const int m_base = tb * (ROWS * G);
+  const int rows_valid = min(ROWS * G, M - m_base);
+  // this workgroup's chunks [ch_lo, ch_hi) of 512 columns
+  const int n_chunks = (C + SC - 1) / SC;
+  const int per = (n_chunks + n_split - 1) / n_split;
+  const int ch_lo = min(n_chunks, sp * per), ch_hi = min(n_chunks, ch_lo + per);
+  const int n_stages = (ch_hi - ch_lo) * G;
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(X + (size_t)m_base * ldx, (size_t)rows_valid * ldx * 2);
+  const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(Wd, (size_t)r * C * 2);
+
+  // direct loads: wave w moves rows 4 w .. 4 w + 3 of a stage (row group g of the workgroup's tokens)
+  uint32_t d_off[4], d_col[4];
+#pragma unroll
+  for (int i = 0; i < 2 * MTL; ++i) {
+    const int row = 2 * MTL * wave + i;
+    d_col[i] = 8 * (lane ^ (row & 15));
+    d_off[i] = (uint32_t)((row * ldx + d_col[i]) * 2);
+  }
+  const uint32_t group_bytes = (uint32_t)(ROWS * ldx * 2);
+  // stage st = chunk ch_lo + st / G, row group st % G; stages past the last one load nothing (every lane out of range)
+  auto dma = [&](int st, auto b_c) {
+    const int ch = ch_lo + st / G, g = st % G;
+#pragma unroll
+    for (int i = 0; i < 2 * MTL; ++i) {
+      const uint32_t dead = (ch < ch_hi && (ch * SC + (int)d_col[i]) < C) ? 0u : 0x80000000u;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (__attribute__((address_space(3))) void*)(buf(b_c) + (2 * MTL * uwave + i) * (SC * 2)),
+                                               16, (d_off[i] + (uint32_t)g * group_bytes) | dead, (uint32_t)ch * (SC * 2), 0, 2);
+    }
+  };
+  uint32_t w_off[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) w_off[t] = (uint32_t)(((16 * t + l16) * (int64_t)C + 8 * q) * 2);
+  auto wld = [&](int ch, u32x4(&wf)[2][RT]) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const int c0 = ch * SC + 32 * (2 * wave + kk);
+      const uint32_t dead = (ch < ch_hi && (c0 + 8 * q) < C) ? 0u : 0x80000000u;
+#pragma unroll
+      for (int t = 0; t < RT; ++t) wf[kk][t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (w_off[t] + 2 * c0) | dead, 0, 0);
+    }
+  };
+  f32x4 acc[G][MTL][RT];
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int u = 0; u < MTL; ++u)
+#pragma unroll
+      for (int t = 0; t < RT; ++t) acc[g][u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto mul = [&](auto b_c, auto g_c, const u32x4(&wf)[2][RT]) {
+    constexpr int g = decltype(g_c)::value;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const int chunk = 4 * (2 * wave + kk) + q;
+#pragma unroll
+      for (int u = 0; u < MTL; ++u) {
+        const u32x4 xf = *reinterpret_cast<const u32x4*>(buf(b_c) + (16 * u + l16) * (SC * 2) + ((chunk ^ l16) * 16));
+#pragma unroll
+        for (int t = 0; t < RT; ++t) acc[g][u][t] = mfma16<T>(xf, wf[kk][t], acc[g][u][t]);
+      }
+    }
+  };
+  // Loads a wave issues after the direct loads of stage st and before that stage's turn: the direct loads of the two
+  // stages after it (2 x 4), and one batch of Wd fragments when turn st - 1 or st - 2 closed a chunk (g = 0 or 1).
+  // A smaller count than the true one only waits longer, so the first turns use the same figures.
+  auto wait_for = [&](auto g_c) {
+    constexpr int g = decltype(g_c)::value;
+    constexpr int YOUNGER = 4 * MTL + ((g == 0 || g == 1) ? 2 * RT : 0);
+    __builtin_amdgcn_s_waitcnt((YOUNGER & 0xF) | ((YOUNGER >> 4) << 14) | 0x0F70);
+  };
+  u32x4 wa[2][RT], wb[2][RT];
+  // turn st: its direct loads have landed -> barrier -> (last row group of a chunk: the next chunk's Wd fragments) ->
+  // the direct loads three stages ahead -> multiply
+  auto turn = [&](int st, auto cur_c, auto refill_c, auto g_c, const u32x4(&wcur)[2][RT], u32x4(&wnext)[2][RT]) {
+    constexpr int g = decltype(g_c)::value;
+    wait_for(g_c);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (g == G - 1) wld(ch_lo + st / G + 1, wnext);
+    dma(st + 3, refill_c);
+    mul(cur_c, g_c, wcur);
+  };
+  using B0 = std::integral_constant<int, 0>;
+  using B1 = std::integral_constant<int, 1>;
+  using B2 = std::integral_constant<int, 2>;
+  using B3 = std::integral_constant<int, 3>;
+  dma(0, B0{});
+  dma(1, B1{});
+  dma(2, B2{});
+  wld(ch_lo, wa);
+  if constexpr (G == 2) {
+    for (int st = 0; st < n_stages; st += 4) {  // two chunks per round
+      turn(st, B0{}, B3{}, B0{}, wa, wb);
+      turn(st + 1, B1{}, B0{}, B1{}, wa, wb);
+      turn(st + 2, B2{}, B1{}, B0{}, wb, wa);
+      turn(st + 3, B3{}, B2{}, B1{}, wb, wa);
+    }
+  } else {
+    for (int st = 0; st < n_stages; st += 8) {
+      turn(st, B0{}, B3{}, B0{}, wa, wb);
+      turn(st + 1, B1{}, B0{}, B1{}, wa, wb);
+      turn(st + 2, B2{}, B1{}, B2{}, wa, wb);
+      turn(st + 3, B3{}, B2{}, B3{}, wa, wb);
+      turn(st + 4, B0{}, B3{}, B0{}, wb, wa);
+      turn(st + 5, B1{}, B0{}, B1{}, wb, wa);
+      turn(st + 6, B2{}, B1{}, B2{}, wb, wa);
+      turn(st + 7, B3{}, B2{}, B3{}, wb, wa);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the surplus direct loads (all lanes out of range) have landed too
+  __syncthreads();
+
+  // the waves' partial tiles are added through stage buffer 0, one row group and RC rank tiles at a time
+  constexpr int RC = RT < 4 ? RT : 4;
+  float(*red)[MTL][RC][64][4] = reinterpret_cast<float(*)[MTL][RC][64][4]>(s0);
+  float* const pdst = partial + (size_t)sp * M * r;
+  static_for<0, G>([&](auto g_c) {
+    constexpr int g = decltype(g_c)::value;
+    static_for<0, RT / RC>([&](auto c_c) {
+      constexpr int t0 = decltype(c_c)::value * RC;
+      if (wave >= NH) {
+#pragma unroll
+        for (int u = 0; u < MTL; ++u)
+#pragma unroll
+          for (int t = 0; t < RC; ++t) *reinterpret_cast<f32x4*>(red[wave - NH][u][t][lane]) = acc[g][u][t0 + t];
+      }
+      __syncthreads();
+      if (wave < NH) {
+#pragma unroll
+        for (int u = 0; u < MTL; ++u)
+#pragma unroll
+          for (int t = 0; t < RC; ++t) {
+            const f32x4 o = *reinterpret_cast<const f32x4*>(red[wave][u][t][lane]);
+            *reinterpret_cast<f32x4*>(red[wave][u][t][lane]) = acc[g][u][t0 + t] + o;
+          }
+      }
+      __syncthreads();
+      for (int o = tid; o < MTL * RC * 256; o += 64 * NW) {
+        const int u = o / (RC * 256), t = (o >> 8) % RC, ln = (o >> 2) & 63, i = o & 3;
+        float v = red[0][u][t][ln][i];
+#pragma unroll
+        for (int w = 1; w < NH; ++w) v += red[w][u][t][ln][i];
+        const int row = m_base + ROWS * g + 16 * u + 4 * (ln >> 4) + i;
+        const int j = 16 * (t0 + t) + (ln & 15);
+        if (row < M && j < r) {
+          if (n_split == 1)
+            out[(size_t)row * ldo + j] = pack1<T>(v);
+          else
+            pdst[(size_t)row * r + j] = v;
+        }
+      }
+      __syncthreads();  // the next tiles reuse the buffer
+    });
+  });
+}
+
+// out[m, j] = round(sum over splits, in index order, of partial[split][m][j]); r % 8 == 0: four ranks per thread
+template <typename T>
+__global__ __launch_bounds__(256) void lora_down_reduce_kernel(const float* __restrict__ partial, int n_split, int M, int r,
+                                                               uint16_t* __restrict__ out, int64_t ldo) {
+  const int64_t q4 = (int64_t)blockIdx.x * 256 + threadIdx.x;  // quad of ranks
+  const int per_row = r / 4;
+  if (q4 >= (int64_t)M * per_row) return;
+  const int m = (int)(q4 / per_row), j = 4 * (int)(q4 % per_row);
+  const size_t plane = (size_t)M * r;
+  f32x4 v = *reinterpret_cast<const f32x4*>(partial + (size_t)m * r + j);
+  for (int s = 1; s < n_split; ++s) v += *reinterpret_cast<const f32x4*>(partial + s * plane + (size_t)m * r + j);
+  u32x2 o;
+  o[0] = pack2<T>(v[0], v[1]);
+  o[1] = pack2<T>(v[2], v[3]);
+  *reinterpret_cast<u32x2*>(out + (size_t)m * ldo + j) = o;
 }
 
 // ---- lora_grad ----------------------------------------------------------------------------------
@@ -611,6 +815,79 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
 #undef DISPATCH
 #undef LAUNCH
   FMSA_CHECK_LAUNCH();
+  return FMSA_OK;
+}
+
+namespace {
+// Shape of the split launch: row groups per workgroup, column ranges, or g = 0 when the kernels without workspace do as
+// well (rank 16 and below: Wd is a quarter of the X bytes a 32-token workgroup reads) or the matrix is too small.
+struct DownSplit {
+  int g, n_tb, n_split;
+};
+DownSplit lora_down_split_shape(int M, int C, int r) {
+  const int rt = (std::min(r, 64) + 15) / 16;  // ranks above 64 go out 64 at a time (accumulator registers)
+  if (rt < 2 || M < 2048 || C < 2048) return {0, 0, 0};
+  const int g = rt <= 2 ? 2 : 4;  // rank 32: 64 tokens per workgroup; 48 / 64: 128
+  const int n_tb = (M + 32 * g - 1) / (32 * g);
+  const int n_chunks = (C + 511) / 512;
+  int n_split = (256 + n_tb - 1) / n_tb;                 // a workgroup per CU at least
+  n_split = std::max(1, std::min(n_split, n_chunks / 2));  // two chunks per range at least
+  return {g, n_tb, n_split};
+}
+}  // namespace
+
+size_t lora_down_workspace(int M, int C, int r) {
+  const DownSplit d = lora_down_split_shape(M, C, r);
+  return d.g && d.n_split > 1 ? (size_t)d.n_split * (size_t)M * (size_t)std::min(r, 64) * sizeof(float) : 0;
+}
+
+// The split kernel where it pays and the caller brought the partial-sum buffer (or none is needed); launch_lora_down otherwise.
+int launch_lora_down_ws(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype, void* out,
+                        int64_t ldo, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  const DownSplit d = lora_down_split_shape(M, C, r);
+  const size_t need = lora_down_workspace(M, C, r);
+  const bool out_ok = ((uintptr_t)out % 8 == 0) && ldo % 4 == 0;  // the reduce pass stores four ranks at a time
+  if (!d.g || (need && (!workspace || workspace_bytes < need || !out_ok)))
+    return launch_lora_down(X, ldx, Wd, M, C, r, act_dtype, out, ldo, st);
+  if (r > 64) {
+    // 64 ranks per pass over X (launches on one stream run in order, so the passes share the workspace); cheaper than one
+    // pass whose accumulators and double-buffered Wd fragments do not fit the registers
+    for (int r0 = 0; r0 < r; r0 += 64) {
+      const int rc = launch_lora_down_ws(X, ldx, (const uint16_t*)Wd + (size_t)r0 * C, M, C, std::min(64, r - r0), act_dtype,
+                                         (uint16_t*)out + r0, ldo, workspace, workspace_bytes, st);
+      if (rc != FMSA_OK) return rc;
+    }
+    return FMSA_OK;
+  }
+  const int rt = (r + 15) / 16;
+  dim3 grid(d.n_tb * d.n_split), block(512);
+#define SPLIT_LAUNCH(TT, RT, G)                                                                                                  \
+  hipLaunchKernelGGL((lora_down_split_kernel<TT, RT, G>), grid, block, 0, st, (const uint16_t*)X, ldx, (const uint16_t*)Wd, M, \
+                     C, r, (uint16_t*)out, ldo, (float*)workspace, d.n_tb, d.n_split)
+#define SPLIT_DISPATCH(TT)                            \
+  switch (rt) {                                       \
+    case 2: SPLIT_LAUNCH(TT, 2, 2); break;            \
+    default: SPLIT_LAUNCH(TT, 4, 4); break;           \
+  }
+  if (act_dtype == FMSA_BF16) {
+    SPLIT_DISPATCH(bf16_t)
+  } else {
+    SPLIT_DISPATCH(f16_t)
+  }
+#undef SPLIT_DISPATCH
+#undef SPLIT_LAUNCH
+  FMSA_CHECK_LAUNCH();
+  if (d.n_split > 1) {
+    const int64_t quads = (int64_t)M * (r / 4);
+    dim3 rgrid((unsigned)((quads + 255) / 256));
+    if (act_dtype == FMSA_BF16)
+      hipLaunchKernelGGL((lora_down_reduce_kernel<bf16_t>), rgrid, dim3(256), 0, st, (const float*)workspace, d.n_split, M, r,
+                         (uint16_t*)out, ldo);
+    else
+      hipLaunchKernelGGL((lora_down_reduce_kernel<f16_t>), rgrid, dim3(256), 0, st, (const float*)workspace, d.n_split, M, r,
+                         (uint16_t*)out, ldo);
+    FMSA_CHECK_LAUNCH();
+  }
   return FMSA_OK;
 }
 

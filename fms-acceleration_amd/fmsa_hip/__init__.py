@@ -29,6 +29,8 @@ EXPORTED_SYMBOLS = (
     "fmsa_gptq_permute_rows",
     "fmsa_permute_cols",
     "fmsa_lora_down",
+    "fmsa_lora_down_workspace",
+    "fmsa_lora_down_ws",
     "fmsa_lora_grad_workspace",
     "fmsa_lora_grad",
     "fmsa_lora_grad_batch_workspace",
@@ -190,6 +192,10 @@ def lib() -> ctypes.CDLL:
     L.fmsa_gptq_permute_rows.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]
     L.fmsa_permute_cols.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int64, c_void_p]
     L.fmsa_lora_down.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int64, c_void_p]
+    L.fmsa_lora_down_workspace.restype = c_size_t
+    L.fmsa_lora_down_workspace.argtypes = [c_int, c_int, c_int]
+    L.fmsa_lora_down_ws.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_size_t,
+                                    c_void_p]
     L.fmsa_lora_grad_workspace.restype = c_size_t
     L.fmsa_lora_grad_workspace.argtypes = [c_int, c_int, c_int]
     L.fmsa_lora_grad.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
@@ -328,8 +334,10 @@ def lora_down(x2d, wd, out=None):
     if out is None:
         out = torch.empty((M, r), dtype=x2d.dtype, device=x2d.device)
     assert out.shape == (M, r) and out.stride(1) == 1 and out.dtype == x2d.dtype
-    _check("fmsa_lora_down", lib().fmsa_lora_down(_ptr(x2d), x2d.stride(0), _ptr(wd), M, C, r, act_enum(x2d.dtype), _ptr(out),
-                                                  out.stride(0), _stream(out)))
+    nbytes = lib().fmsa_lora_down_workspace(M, C, r)
+    ws = _workspace(nbytes, x2d.device) if nbytes else None
+    _check("fmsa_lora_down_ws", lib().fmsa_lora_down_ws(_ptr(x2d), x2d.stride(0), _ptr(wd), M, C, r, act_enum(x2d.dtype), _ptr(out),
+                                                        out.stride(0), _ptr(ws), 0 if ws is None else ws.numel(), _stream(out)))
     return out
 
 

@@ -157,6 +157,19 @@ def test_bwd_and_skinny_validation():
     m2 = fmsa_hip.BwdProj(_w(), 0x9000, 0xA000, 64, 0xB000, 16, 0xC000, 0xF000, 64, 16, 1.0)
     assert f((fmsa_hip.BwdProj * 2)(m1, m2), 2, 8, 0, 0xD000, 64, None, None, None, 0, 1, None) == -5  # two masks
     assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 64, 12, 1, 0x3000, 16, None) == -5
+    # the flavour with a partial-sum buffer: same argument checks; the size query answers 0 where no buffer is used
+    dw, dws = lib.fmsa_lora_down_workspace, lib.fmsa_lora_down_ws
+    assert dw(8192, 4096, 16) == 0 and dw(512, 4096, 64) == 0 and dw(4096, 1024, 64) == 0 and dw(0, 4096, 64) == 0
+    assert dw(4096, 28672, 64) == 8 * 4096 * 64 * 4 and dw(8192, 4096, 32) == 2 * 8192 * 32 * 4
+    assert dw(4096, 8192, 128) == dw(4096, 8192, 64)   # above 64 ranks: 64 at a time through the same buffer
+    assert dw(16384, 14336, 32) == 0                   # enough tokens for a workgroup per CU: no column split
+    assert dws(None, 64, 0x2000, 8, 64, 16, 1, 0x3000, 16, None, 0, None) == -1
+    assert dws(0x1000, 64, 0x2000, 8, 64, 12, 1, 0x3000, 16, None, 0, None) == -5
+    assert dws(0x1000, 64, 0x2000, 8, 60, 16, 1, 0x3000, 16, None, 0, None) == -2
+    assert dws(0x1000, 64, 0x2000, 8, 64, 16, 1, 0x3000, 8, None, 0, None) == -2
+    assert dws(0x1000, 64, 0x2000, 8, 64, 16, 2, 0x3000, 16, None, 0, None) == -4
+    assert dws(0x1004, 64, 0x2000, 8, 64, 16, 1, 0x3000, 16, None, 0, None) == -3
+    assert dws(0x1000, 64, 0x2000, 8, 64, 16, 1, 0x3000, 16, 0x4004, 1 << 20, None) == -3
     assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 60, 16, 1, 0x3000, 16, None) == -2
     assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 64, 16, 1, 0x3000, 8, None) == -2   # ldout < r
     assert lib.fmsa_lora_grad_workspace(8192, 4096, 16) > 0

@@ -95,6 +95,47 @@ def test_lora_down_many_tokens(M, C, r, dtype):
     assert torch.equal(fmsa_hip.lora_down(x, wd), out)  # run-to-run bit-stable, whatever the output stride
 
 
+@pytest.mark.parametrize("M,C,r", [(4096, 8192, 64), (2048, 4096, 32), (2100, 2048, 128), (16384, 14336, 32)])
+def test_lora_down_with_and_without_workspace(M, C, r):
+    """From rank 32 on fmsa_lora_down_ws takes 64-128 tokens per workgroup and splits the columns over workgroups whose
+    sums meet in the workspace; without a workspace, or with an output the reduce pass cannot store into four ranks at a
+    time, it runs as fmsa_lora_down does.  Every route against the fp32 product; each is bit-stable run to run."""
+    import ctypes
+
+    import fmsa_hip
+
+    lib = fmsa_hip.lib()
+    dtype = torch.bfloat16
+    x = dev(randn((M, C), 21, dtype))
+    wd = dev(randn((r, C), 22, dtype, 0.05))
+    ref = (x.float() @ wd.float().t()).cpu()
+    need = lib.fmsa_lora_down_workspace(M, C, r)
+    assert (need > 0) == (M < 16384)  # 16384 tokens at rank 32: 256 workgroups of 64 tokens, no column split
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=x.device)
+
+    def run(out, workspace, nbytes):
+        rc = lib.fmsa_lora_down_ws(x.data_ptr(), x.stride(0), wd.data_ptr(), M, C, r, fmsa_hip.act_enum(dtype), out.data_ptr(),
+                                   out.stride(0), workspace, nbytes, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, rc
+        return out
+
+    with_ws = run(torch.empty(M, r, dtype=dtype, device=x.device), ws.data_ptr(), ws.numel())
+    assert torch.equal(with_ws, run(torch.empty_like(with_ws), ws.data_ptr(), ws.numel()))
+    without = run(torch.empty_like(with_ws), None, 0)
+    plain = fmsa_hip.lora_down(x, wd)
+    small = run(torch.empty_like(with_ws), ws.data_ptr(), max(need // 2, 1)) if need else without
+    odd = torch.zeros(M, r + 6, dtype=dtype, device=x.device)  # rows 4 bytes off an 8-byte boundary, stride % 4 != 0
+    run(odd[:, 2 : 2 + r], ws.data_ptr(), ws.numel())
+    for out in (with_ws, without, plain, small, odd[:, 2 : 2 + r]):
+        assert olora.max_rel_err(out.cpu(), ref) < 5e-3
+    assert torch.equal(plain, with_ws)      # the binding brings the workspace
+    assert torch.equal(small, without)      # too small a buffer is as good as none
+    assert torch.all(odd[:, :2] == 0) and torch.all(odd[:, 2 + r :] == 0)
+    if need:
+        assert lib.fmsa_lora_down_ws(x.data_ptr(), x.stride(0), wd.data_ptr(), M, C, r, fmsa_hip.act_enum(dtype), with_ws.data_ptr(),
+                                     with_ws.stride(0), ws.data_ptr() + 4, ws.numel() - 4, None) == -3
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,C,r,tr", [(512, 2048, 16, False), (200, 1056, 8, True), (4096, 4096, 16, True), (96, 136, 24, False), (70, 4104, 64, True),
                                       (1000, 2048, 96, False), (333, 520, 128, True)])
