@@ -55,7 +55,14 @@ _ROTATED = {}
 
 
 def mark_rotated(Q, K):
-    _ROTATED[Q.untyped_storage().data_ptr()] = (Q, K)
+    key = Q.untyped_storage().data_ptr()
+    _ROTATED[key] = (Q, K)
+    return key
+
+
+def unmark_rotated(key) -> bool:
+    """Drops a mark that was never consumed; True if it was still there."""
+    return _ROTATED.pop(key, None) is not None
 
 
 def fast_rope_embedding(Q, K, cos, sin, position_ids=None, unsqueeze_dim=1):

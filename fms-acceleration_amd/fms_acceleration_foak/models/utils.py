@@ -63,7 +63,7 @@ def _build_fused_forwards(attn: torch.nn.Module, fused_operation: Callable, subm
     tables = {}
 
     if rope_operation is not None:
-        from ..kernels.unsloth.rope_embedding import mark_rotated  # pylint: disable=import-outside-toplevel
+        from ..kernels.unsloth.rope_embedding import mark_rotated, unmark_rotated  # pylint: disable=import-outside-toplevel
 
         def _keep_tables(module, args, kwargs):
             tables["pe"] = kwargs.get("position_embeddings", args[1] if len(args) > 1 else None)
@@ -74,8 +74,14 @@ def _build_fused_forwards(attn: torch.nn.Module, fused_operation: Callable, subm
         if not any(n in pending for n in submodule_names):
             pe = tables.pop("pe", None)
             if rope_operation is not None and pe is not None and X.dim() == 3:
+                stale = tables.pop("marked", None)
+                if stale is not None and unmark_rotated(stale):
+                    # the Q / K of the previous call were never handed to apply_rotary_pos_emb: this attention does
+                    # not rotate what it is given position_embeddings for, and its outputs must not come rotated
+                    raise RuntimeError("fused Q/K/V with rotary embedding: the attention did not call apply_rotary_pos_emb "
+                                       "on the previous projections; use fast_rope_embeddings: true for this model")
                 outs = rope_operation(attn, X, pe[0], pe[1])
-                mark_rotated(outs[0], outs[1])
+                tables["marked"] = mark_rotated(outs[0], outs[1])
             else:
                 outs = fused_operation(attn, X)
             outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]

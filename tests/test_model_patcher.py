@@ -260,10 +260,21 @@ def test_qkv_wrapper_with_rope_tables():
     with pytest.raises(RuntimeError, match="K does not"):
         re_mod.fast_rope_embedding(q, k.clone(), None, None)
     assert not re_mod._ROTATED
+    # an attention that is given tables but never rotates: the second call finds the first mark unconsumed and refuses
+    class NoRope(torch.nn.Module):
+        def forward(self, hidden_states, position_embeddings=None):
+            return [fwd2[n](None, hidden_states) for n in names]
+
+    lazy = NoRope()
+    fwd2 = dict(_build_fused_forwards(lazy, plain, names, with_rope))
+    lazy(x, position_embeddings=("c", "s"))
+    with pytest.raises(RuntimeError, match="did not call apply_rotary_pos_emb"):
+        lazy(x, position_embeddings=("c", "s"))
+    assert not re_mod._ROTATED
     # without tables the plain fused operation runs and nothing is marked
     for n in names:
         out = fwd[n](None, x)
-    assert out.flatten()[0] == 3 and not re_mod._ROTATED and len(seen) == 1
+    assert out.flatten()[0] == 3 and not re_mod._ROTATED and len(seen) == 2  # (the two calls with tables above)
 
 
 def test_fast_rope_embeddings_fused_qkv_is_accepted():
