@@ -66,13 +66,16 @@ struct FwdArgs {
 FMSA_DEVI FwdProjDev select_proj(const FwdArgs& a, int p) { return p == 0 ? a.p[0] : (p == 1 ? a.p[1] : a.p[2]); }
 
 // GPS = scale groups per 64-wide K stage: 1 for group_size % 64 == 0, 2 / 4 for group sizes 32 / 16.
-// CODEBOOK: the nibbles index a 16-entry table and one fp32 scale per (group, column) multiplies the
-// entry (W = code[q] * block_scale); otherwise the affine GPTQ form W = scale * (q - zero).
+// CODEBOOK (1, 2): the nibbles index a 16-entry table and one fp32 scale per (group, column) multiplies the
+// entry (W = code[q] * block_scale); 0: the affine GPTQ form W = scale * (q - zero).  1 gathers code[q] from the
+// lanes of the wave (one ds_bpermute per weight) and multiplies; 2 (GPS == 1) multiplies the 16 entries by the lane's
+// block scale once per stage and column, keeps the 16 rounded products as two byte planes in registers, and looks the
+// weights up with byte permutes: the same products, no gather on the LDS pipe that the X fragments keep busy.
 // ROPE (1: cos / sin tables in the activation type, 2: in fp32; 0: none): the Q / K projections of an attention block
 // leave the kernel with the rotary embedding applied
 // (kernels/unsloth/rope_embedding.py:36-65 of the reference: (q1, q2) <- (q1 cos - q2 sin, q2 cos + q1 sin) on the two
 // halves of every head, on the projection output ROUNDED to the storage type, fp32 arithmetic, one more rounding).
-template <typename T, int GPS, bool KTAIL, bool CODEBOOK, int ROPE = 0>
+template <typename T, int GPS, bool KTAIL, int CODEBOOK, int ROPE = 0>
 __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // two separate arrays (not one 2-D array): every access names its buffer statically, which is
   // what lets the compiler see that fragment reads of one buffer do not depend on the direct loads
@@ -136,10 +139,26 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     gs[j] = __builtin_amdgcn_readfirstlane(P.group_size);
     qbase[j] = reinterpret_cast<const char*>(P.qweight);
     scbase[j] = CODEBOOK ? reinterpret_cast<const char*>(P.block_scale) : reinterpret_cast<const char*>(P.scales);
-    lut[j] = CODEBOOK ? P.code[lane & 15] : 0.f;
+    lut[j] = CODEBOOK == 1 ? P.code[lane & 15] : 0.f;
     zbase[j] = reinterpret_cast<const char*>(P.qzeros);
     zshift[j] = 4 * (col & 7);
     zoff[j] = (float)P.zero_offset;
+  }
+
+  // table flavour: the code book as wave-uniform values (the launcher takes this flavour only when the projections of
+  // the launch share one code book), and per column tile the byte planes of the current stage's 16 rounded products:
+  // byte e of tlo[set][j][d] / thi[set][j][d] = low / high byte of entry 4 d + e.  Two sets: while the stage in slot SB
+  // looks its weights up in set SB, the steps of that stage build set SB ^ 1 for the next one, a quarter per step, so
+  // the 80 instructions of a table pair sit between MFMAs like the rest.  That needs the block scale one stage earlier
+  // than the weights: load_stage(st) fetches the scale of stage st + 1.
+  float cd[16];
+  uint32_t tlo[NBUF][NT][4], thi[NBUF][NT][4];
+  int gshift[NT];  // log2 of the block size (the launcher takes this flavour for powers of two only)
+  if constexpr (CODEBOOK == 2) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) cd[i] = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(a.p[0].code[i])));
+#pragma unroll
+    for (int j = 0; j < NT; ++j) gshift[j] = 31 - __builtin_clz(gs[j]);
   }
 
   const int K = a.K;
@@ -240,7 +259,10 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
           gu = (ku < K ? ku : st * BK) / gs[j];
         }
         gu = __builtin_amdgcn_readfirstlane(gu);  // uniform; keeps the scalar offsets out of vector registers
-        if constexpr (CODEBOOK) {
+        if constexpr (CODEBOOK == 2) {
+          const int g1 = __builtin_amdgcn_readfirstlane(min(((st + 1) * BK) >> gshift[j], n_groups_j[j] - 1));
+          zw_raw[SB ^ 1][j][u] = __builtin_amdgcn_raw_buffer_load_b32(sc_rsrc[j], sc_off[j], (uint32_t)g1 * Np[j] * 4, 0);
+        } else if constexpr (CODEBOOK == 1) {
           zw_raw[SB][j][u] = __builtin_amdgcn_raw_buffer_load_b32(sc_rsrc[j], sc_off[j], (uint32_t)gu * Np[j] * 4, 0);
         } else {
           sc_raw[SB][j][u] = __builtin_amdgcn_raw_buffer_load_b16(sc_rsrc[j], sc_off[j], (uint32_t)gu * Np[j] * 2, 0);
@@ -262,7 +284,9 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     for (int j = 0; j < NT; ++j) {
 #pragma unroll
       for (int u = 0; u < GPS; ++u) {
-        if constexpr (CODEBOOK) {
+        if constexpr (CODEBOOK == 2) {
+          // (the tables are built step by step in prefetch)
+        } else if constexpr (CODEBOOK == 1) {
           sf[j][u] = __uint_as_float(zw_raw[SB][j][u]);
         } else {
           sf[j][u] = fp16_bits_to_f32(sc_raw[SB][j][u]);
@@ -279,6 +303,19 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // into the other half of xf / wf.  The stage barrier sits after step 2, so step 3 can already
   // fetch step 0 of the next stage from the next LDS buffer.
   u32x4 xf[2][MT], wf[2][NT];
+  // entries 4 d .. 4 d + 3 of table set SET from the block scales in raw slot SET: the products rounded to the storage
+  // type in pairs, then the two byte planes
+  auto build_table_part = [&](auto set_c, auto d_c) {
+    constexpr int SET = decltype(set_c)::value;
+    constexpr int d = decltype(d_c)::value;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const float sc = __uint_as_float(zw_raw[SET][j][0]);
+      const uint32_t p0 = pack2<T>(cd[4 * d] * sc, cd[4 * d + 1] * sc), p1 = pack2<T>(cd[4 * d + 2] * sc, cd[4 * d + 3] * sc);
+      tlo[SET][j][d] = __builtin_amdgcn_perm(p1, p0, 0x06040200u);
+      thi[SET][j][d] = __builtin_amdgcn_perm(p1, p0, 0x07050301u);
+    }
+  };
   auto prefetch = [&](auto sb_c, auto t_c, auto par_c) {
     constexpr int SB = decltype(sb_c)::value;
     constexpr int t = decltype(t_c)::value;
@@ -287,7 +324,29 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2);
 #pragma unroll
-    for (int j = 0; j < NT; ++j) wf[par][j] = dequant8<T>(qw[SB][j][t], sf[j][t * GPS / 4], sf16[j][t * GPS / 4], nsz[j][t * GPS / 4]);
+    for (int j = 0; j < NT; ++j) {
+      if constexpr (CODEBOOK == 2) {
+        // nibble 2b / 2b + 1 of the word (weights k = 2b, 2b + 1 of the step) sit in byte b: per byte plane two
+        // permutes over entries 0-7 and 8-15 with the nibble's low three bits, a third picks by its top bit
+        const uint32_t w = qw[SB][j][t];
+        const uint32_t se = w & 0x07070707u, so = (w >> 4) & 0x07070707u;
+        const uint32_t pe = ((w >> 1) & 0x04040404u) | 0x03020100u, po = ((w >> 5) & 0x04040404u) | 0x03020100u;
+        const uint32_t loe = __builtin_amdgcn_perm(__builtin_amdgcn_perm(tlo[SB][j][3], tlo[SB][j][2], se), __builtin_amdgcn_perm(tlo[SB][j][1], tlo[SB][j][0], se), pe);
+        const uint32_t hie = __builtin_amdgcn_perm(__builtin_amdgcn_perm(thi[SB][j][3], thi[SB][j][2], se), __builtin_amdgcn_perm(thi[SB][j][1], thi[SB][j][0], se), pe);
+        const uint32_t loo = __builtin_amdgcn_perm(__builtin_amdgcn_perm(tlo[SB][j][3], tlo[SB][j][2], so), __builtin_amdgcn_perm(tlo[SB][j][1], tlo[SB][j][0], so), po);
+        const uint32_t hio = __builtin_amdgcn_perm(__builtin_amdgcn_perm(thi[SB][j][3], thi[SB][j][2], so), __builtin_amdgcn_perm(thi[SB][j][1], thi[SB][j][0], so), po);
+        // 16-bit values of weights (0, 2), (4, 6) and (1, 3), (5, 7), then the pairs (k, k + 1) the fragment holds
+        const uint32_t e01 = __builtin_amdgcn_perm(hie, loe, 0x05010400u), e23 = __builtin_amdgcn_perm(hie, loe, 0x07030602u);
+        const uint32_t o01 = __builtin_amdgcn_perm(hio, loo, 0x05010400u), o23 = __builtin_amdgcn_perm(hio, loo, 0x07030602u);
+        wf[par][j][0] = __builtin_amdgcn_perm(o01, e01, 0x05040100u);
+        wf[par][j][1] = __builtin_amdgcn_perm(o01, e01, 0x07060302u);
+        wf[par][j][2] = __builtin_amdgcn_perm(o23, e23, 0x05040100u);
+        wf[par][j][3] = __builtin_amdgcn_perm(o23, e23, 0x07060302u);
+      } else {
+        wf[par][j] = dequant8<T>(qw[SB][j][t], sf[j][t * GPS / 4], sf16[j][t * GPS / 4], nsz[j][t * GPS / 4]);
+      }
+    }
+    if constexpr (CODEBOOK == 2) build_table_part(std::integral_constant<int, SB ^ 1>{}, t_c);
   };
   // Code-book flavour in two phases, so that a step's first 8 MFMAs cover the table gathers and its
   // last 8 the arithmetic on what they returned.  Phase a: the 8 X fragments and the 16 gathers
@@ -348,7 +407,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, CODEBOOK == 2 ? 5 : 3, 0);
       if ((i & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       if (with_vmem) {
         if (i < 6)
@@ -403,7 +462,7 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   // one 16-wide K step: the MFMAs of parity `cur` while fragments and weights of (buffer nb, step nt)
   // are produced into parity `nx`
   auto step = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c) {
-    if constexpr (CODEBOOK) {
+    if constexpr (CODEBOOK == 1) {
       prefetch_a(nb_c, nt_c, nx_c);
       mfma_half(cur_c, I0{});
       interleave_a();
@@ -457,12 +516,22 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
                                                16, (uint32_t)(((col0[j] + prow) * rp + 8 * phalf) * 2) | dead, 0, 0, 0);
     }
   }
+  if constexpr (CODEBOOK == 2) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) zw_raw[0][j][0] = __builtin_amdgcn_raw_buffer_load_b32(sc_rsrc[j], sc_off[j], 0, 0);
+  }
   load_stage(0, I0{});
   __builtin_amdgcn_s_waitcnt(WAIT_VM0);
   commit_stage(I0{});
+  if constexpr (CODEBOOK == 2) {  // the first stage's tables, all at once
+    build_table_part(I0{}, I0{});
+    build_table_part(I0{}, I1{});
+    build_table_part(I0{}, I2{});
+    build_table_part(I0{}, I3{});
+  }
   __syncthreads();
   load_stage(min(1, n_stages - 1), I1{});
-  if constexpr (CODEBOOK) {
+  if constexpr (CODEBOOK == 1) {
     prefetch_a(I0{}, I0{}, I0{});
     prefetch_b(I0{}, I0{});
   } else {
@@ -783,6 +852,10 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
   }
   const bool ktail = (a.K % BK) != 0;
   const bool codebook = projs[0].w.format == FMSA_WEIGHT_CODEBOOK;  // api.hip: all projections of a launch share the format
+  // table flavour: one code book for the launch, one block per 64-wide stage
+  bool table = codebook && gps == 1 && !rope;
+  for (int p = 0; p < n_proj; ++p)
+    table = table && projs[p].w.code == projs[0].w.code && (projs[p].w.group_size & (projs[p].w.group_size - 1)) == 0;
 #define LAUNCH3(TT, KT, CB)                                                                          \
   do {                                                                                               \
     if (rope && rope->dtype == FMSA_F32) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, false, CB, 2>), grid, block, 0, st, a); \
@@ -793,8 +866,9 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
   } while (0)
 #define LAUNCH2(TT, KT)          \
   do {                           \
-    if (codebook) LAUNCH3(TT, KT, true); \
-    else LAUNCH3(TT, KT, false); \
+    if (table) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, KT, 2>), grid, block, 0, st, a); \
+    else if (codebook) LAUNCH3(TT, KT, 1); \
+    else LAUNCH3(TT, KT, 0); \
   } while (0)
 #define LAUNCH(TT)            \
   do {                        \

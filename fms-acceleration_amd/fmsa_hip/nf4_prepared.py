@@ -33,6 +33,22 @@ def normalize_quant_state(quant_state):
     return _State(absmax=absmax, shape=tuple(shape), dtype=dtype, blocksize=blocksize, offset=offset, state2=state2, code=code)
 
 
+_code_books = {}
+
+
+def _shared_code_book(code, device):
+    """One device copy per distinct 16-entry code book: weights quantised with the same book (all NF4 weights of a
+    model) then hand the kernels the same pointer, which is what lets a launch over several projections keep the
+    book in scalar registers.  Read once per prepared weight, on the same path as the re-layout of its codes."""
+    host = code.detach().to(device="cpu", dtype=torch.float32).reshape(-1)
+    key = (device.type, device.index, tuple(host.tolist()))
+    book = _code_books.get(key)
+    if book is None:
+        book = host.to(device).contiguous()
+        _code_books[key] = book
+    return book
+
+
 class PreparedNf4Weight:
     """The C-ABI view (`struct`, code-book format) of one NF4 linear of shape [N, K]."""
 
@@ -54,7 +70,7 @@ class PreparedNf4Weight:
                 f"divisible by 32 (got [{N}, {K}], blocksize {bs})")
         qweight, block_scale = fmsa_hip.nf4_prepare(data.reshape(-1), quant_state.absmax, state2.absmax, state2.code,
                                                     float(quant_state.offset), (N, K), bs, int(state2.blocksize))
-        code = quant_state.code.to(device=data.device, dtype=torch.float32).contiguous()
+        code = _shared_code_book(quant_state.code, data.device)
         self.K, self.N, self.group_size = K, N, bs
         self.perm = self.perm_key = None  # no act-order for NF4
         self.nsz = None   # the input-gradient kernel reads block_scale through the struct
