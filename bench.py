@@ -516,7 +516,8 @@ def yardsticks(device):
     out = {"library_bf16_gemm": {"shape": f"[{M_TOKENS}, {HIDDEN}] x [{HIDDEN}, {2 * INTER}]", "ms": t * 1e3,
                                  "tflops": 2.0 * M_TOKENS * HIDDEN * 2 * INTER / t / 1e12}}
     del x, w, y
-    for mode, name in ((0, "mfma_loop_zero_operands"), (1, "mfma_loop_random_operands"), (2, "mfma_loop_random_operands_with_direct_loads")):
+    for mode, name in ((0, "mfma_loop_zero_operands"), (1, "mfma_loop_random_operands"), (2, "mfma_loop_random_operands_with_direct_loads"),
+                       (3, "mfma_loop_random_operands_with_direct_loads_and_lds_fragment_reads")):
         flop = [0.0]
 
         def run():

@@ -651,6 +651,7 @@ def cross_entropy_fused_(logits2d, labels, scale=None, label_smoothing=0.0, igno
 def probe_mfma(mode: int, iters: int = 20000, n_workgroups: int = 1024, device="cuda"):
     """Launches the register-only MFMA loop (see fmsa_probe_mfma in include/fmsa.h); returns its FLOP count."""
     out = torch.empty(n_workgroups * 256, dtype=torch.float32, device=device)
-    src = torch.zeros(1 << 18, dtype=torch.int32, device=device)
+    # bf16 pairs in +-[1, 2), the kind of operand the loop keeps in registers (mode 3 feeds them to the MFMAs through LDS)
+    src = (torch.randint(0, 1 << 32, (1 << 18,), dtype=torch.int64, device=device) & 0x807F807F | 0x3F803F80).to(torch.int32)
     _check("fmsa_probe_mfma", lib().fmsa_probe_mfma(mode, iters, n_workgroups, _ptr(out), _ptr(src), _stream(out)))
     return float(n_workgroups) * 4 * iters * 16 * 32768.0

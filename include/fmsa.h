@@ -375,7 +375,9 @@ int fmsa_cross_entropy_fused(void* logits, int64_t ld, const int64_t* labels, in
  *   mode 0  all-zero operands (what the clock allows),
  *   mode 1  random bf16 operands (what the power limit leaves),
  *   mode 2  as 1, plus one 1 KB direct-to-LDS load per wave and 8 MFMAs from `src` (>= 1 MiB), the
- *           ratio of the GEMM kernels' main loops.
+ *           ratio of the GEMM kernels' main loops,
+ *   mode 3  as 2, with the A operands read from LDS (one 1 KB fragment read per wave and 2 MFMAs, a workgroup
+ *           barrier per 64 MFMAs): the operand traffic of a main loop without the unpacking.
  * FLOP of a launch = n_workgroups * 4 * iters * 16 * 32768.  `out`: n_workgroups * 256 floats.
  * ------------------------------------------------------------------------------------------ */
 int fmsa_probe_mfma(int mode, int iters, int n_workgroups, void* out, const void* src, void* stream);
