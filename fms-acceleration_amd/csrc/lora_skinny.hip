@@ -458,10 +458,9 @@ __global__ __launch_bounds__(256) void lora_down_reduce_kernel(const float* __re
 // ---- lora_grad ----------------------------------------------------------------------------------
 // out[j, c] = sum_m L[m, j] * R[m, c]: the contraction runs over tokens, which is the row index of
 // both row-major operands, so each MFMA fragment (8 consecutive contraction elements per lane) is a
-// column walk.  Tiles of 32 tokens are staged through LDS (coalesced 16-byte global loads in, 16-bit
-// column reads out); the 32 tokens of a tile are assigned to the MFMA's contraction index as
-// k = 8*kg + e  <->  token 4*e + kg, and rows are padded by 32 B, which makes the four kg groups of a
-// wave hit disjoint banks.
+// column walk.  Tiles of 32 tokens are staged through LDS (coalesced 16-byte global loads in, transposing
+// 8-byte reads out: column_frag below); token e of a tile is the MFMA's contraction index e, rows are padded
+// by 32 B.
 // Pass 1: workgroup = 128 columns of R x one fixed range of tokens (split); wave w owns columns
 // 32w .. 32w+31 (two 16-wide MFMA tiles) and all r ranks.  Partial sums go to partial[split][r][C]
 // (fp32).  Pass 2 adds the splits in index order, so the result does not depend on scheduling.
@@ -511,9 +510,11 @@ FMSA_DEVI LoraGradJobDev select_job(const LoraGradArgs& a, int block) {
 // LDS and are summed in wave order by the whole workgroup one iteration later (behind the barrier the
 // loop has anyway), and leave as the column block's partial T[column block][token][rank] (fp32).  The
 // reduce pass adds the column blocks in index order and rounds once: deterministic like the rest.
-template <typename T, int RT, bool WITH_T>
-__global__ __launch_bounds__(WITH_T ? 512 : 256) void lora_grad_partial_kernel(const LoraGradArgs a) {
-  constexpr int NWV = WITH_T ? 8 : 4;       // waves
+// WIDE: eight waves and 256 columns per workgroup without the T product, for ranks from 48 on: the L tile every workgroup
+// re-reads is r / 128 of the R bytes it consumes at 128 columns, half that at 256.
+template <typename T, int RT, bool WITH_T, bool WIDE = false>
+__global__ __launch_bounds__((WITH_T || WIDE) ? 512 : 256) void lora_grad_partial_kernel(const LoraGradArgs a) {
+  constexpr int NWV = (WITH_T || WIDE) ? 8 : 4;  // waves
   constexpr int NTH = 64 * NWV;             // threads
   constexpr int TC = 32 * NWV;              // columns of R per workgroup
   constexpr int LG_RSTRIDE = TC + 16;       // elements: row + 32 B pad
@@ -580,16 +581,18 @@ __global__ __launch_bounds__(WITH_T ? 512 : 256) void lora_grad_partial_kernel(c
     for (int p = 0; p < LP; ++p)
       if (l_thread[p]) *reinterpret_cast<u32x4*>(&l_lds[buf][l_row[p] * LSTRIDE + 8 * l_chunk[p]]) = lst[p];
   };
-  // 8 contraction elements of column `col`: tokens 4*e + kg, e = 0..7
-  auto column_frag = [&](const uint16_t* base, int stride, int col) {
-    u32x4 f;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const uint32_t lo = base[(8 * e + kg) * stride + col];
-      const uint32_t hi = base[(8 * e + 4 + kg) * stride + col];
-      f[e] = lo | (hi << 16);
-    }
-    return f;
+  // The MFMA operand of a 16-column tile starting at column `col0`: lane 16 kg + m gets column col0 + m at the 8 tokens
+  // 8 kg .. 8 kg + 7 (contraction index k = 8 kg + e <-> token 8 kg + e of the tile).  Two transposing LDS reads
+  // (ds_read_b64_tr_b16) do it: in a group of 16 lanes, lane 4 a + b receives element b of the four 16-bit values that
+  // lanes a, a + 4, a + 8, a + 12 address, so lane j of the group addresses token 8 kg + 4 h + j / 4, columns
+  // col0 + 4 (j % 4) .. + 3 (h = 0, 1: the two reads).  Was eight 16-bit reads and their packing per operand.
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  auto column_frag = [&](const uint16_t* base, int stride, int col0) {
+    const uint16_t* p = base + (8 * kg + (l16 >> 2)) * stride + col0 + 4 * (l16 & 3);
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p + 4 * stride));
+    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+    return u32x4{l2[0], l2[1], h2[0], h2[1]};
   };
 
   f32x4 acc[2][RT];
@@ -651,9 +654,9 @@ __global__ __launch_bounds__(WITH_T ? 512 : 256) void lora_grad_partial_kernel(c
     u32x4 lf[RT], rf[2];
 #pragma unroll
     for (int t = 0; t < RT; ++t)
-      if (t < rt) lf[t] = column_frag(l_lds[buf], LSTRIDE, 16 * t + l16);
+      if (t < rt) lf[t] = column_frag(l_lds[buf], LSTRIDE, 16 * t);
 #pragma unroll
-    for (int g = 0; g < 2; ++g) rf[g] = column_frag(r_lds[buf], LG_RSTRIDE, 32 * wave + 16 * g + l16);
+    for (int g = 0; g < 2; ++g) rf[g] = column_frag(r_lds[buf], LG_RSTRIDE, 32 * wave + 16 * g);
 #pragma unroll
     for (int t = 0; t < RT; ++t)
       if (t < rt) {
@@ -913,7 +916,10 @@ int launch_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, in
   a.act_dtype = act_dtype;
   bool any_t = false;
   for (int q = 0; q < n_jobs; ++q) any_t = any_t || jobs[q].Wt != nullptr;
-  const int tc = any_t ? LG_TC_T : LG_TC;  // the launch's flavour decides the column-block width of all its jobs
+  int r_all = 0;
+  for (int q = 0; q < n_jobs; ++q) r_all = jobs[q].r > r_all ? jobs[q].r : r_all;
+  const bool wide = any_t || r_all > 32;
+  const int tc = wide ? LG_TC_T : LG_TC;  // the launch's flavour decides the column-block width of all its jobs
   int blocks = 0, rblocks = 0, r_max = 0;
   size_t ws_off = 0;
   for (int q = 0; q < n_jobs; ++q) {
@@ -948,15 +954,15 @@ int launch_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, in
     }
     r_max = s.r > r_max ? s.r : r_max;
   }
-  dim3 grid1(blocks), grid2(rblocks), block(256), block1(any_t ? 512 : 256);
+  dim3 grid1(blocks), grid2(rblocks), block(256), block1(wide ? 512 : 256);
   const int rt = (r_max + 15) / 16;
 #define LAUNCH(TT, RT, WT) hipLaunchKernelGGL((lora_grad_partial_kernel<TT, RT, WT>), grid1, block1, 0, st, a)
 #define DISPATCH(TT)                                                  \
   switch (rt) {                                                       \
     case 1: if (any_t) LAUNCH(TT, 1, true); else LAUNCH(TT, 1, false); break; \
     case 2: if (any_t) LAUNCH(TT, 2, true); else LAUNCH(TT, 2, false); break; \
-    case 3: case 4: LAUNCH(TT, 4, false); break;                      \
-    default: LAUNCH(TT, 8, false); break;                             \
+    case 3: case 4: hipLaunchKernelGGL((lora_grad_partial_kernel<TT, 4, false, true>), grid1, block1, 0, st, a); break; \
+    default: hipLaunchKernelGGL((lora_grad_partial_kernel<TT, 8, false, true>), grid1, block1, 0, st, a); break;         \
   }
   if (act_dtype == FMSA_BF16) {
     DISPATCH(bf16_t)
