@@ -823,13 +823,16 @@ int launch_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, i
 
 namespace {
 // Shape of the split launch: row groups per workgroup, column ranges, or g = 0 when the kernels without workspace do as
-// well (rank 16 and below: Wd is a quarter of the X bytes a 32-token workgroup reads) or the matrix is too small.
+// well or the matrix is too small.  (At rank 16 and below Wd is a small part of the traffic; what the split kernel adds there
+// is 64 tokens per workgroup with 1 KB row runs through LDS and column ranges that keep every CU busy: 21 -> 17 us on
+// 8192 x 4096.)
 struct DownSplit {
   int g, n_tb, n_split;
 };
 DownSplit lora_down_split_shape(int M, int C, int r) {
   const int rt = (std::min(r, 64) + 15) / 16;  // ranks above 64 go out 64 at a time (accumulator registers)
-  if (rt < 2 || M < 2048 || C < 2048) return {0, 0, 0};
+  if (M < 2048 || C < 2048) return {0, 0, 0};
+  if (rt < 2 && M >= 16384) return {0, 0, 0};  // rank 16 and below with a workgroup per CU anyway: the 32-token kernels do as well
   const int g = rt <= 2 ? 2 : 4;  // rank 32: 64 tokens per workgroup; 48 / 64: 128
   const int n_tb = (M + 32 * g - 1) / (32 * g);
   const int n_chunks = (C + 511) / 512;
@@ -869,6 +872,7 @@ int launch_lora_down_ws(const void* X, int64_t ldx, const void* Wd, int M, int C
                      C, r, (uint16_t*)out, ldo, (float*)workspace, d.n_tb, d.n_split)
 #define SPLIT_DISPATCH(TT)                            \
   switch (rt) {                                       \
+    case 1: SPLIT_LAUNCH(TT, 1, 2); break;            \
     case 2: SPLIT_LAUNCH(TT, 2, 2); break;            \
     default: SPLIT_LAUNCH(TT, 4, 4); break;           \
   }

@@ -108,8 +108,8 @@ int fmsa_permute_cols(const void* in, int64_t ld_in, const int32_t* perm, int M,
 int fmsa_lora_down(const void* X, int64_t ldx, const void* Wd, int M, int C, int r, int act_dtype,
                    void* out, int64_t ldout, void* stream);
 
-/* The same product with a partial-sum buffer at hand (same reference lines as fmsa_lora_down).  From rank 32 on a
- * workgroup takes 64-128 tokens, so that Wd is re-read that much less often, and where M then leaves CUs without work
+/* The same product with a partial-sum buffer at hand (same reference lines as fmsa_lora_down).  A workgroup takes
+ * 64-128 tokens, so that Wd is re-read that much less often, and where M then leaves CUs without work
  * the columns are split over workgroups whose fp32 sums meet in `workspace` ([splits][M][r] fp32, no initialisation
  * needed, added in index order: the result does not depend on scheduling).  fmsa_lora_down_workspace gives the bytes
  * (0: the call needs none); with a buffer that is missing, too small, or an `out` that is not 8-byte aligned with

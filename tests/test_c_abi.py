@@ -159,7 +159,8 @@ def test_bwd_and_skinny_validation():
     assert lib.fmsa_lora_down(0x1000, 64, 0x2000, 8, 64, 12, 1, 0x3000, 16, None) == -5
     # the flavour with a partial-sum buffer: same argument checks; the size query answers 0 where no buffer is used
     dw, dws = lib.fmsa_lora_down_workspace, lib.fmsa_lora_down_ws
-    assert dw(8192, 4096, 16) == 0 and dw(512, 4096, 64) == 0 and dw(4096, 1024, 64) == 0 and dw(0, 4096, 64) == 0
+    assert dw(16384, 4096, 16) == 0 and dw(512, 4096, 64) == 0 and dw(4096, 1024, 64) == 0 and dw(0, 4096, 64) == 0
+    assert dw(8192, 4096, 16) == 2 * 8192 * 16 * 4
     assert dw(4096, 28672, 64) == 8 * 4096 * 64 * 4 and dw(8192, 4096, 32) == 2 * 8192 * 32 * 4
     assert dw(4096, 8192, 128) == dw(4096, 8192, 64)   # above 64 ranks: 64 at a time through the same buffer
     assert dw(16384, 14336, 32) == 0                   # enough tokens for a workgroup per CU: no column split
