@@ -73,9 +73,12 @@ def dequant_absmax(q) -> np.ndarray:
     return (q["code2"][q["absmax_q"]] * q["absmax2"][b // q["blocksize2"]]).astype(np.float32) + np.float32(q["offset"])
 
 
-def dequant(q, out="bf16"):
-    """Dense weight [N, K] (row-major, as stored), one RNE rounding of the fp32 product to `out`."""
+def dequant(q, out="bf16", code=None):
+    """Dense weight [N, K] (row-major, as stored), one RNE rounding of the fp32 product to `out`.  `code`: the 16-entry
+    code book the indices refer to (the quant state's `code`; default the NF4 table)."""
     import torch
+
+    NF4 = globals()["NF4"] if code is None else np.asarray(code, dtype=np.float32)  # noqa: N806
 
     absmax = dequant_absmax(q)
     p = q["packed"].reshape(-1)

@@ -222,6 +222,35 @@ def test_codebook_kernels(M, K, N, r, blocksize, dtype):
     assert olora.max_rel_err(dx.cpu(), dx_ref) < TOL
 
 
+def test_other_code_book():
+    """The kernels take the 16-entry code book from the quant state: with bitsandbytes' FP4 table (not sorted, two
+    zeros) in place of NF4 the dense weight, the fused forward (the flavour that keeps rounded products in registers)
+    and the input gradient follow the oracle with the same table."""
+    import fmsa_hip
+
+    fp4 = (np.array([0, 0.0625, 8, 12, 4, 6, 2, 3, -0.0, -0.0625, -8, -12, -4, -6, -2, -3], dtype=np.float64) / 12).astype(np.float32)
+    N, K, M, r, dtype = 256, 512, 200, 16, torch.bfloat16
+    w, keep, q = _prepared(N, K, 77)
+    code = torch.from_numpy(fp4).cuda()
+    w = fmsa_hip.make_codebook_weight(keep[0], code, keep[1], 64)
+    Wd = fmsa_hip.weight_dequant(w, torch.device("cuda"), dtype)
+    assert torch.equal(Wd.cpu(), onf4.dequant(q, "bf16", code=fp4).t().contiguous())
+    W = onf4.dequant(q, "fp32", code=fp4).t().contiguous()
+    A, B = olora.make_lora(K, N, r, 5)
+    A16, B16 = A.to(dtype), B.to(dtype)
+    x = randn((M, K), 6, dtype)
+    xd = x.cuda()
+    U = fmsa_hip.lora_down(xd, A16.cuda())
+    (y,) = fmsa_hip.gptq_lora_fwd(xd, [{"w": w, "U": U, "B": B16.cuda(), "bias": None, "r": r, "s": 2.0}])
+    assert olora.max_rel_err(y.cpu(), olora.lora_linear(x.float(), W, A16.float(), B16.float(), 2.0, None)) < TOL
+    dy = randn((M, N), 8, dtype)
+    T = fmsa_hip.lora_down(dy.cuda(), B16.t().contiguous().cuda())
+    dx = fmsa_hip.gptq_lora_bwd_dx([{"w": w, "nsz": None, "dY": dy.cuda(), "T": T, "At": A16.t().contiguous().cuda(), "mask_src": xd,
+                                     "r": r, "s": 2.0}], M, K)
+    dx_ref, _, _ = olora.lora_w_manual(x.float(), W, A16.float(), B16.float(), 2.0, dy.float())
+    assert olora.max_rel_err(dx.cpu(), dx_ref) < TOL
+
+
 def test_list_style_quant_state_is_accepted():
     """The older bitsandbytes quant state, a list of lists (reference fused_ops/unsloth_lora/utils.py:100-105), gives
     the same dense weight and the same prepared weight as the object form; a list without compressed statistics raises."""
