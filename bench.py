@@ -488,6 +488,33 @@ def qkv_rope_config(device, dtype, attn, steps=200, warmup=20):
             "us_with_rope_in_epilogue": us["in_epilogue"]}
 
 
+def attention_config(device, dtype, attn, steps=20, warmup=5):
+    """The attention half of the layer alone (the baseline description's third configuration): LoRA_QKV + LoRA_W(o_proj)
+    forward + backward at the Llama-3-8B shape."""
+    import torch
+
+    from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_o_v2, apply_lora_qkv
+
+    gen = torch.Generator(device=device).manual_seed(3)
+    rn = lambda *s: torch.randn(*s, generator=gen, device=device).to(dtype)  # noqa: E731
+    x_attn, x_o = rn(1, M_TOKENS, HIDDEN).requires_grad_(True), rn(1, M_TOKENS, N_HEADS * HEAD_DIM).requires_grad_(True)
+    grads = [rn(1, M_TOKENS, N_HEADS * HEAD_DIM), rn(1, M_TOKENS, N_KV * HEAD_DIM), rn(1, M_TOKENS, N_KV * HEAD_DIM), rn(1, M_TOKENS, HIDDEN)]
+    params = [p for p in attn.parameters() if p.requires_grad]
+
+    def step():
+        for t in (x_attn, x_o, *params):
+            t.grad = None
+        Q, K, V = apply_lora_qkv(attn, x_attn)
+        O = apply_lora_o_v2(attn.o_proj, x_o)
+        torch.autograd.backward([Q, K, V, O], grads)
+
+    dt = time_steps(step, steps, warmup)
+    fl = layer_flops(M_TOKENS) - mlp_flops(M_TOKENS, HIDDEN, INTER, RANK)
+    return {"ms_per_step": dt * 1e3, "tokens_per_s": M_TOKENS / dt, "tflops": fl / dt / 1e12,
+            "frac_bf16_mfma_peak": fl / dt / 1e12 / PEAK_BF16_TFLOPS,
+            "workload": "LoRA_QKV + LoRA_W(o_proj) fwd+bwd, 8192 tokens, 32 + 8 heads of 128, GPTQ g128, r=16"}
+
+
 def yardsticks(device):
     """What the machine at hand sustains, next to the fused kernels' figures: the vendor library's plain bf16 GEMM of
     the gate/up shape (no dequantisation, no LoRA, no SwiGLU), and the register-only MFMA loop of the library with
@@ -663,9 +690,11 @@ def main():
     if not args.no_other_configs:
         del step
         rope_cfg = qkv_rope_config(device, dtype, attn)
+        attn_cfg = attention_config(device, dtype, attn)
         attn = None
         torch.cuda.empty_cache()
         result["other_configs"] = other_configs(device, dtype, mlp)
+        result["other_configs"]["config3_llama3_8b_attention"] = attn_cfg
         result["other_configs"]["qkv_with_rope_llama3_8b"] = rope_cfg
     print(json.dumps(result))
 
