@@ -853,7 +853,7 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
   const bool ktail = (a.K % BK) != 0;
   const bool codebook = projs[0].w.format == FMSA_WEIGHT_CODEBOOK;  // api.hip: all projections of a launch share the format
   // table flavour: one code book for the launch, one block per 64-wide stage
-  bool table = codebook && gps == 1 && !rope;
+  bool table = codebook && gps == 1;
   for (int p = 0; p < n_proj; ++p)
     table = table && projs[p].w.code == projs[0].w.code && (projs[p].w.group_size & (projs[p].w.group_size - 1)) == 0;
 #define LAUNCH3(TT, KT, CB)                                                                          \
@@ -866,7 +866,9 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
   } while (0)
 #define LAUNCH2(TT, KT)          \
   do {                           \
-    if (table) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, KT, 2>), grid, block, 0, st, a); \
+    if (table && rope && rope->dtype == FMSA_F32) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, false, 2, 2>), grid, block, 0, st, a); \
+    else if (table && rope) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, false, 2, 1>), grid, block, 0, st, a); \
+    else if (table) hipLaunchKernelGGL((gptq_lora_fwd_kernel<TT, 1, KT, 2>), grid, block, 0, st, a); \
     else if (codebook) LAUNCH3(TT, KT, 1); \
     else LAUNCH3(TT, KT, 0); \
   } while (0)

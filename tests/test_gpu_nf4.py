@@ -205,14 +205,16 @@ def test_codebook_kernels(M, K, N, r, blocksize, dtype):
     (y,) = fmsa_hip.gptq_lora_fwd(xd, [{"w": w, "U": U, "B": B16.cuda(), "bias": bias.cuda(), "r": r, "s": s}])
     y_ref = olora.lora_linear(x.float(), W, A16.float(), B16.float(), s, bias.float())
     assert olora.max_rel_err(y.cpu(), y_ref) < TOL
-    if blocksize % 64 == 0 and K % 64 == 0:
-        # One block per 64-wide stage: the launch above took the flavour that keeps the 16 rounded products of a block
-        # and column as byte planes in registers.  The rotating entry point (here with no projection named) stays on the
-        # flavour that gathers the code values from the lanes and multiplies: the same products, bit for bit.
-        ones = torch.ones((M, 16), dtype=dtype, device="cuda")
-        (y_gather,) = fmsa_hip.gptq_lora_fwd(xd, [{"w": w, "U": U, "B": B16.cuda(), "bias": bias.cuda(), "r": r, "s": s}],
-                                             rope=(ones, ones, 16, 0))
-        assert torch.equal(y, y_gather)
+    if blocksize % 64 == 0:
+        # One block per 64-wide stage and one code book for the launch: the launch above took the flavour that keeps the
+        # 16 rounded products of a block and column as byte planes in registers.  A launch over two projections whose code
+        # books are different tensors (equal values) stays on the flavour that gathers the code values from the lanes and
+        # multiplies: the same products, so the same output bit for bit.
+        proj = {"w": w, "U": U, "B": B16.cuda(), "bias": bias.cuda(), "r": r, "s": s}
+        code_twin = keep[2].clone()  # (kept alive: the struct holds its address)
+        w_twin = fmsa_hip.make_codebook_weight(keep[0], code_twin, keep[1], blocksize)
+        y_a, y_b = fmsa_hip.gptq_lora_fwd(xd, [proj, dict(proj, w=w_twin)])
+        assert torch.equal(y, y_a) and torch.equal(y, y_b)
     dy = randn((M, N), 8, dtype)
     dyd = dy.cuda()
     T = fmsa_hip.lora_down(dyd, B16.t().contiguous().cuda())
