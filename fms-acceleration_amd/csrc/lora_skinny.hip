@@ -461,11 +461,12 @@ __global__ __launch_bounds__(256) void lora_down_reduce_kernel(const float* __re
 // column walk.  Tiles of 32 tokens are staged through LDS (coalesced 16-byte global loads in, transposing
 // 8-byte reads out: column_frag below); token e of a tile is the MFMA's contraction index e, rows are padded
 // by 32 B.
-// Pass 1: workgroup = 128 columns of R x one fixed range of tokens (split); wave w owns columns
+// Pass 1: workgroup = 128 (four waves) or 256 (eight waves: what the launcher uses) columns of R x one fixed range of
+// tokens (split); wave w owns columns
 // 32w .. 32w+31 (two 16-wide MFMA tiles) and all r ranks.  Partial sums go to partial[split][r][C]
 // (fp32).  Pass 2 adds the splits in index order, so the result does not depend on scheduling.
 constexpr int LG_TM = 32;               // tokens per tile
-constexpr int LG_TC = 128;     // columns of R per workgroup (4 waves x 32)
+constexpr int LG_TC = 128;     // columns of R per workgroup of the 4-wave flavour; also the unit the number of splits is derived from
 constexpr int LG_TC_T = 256;   // ... of the flavour that also produces T (8 waves): half as many partial T's
 
 // Several gradients over the same M tokens go out as ONE launch of each pass (the dA of stacked
