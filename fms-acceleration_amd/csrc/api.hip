@@ -241,7 +241,7 @@ int fmsa_lora_grad_static(const void* L, int64_t ldl, const void* R, int64_t ldr
 
 int fmsa_probe_mfma(int mode, int iters, int n_workgroups, void* out, const void* src, void* stream) {
   if (!out || (mode >= 2 && !src)) return FMSA_ERR_NULL;
-  if (mode < 0 || mode > 3 || iters <= 0 || n_workgroups <= 0 || n_workgroups > 65536) return FMSA_ERR_SHAPE;
+  if (mode < 0 || mode > 3 || iters <= 0 || (iters & 1) || n_workgroups <= 0 || n_workgroups > 65536) return FMSA_ERR_SHAPE;
   return launch_probe_mfma(mode, iters, n_workgroups, (float*)out, src, (hipStream_t)stream);
 }
 

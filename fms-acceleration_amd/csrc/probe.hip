@@ -45,29 +45,34 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float* out, const uint3
       a[f][j] = ha;
       b[f][j] = hb;
     }
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: the loads' LDS address and scalar offset derive from it
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(src, 1u << 20);
-  u32x4 an[8];  // MODE 3: the fragments of the next iteration
+  u32x4 a2[8];  // MODE 3: the second of two fragment sets; the MFMAs of one iteration run on one set while the reads fill the other
   if (MODE == 3) {
     for (int i = lane; i < 2048; i += 64) lds_f[wave * 2048 + i] = (probe_hash(blockIdx.x * 8192 + wave * 2048 + i) & 0x807f807fu) | 0x3f803f80u;
     __syncthreads();
+#pragma unroll
+    for (int f = 0; f < 8; ++f) a2[f] = a[f];
   }
-  for (int it = 0; it < iters; ++it) {
+  // one iteration: 16 MFMAs on fragment set `cur`; every second MFMA is followed by a fragment read into set `nxt` (MODE 3),
+  // MFMAs 0 and 8 by a direct load (MODE >= 2)
+  auto iteration = [&](int it, u32x4(&cur)[8], u32x4(&nxt)[8]) {
     if (MODE == 3 && (it & 3) == 0) __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      acc[i] = mfma32<bf16_t>(a[i & 7], b[(i >> 1) & 7], acc[i]);
+      acc[i] = mfma32<bf16_t>(cur[i & 7], b[(i >> 1) & 7], acc[i]);
       if (MODE == 3 && (i & 1) == 0)
-        an[i >> 1] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(lds_f) + ((((it + 1) & 3) * 8 + (i >> 1)) * 1024 + lane * 16));
+        nxt[i >> 1] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(lds_f) + ((((it + 1) & 3) * 8 + (i >> 1)) * 1024 + lane * 16));
       if (MODE >= 2 && (i & 7) == 0)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(reinterpret_cast<char*>(lds) + (2 * wave + (i >> 3)) * 1024),
                                                  16, lane * 16, (uint32_t)((it & 63) * 16384 + (2 * wave + (i >> 3)) * 1024), 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (MODE == 3) {
-#pragma unroll
-      for (int f = 0; f < 8; ++f) a[f] = an[f];
-    }
+  };
+  for (int it = 0; it < iters; it += 2) {  // (iters is even)
+    iteration(it, a, a2);
+    iteration(it + 1, a2, a);
   }
   if (MODE >= 2) __builtin_amdgcn_s_waitcnt(0x0F70);
   float s = 0.f;

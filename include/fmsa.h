@@ -371,7 +371,7 @@ int fmsa_cross_entropy_fused(void* logits, int64_t ld, const int64_t* labels, in
 
 /* ------------------------------------------------------------------------------------------
  * Measurement support (no counterpart in the reference; used by bench.py --yardsticks).
- * A register-only loop of `iters` x 16 MFMA 32x32x16 bf16 per wave, 4 waves per workgroup:
+ * A register-only loop of `iters` (even) x 16 MFMA 32x32x16 bf16 per wave, 4 waves per workgroup:
  *   mode 0  all-zero operands (what the clock allows),
  *   mode 1  random bf16 operands (what the power limit leaves),
  *   mode 2  as 1, plus one 1 KB direct-to-LDS load per wave and 8 MFMAs from `src` (>= 1 MiB), the
