@@ -69,6 +69,17 @@ def test_codebook_weight_validation():
     assert p(ctypes.byref(nf4()), 0x5004, 0x6000, None) == -3
 
 
+def test_probe_validation():
+    """The measurement entry point checks its arguments before any HIP call too."""
+    f = fmsa_hip.lib().fmsa_probe_mfma
+    assert f(0, 100, 16, None, None, None) == -1
+    assert f(2, 100, 16, 0x1000, None, None) == -1      # modes with direct loads need a source
+    assert f(4, 100, 16, 0x1000, 0x2000, None) == -2
+    assert f(1, 0, 16, 0x1000, None, None) == -2
+    assert f(1, 101, 16, 0x1000, None, None) == -2      # two fragment sets used in turn: an even number of iterations
+    assert f(1, 100, 0, 0x1000, None, None) == -2
+
+
 def test_dequant_validation():
     lib = fmsa_hip.lib()
     f = lib.fmsa_gptq_dequant
