@@ -81,7 +81,7 @@ def _check(apply_rope, apply_plain, attn, refs, Ns, Bz, S, K, hd, dtype, cos, si
 @pytest.mark.parametrize("dtype,cdt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
                                        (torch.bfloat16, torch.float32)])
 @pytest.mark.parametrize("act_order", [False, True, "shared"])
-@pytest.mark.parametrize("Bz,S,hd", [(2, 96, 128), (1, 50, 64), (3, 37, 32)])
+@pytest.mark.parametrize("Bz,S,hd", [(2, 96, 128), (1, 50, 64), (3, 37, 32), (2, 40, 256), (1, 33, 16)])
 def test_gptq_qkv_rope(Bz, S, hd, dtype, cdt, act_order):
     from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_qkv, apply_lora_qkv_rope
 
