@@ -63,42 +63,21 @@ class AutoGPTQAccelerationPlugin(AccelerationPlugin):
         """Installs the adapters of `peft_config` (a peft LoraConfig, or any object / dict with `r`,
         `lora_alpha`, `lora_dropout`, `target_modules`) on the matching QuantLinear modules, freezes
         everything else and returns `(None,)` in place of the config, so that the trainer does not
-        wrap the model again (reference :269-330)."""
-        import torch  # pylint: disable=import-outside-toplevel
-
-        from .lora import LoraLinear  # pylint: disable=import-outside-toplevel
+        wrap the model again (reference :269-330).  `target_modules` follows peft: a list matches by name
+        or dotted suffix, a string is a regular expression ("all-linear" aside), None takes the default of
+        the model type."""
+        from .lora import install_lora_adapters  # pylint: disable=import-outside-toplevel
         from .qlinear import QuantLinear  # pylint: disable=import-outside-toplevel
 
         (peft_config,) = modifiable_args
         assert peft_config is not None, "need peft_config to install PEFT adapters"
-        get = (lambda k, d=None: peft_config.get(k, d)) if isinstance(peft_config, dict) else (lambda k, d=None: getattr(peft_config, k, d))
-        r, alpha, dropout = get("r"), get("lora_alpha"), float(get("lora_dropout", 0.0) or 0.0)
-        targets = get("target_modules")
-        if not r or alpha is None:
-            raise ValueError("peft_config needs `r` and `lora_alpha` to install LoRA adapters")
-        if isinstance(targets, str):
-            targets = None if targets == "all-linear" else [targets]
-        targets = None if targets is None else set(targets)
+        installed = install_lora_adapters(model, peft_config, QuantLinear)  # raises before anything is modified
         # the marker FastKernelsAccelerationPlugin.augmentation looks for (:235-236 of the reference)
         setattr(model, "quantization_method", "gptq")
         setattr(model, "is_loaded_in_4bit", True)
-        for p in model.parameters():
-            p.requires_grad_(False)
-        installed = []
-        for parent_name, parent in list(model.named_modules()):
-            for child_name, child in list(parent.named_children()):
-                if isinstance(child, QuantLinear) and (targets is None or child_name in targets):
-                    wrapped = LoraLinear(child, int(r), float(alpha), dropout)
-                    wrapped.to(child.qweight.device)
-                    setattr(parent, child_name, wrapped)
-                    installed.append(f"{parent_name}.{child_name}" if parent_name else child_name)
-        if not installed:
-            raise ValueError(f"no QuantLinear module matches target_modules={sorted(targets) if targets else 'all-linear'}: "
-                             "nothing to train (was the model loaded through this plugin's model_loader?)")
         if getattr(train_args, "gradient_checkpointing", False) and hasattr(model, "enable_input_require_grads"):
             model.enable_input_require_grads()  # what prepare_model_for_kbit_training does for checkpointed models
         model._fmsa_lora_modules = installed
-        del torch
         return model, (None,)
 
 

@@ -65,3 +65,71 @@ class LoraLinear(nn.Module):
             xd = self.lora_dropout[name](x).to(A.weight.dtype)
             result = result + (B(A(xd)) * self.scaling[name]).to(result.dtype)
         return result
+
+
+# peft's per-architecture defaults for `target_modules=None` (peft.utils.constants:
+# TRANSFORMERS_MODELS_TO_LORA_TARGET_MODULES_MAPPING) for the architectures the fused-LoRA rules cover
+DEFAULT_TARGET_MODULES = {
+    "llama": ["q_proj", "v_proj"],
+    "mistral": ["q_proj", "v_proj"],
+    "mixtral": ["q_proj", "v_proj"],
+    "granite": ["q_proj", "v_proj"],
+    "granitemoe": ["q_proj", "v_proj"],
+    "granitemoeshared": ["q_proj", "v_proj"],
+    "granitemoehybrid": ["q_proj", "v_proj"],
+}
+
+
+def _config_get(peft_config, key, default=None):
+    return peft_config.get(key, default) if isinstance(peft_config, dict) else getattr(peft_config, key, default)
+
+
+def _target_matcher(model, targets):
+    """peft's matching of `target_modules` against a module's dotted name (peft.tuners.tuners_utils:
+    check_target_module_exists): a string is a regular expression that must match the whole name (except
+    "all-linear": every base layer but the output embedding), a list matches a name that equals an entry or
+    ends with "." + entry; None falls back to the default of the model type."""
+    import re  # pylint: disable=import-outside-toplevel
+
+    if targets is None:
+        model_type = getattr(getattr(model, "config", None), "model_type", None)
+        if model_type not in DEFAULT_TARGET_MODULES:
+            raise ValueError(f"peft_config has no target_modules and the model type {model_type!r} has no default: name them")
+        targets = DEFAULT_TARGET_MODULES[model_type]
+    if isinstance(targets, str):
+        if targets == "all-linear":
+            out = getattr(model, "get_output_embeddings", lambda: None)()
+            return (lambda name, mod: mod is not out), "all-linear"
+        pattern = re.compile(targets)
+        return (lambda name, mod: pattern.fullmatch(name) is not None), targets
+    targets = list(targets)
+    return (lambda name, mod: any(name == t or name.endswith("." + t) for t in targets)), sorted(targets)
+
+
+def install_lora_adapters(model, peft_config, base_classes, adapter_name="default"):
+    """Wraps every module of `model` that is an instance of `base_classes` and is named by
+    `peft_config.target_modules` in a LoraLinear (what peft's get_peft_model does with its own LoRA layer),
+    then freezes every other parameter.  The matching runs first: a configuration that matches nothing raises
+    and leaves the model untouched.  Returns the dotted names of the wrapped modules."""
+    r, alpha = _config_get(peft_config, "r"), _config_get(peft_config, "lora_alpha")
+    dropout = float(_config_get(peft_config, "lora_dropout", 0.0) or 0.0)
+    if not r or alpha is None:
+        raise ValueError("peft_config needs `r` and `lora_alpha` to install LoRA adapters")
+    match, shown = _target_matcher(model, _config_get(peft_config, "target_modules"))
+    found = []
+    for parent_name, parent in model.named_modules():
+        for child_name, child in parent.named_children():
+            full = f"{parent_name}.{child_name}" if parent_name else child_name
+            if isinstance(child, base_classes) and match(full, child):
+                found.append((parent, child_name, child, full))
+    if not found:
+        names = ", ".join(c.__name__ for c in (base_classes if isinstance(base_classes, tuple) else (base_classes,)))
+        raise ValueError(f"no {names} module matches target_modules={shown}: nothing to train "
+                         "(was the model loaded through this plugin's model_loader?)")
+    for p in model.parameters():
+        p.requires_grad_(False)
+    for parent, child_name, child, _ in found:
+        wrapped = LoraLinear(child, int(r), float(alpha), dropout, adapter_name=adapter_name)
+        device = next((t.device for t in list(child.parameters()) + list(child.buffers())), None)
+        setattr(parent, child_name, wrapped.to(device) if device is not None else wrapped)
+    return [full for *_, full in found]

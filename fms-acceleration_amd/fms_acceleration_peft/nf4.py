@@ -7,9 +7,10 @@ quantised), `shape`, `dtype`, `blocksize`, `code`, `offset` and `state2` (`absma
 `blocksize`).  bitsandbytes is not installed where this is built; a real Linear4bit exposes the same
 attributes and is accepted by the fused operators as is.
 
-`quantize_nf4` builds such a weight from a dense matrix (blockwise absmax, nearest of the 16 NF4
-codes, even element in the high nibble; absmax minus its mean re-quantised to 8 bits in blocks of
-256) -- how synthetic NF4 checkpoints are made for tests and benchmarks.
+`quantize_4bit` builds such a weight from a dense matrix (blockwise absmax, nearest of the 16 codes
+of the NF4 or FP4 book, even element in the high nibble; absmax minus its mean re-quantised to 8
+bits in blocks of 256) -- how synthetic 4-bit checkpoints are made for tests and benchmarks, and how
+the plugin's loader quantises a dense checkpoint.
 """
 from __future__ import annotations
 
@@ -20,6 +21,13 @@ NF4_CODE = [-1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453
             -0.18477343022823334, -0.09105003625154495, 0.0, 0.07958029955625534, 0.16093020141124725,
             0.24611230194568634, 0.33791524171829224, 0.44070982933044434, 0.5626170039176941,
             0.7229568362236023, 1.0]
+
+
+# bitsandbytes' FP4 book (functional.get_4bit_type("fp4")): sign bit, then E2M1-like magnitudes in the library's own
+# code order, divided by the largest (12).  Not sorted: index i is what the packed nibble holds.
+FP4_CODE = [v / 12.0 for v in (0.0, 0.0625, 8.0, 12.0, 4.0, 6.0, 2.0, 3.0, -0.0, -0.0625, -8.0, -12.0, -4.0, -6.0, -2.0, -3.0)]
+
+CODE_BOOKS = {"nf4": NF4_CODE, "fp4": FP4_CODE}
 
 
 def dynamic_map_8bit() -> torch.Tensor:
@@ -56,16 +64,19 @@ class QuantState:
 
 
 def _nearest(codebook: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
-    mid = (codebook[:-1].double() + codebook[1:].double()) / 2
-    return torch.bucketize(x.double(), mid, right=False)
+    """Index of the nearest entry; the book need not be sorted (ties go to the smaller value)."""
+    order = torch.argsort(codebook, stable=True)
+    srt = codebook[order]
+    mid = (srt[:-1].double() + srt[1:].double()) / 2
+    return order[torch.bucketize(x.double(), mid, right=False)]
 
 
 @torch.no_grad()
-def quantize_nf4(W: torch.Tensor, blocksize: int = 64, blocksize2: int = 256, dtype=torch.bfloat16):
+def quantize_4bit(W: torch.Tensor, blocksize: int = 64, blocksize2: int = 256, dtype=torch.bfloat16, quant_type: str = "nf4"):
     """W [N, K] -> (packed uint8 [N*K/2, 1], QuantState)."""
     W = W.float()
     dev = W.device
-    code = torch.tensor(NF4_CODE, dtype=torch.float32, device=dev)
+    code = torch.tensor(CODE_BOOKS[quant_type], dtype=torch.float32, device=dev)
     blocks = W.reshape(-1, blocksize)
     absmax = blocks.abs().amax(dim=1)
     safe = torch.where(absmax == 0, torch.ones_like(absmax), absmax)
@@ -79,8 +90,13 @@ def quantize_nf4(W: torch.Tensor, blocksize: int = 64, blocksize2: int = 256, dt
     safe2 = torch.where(absmax2 == 0, torch.ones_like(absmax2), absmax2)
     code2 = dynamic_map_8bit().to(dev)
     absmax_q = _nearest(code2, ab / safe2[:, None]).reshape(-1)[: a.numel()].to(torch.uint8)
-    state = QuantState(absmax_q, W.shape, dtype, blocksize, code, offset.reshape(()), QuantState2(absmax2, code2, blocksize2))
+    state = QuantState(absmax_q, W.shape, dtype, blocksize, code, offset.reshape(()), QuantState2(absmax2, code2, blocksize2),
+                       quant_type=quant_type)
     return packed, state
+
+
+def quantize_nf4(W, blocksize=64, blocksize2=256, dtype=torch.bfloat16):
+    return quantize_4bit(W, blocksize, blocksize2, dtype, "nf4")
 
 
 class Params4bit(nn.Parameter):
@@ -92,8 +108,37 @@ class Params4bit(nn.Parameter):
         return self
 
 
+class Linear4bitFunction(torch.autograd.Function):
+    """y = x @ deq(W)^T, dx = dy @ deq(W) for a frozen 4-bit weight (what bitsandbytes' MatMul4Bit computes:
+    dequantise, then a dense matmul; no gradient for the weight).  16-bit activations go through the fused
+    dequant-GEMM kernels with the adapter switched off (r = 0): the codes are looked up on their way into the MFMA
+    and no dense matrix is written."""
+
+    @staticmethod
+    def forward(ctx, x, weight, quant_state):
+        import fmsa_hip
+        from fmsa_hip.nf4_prepared import prepare
+
+        w = prepare(weight, quant_state)
+        ctx.w = w
+        x2 = x if x.is_contiguous() else x.contiguous()
+        (y,) = fmsa_hip.gptq_lora_fwd(x2, [{"w": w.struct, "U": None, "B": None, "bias": None, "r": 0, "s": 0.0}])
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        import fmsa_hip
+
+        w = ctx.w
+        dy2 = dy if dy.is_contiguous() else dy.contiguous()
+        dx = fmsa_hip.gptq_lora_bwd_dx(
+            [{"w": w.struct, "nsz": w.nsz, "dY": dy2, "T": None, "At": None, "mask_src": None, "r": 0, "s": 0.0}], dy2.shape[0], w.K)
+        return dx, None, None
+
+
 class Linear4bit(nn.Module):
-    """NF4 linear.  `forward` is the unfused path: dequantise (HIP kernel) then matmul."""
+    """4-bit (NF4 / FP4 code book) linear.  `forward` is the module-level path without LoRA fusion: the fused
+    dequant-GEMM kernels with r = 0 for 16-bit activations, dequantise (HIP kernel) + matmul otherwise."""
 
     def __init__(self, in_features, out_features, bias=False, compute_dtype=torch.bfloat16):
         super().__init__()
@@ -102,10 +147,11 @@ class Linear4bit(nn.Module):
         self.bias = nn.Parameter(torch.zeros(out_features, dtype=compute_dtype), requires_grad=False) if bias else None
 
     @classmethod
-    def from_dense(cls, weight: torch.Tensor, bias=None, compute_dtype=torch.bfloat16, blocksize=64, blocksize2=256):
+    def from_dense(cls, weight: torch.Tensor, bias=None, compute_dtype=torch.bfloat16, blocksize=64, blocksize2=256,
+                   quant_type="nf4"):
         N, K = weight.shape
         self = cls(K, N, bias is not None, compute_dtype)
-        packed, state = quantize_nf4(weight, blocksize, blocksize2, compute_dtype)
+        packed, state = quantize_4bit(weight, blocksize, blocksize2, compute_dtype, quant_type)
         self.weight = Params4bit(packed, state)
         if bias is not None:
             self.bias.data.copy_(bias)
@@ -131,5 +177,13 @@ class Linear4bit(nn.Module):
                                     dtype or qs.dtype)
 
     def forward(self, x):
-        out = x @ self.dequantize(x.dtype).t()
+        qs = self.weight.quant_state
+        fused = (x.is_cuda and x.dtype in (torch.float16, torch.bfloat16) and qs is not None and qs.state2 is not None
+                 and self.in_features % qs.blocksize == 0 and qs.blocksize % 32 == 0
+                 and self.in_features % 32 == 0 and self.out_features % 32 == 0)
+        if fused:
+            out = Linear4bitFunction.apply(x.reshape(-1, x.shape[-1]), self.weight, qs)
+            out = out.reshape(x.shape[:-1] + (self.out_features,))
+        else:
+            out = x @ self.dequantize(x.dtype).t()
         return out + self.bias.to(out.dtype) if self.bias is not None else out

@@ -37,6 +37,126 @@ def test_linear4bit_container_and_parameter_scrape():
     assert get_lora_parameters(lin)[3:] == (None, None, None, None)
 
 
+def test_fp4_book_and_unsorted_nearest():
+    """The FP4 book is bitsandbytes' (sign bit, then 0, 1/192, 2/3, 1, 1/3, 1/2, 1/6, 1/4 in its code order): not sorted,
+    so the quantiser's nearest-entry search must not assume order; exact multiples of the block maximum are fixed points."""
+    from fms_acceleration_peft.nf4 import FP4_CODE, quantize_4bit
+
+    assert len(FP4_CODE) == 16 and FP4_CODE[3] == 1.0 and FP4_CODE[11] == -1.0 and FP4_CODE[0] == 0.0
+    assert [round(v * 12, 4) for v in FP4_CODE[:8]] == [0.0, 0.0625, 8.0, 12.0, 4.0, 6.0, 2.0, 3.0]
+    assert FP4_CODE[8:] == [-v for v in FP4_CODE[:8]]
+    gen = torch.Generator().manual_seed(0)
+    idx = torch.randint(1, 16, (4, 64), generator=gen)
+    idx[idx == 8] = 0  # -0 and +0 quantise alike
+    idx[:, 0] = 3       # the block maximum
+    W = torch.tensor(FP4_CODE)[idx] * 0.5
+    packed, st = quantize_4bit(W, quant_type="fp4")
+    codes = torch.stack([packed.reshape(-1) >> 4, packed.reshape(-1) & 0xF], dim=1).reshape(4, 64)
+    assert torch.equal(codes.long(), idx) and st.quant_type == "fp4"
+    assert torch.equal(st.code, torch.tensor(FP4_CODE))
+
+
+def _tiny_llama_dir(tmp_path):
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    cfg = LlamaConfig(hidden_size=64, intermediate_size=128, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=2, vocab_size=64)
+    cfg.architectures = ["LlamaForCausalLM"]
+    torch.manual_seed(0)
+    LlamaForCausalLM(cfg).save_pretrained(str(tmp_path))
+    return cfg
+
+
+def test_bnb_plugin_loader_augmentation_and_fused_rules(tmp_path, monkeypatch):
+    """configs/accelerated-peft-bnb-nf4-foak.yaml -> framework -> model_loader (local dense checkpoint quantised on
+    load) -> BNB augmentation (adapters from a duck-typed peft_config, `(None,)` handed back; reference
+    framework_plugin_bnb.py:192-218) -> fast-kernels augmentation -> ModelPatcher: qkvo and mlp rules fire."""
+    import os
+
+    import pytest
+    import yaml
+
+    import fms_acceleration  # noqa: F401
+    from fms_acceleration.framework import AccelerationFramework
+    from fms_acceleration.model_patcher import ModelPatcher, patch_model
+    from fms_acceleration.utils.test_utils import instantiate_model_patcher
+    from fms_acceleration_foak.fused_ops.unsloth_lora.bnb.fast_lora import apply_lora_mlp_swiglu
+    from fms_acceleration_peft import BNBAccelerationPlugin, Linear4bit, LoraLinear
+
+    _tiny_llama_dir(tmp_path)
+    here = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(here, "fms-acceleration_amd", "configs", "accelerated-peft-bnb-nf4-foak.yaml")) as f:
+        config = yaml.safe_load(f)
+    for quant_type in ("nf4", "fp4"):
+        config["plugins"]["peft"]["quantization"]["bitsandbytes"]["quant_type"] = quant_type
+        # only the fused-LoRA rules: the kernel rules replace functions of transformers' modules for the whole process
+        config["plugins"]["peft"]["quantization"]["fused_ops_and_kernels"].update(
+            fast_loss=False, fast_rms_layernorm=False, fast_rope_embeddings=False)
+        cfg_file = tmp_path / f"{quant_type}.yaml"
+        cfg_file.write_text(yaml.safe_dump(config))
+        monkeypatch.setattr(AccelerationFramework, "active_plugins", [])  # class-level state, as in the reference
+        monkeypatch.setattr(AccelerationFramework, "plugins_require_custom_loading", [])
+        fw = AccelerationFramework(str(cfg_file))
+        assert [type(p).__name__ for _, p in fw.active_plugins] == ["BNBAccelerationPlugin", "FastKernelsAccelerationPlugin"]
+        model = fw.model_loader(str(tmp_path), torch_dtype=torch.bfloat16, device="cpu")
+        quantised = [m for m in model.modules() if isinstance(m, Linear4bit)]
+        assert len(quantised) == 14 and isinstance(model.lm_head, torch.nn.Linear)
+        assert all(m.weight.quant_state.quant_type == quant_type and m.weight.quant_state.nested for m in quantised)
+        train_args = type("T", (), {"bf16": True, "fp16": False, "gradient_checkpointing": False})()
+        peft_config = {"r": 8, "lora_alpha": 16, "lora_dropout": 0.0, "target_modules": "all-linear"}
+        with instantiate_model_patcher():
+            out, args = fw.augmentation(model, train_args, (peft_config,))
+            assert out is model and args == (None,)
+            wrapped = [m for m in model.modules() if isinstance(m, LoraLinear)]
+            assert len(wrapped) == 14 and all(isinstance(m.base_layer, Linear4bit) for m in wrapped)
+            trainable = [n for n, p in model.named_parameters() if p.requires_grad]
+            assert len(trainable) == 28 and all("lora_" in n for n in trainable)
+            patch_model(model)
+            done = sorted(h.rule_id for h in ModelPatcher.history)
+            assert done.count("llama-mlp") == 2   # one per decoder layer
+            assert [d for d in done if d.startswith("llama-qkvo")] == sorted(["llama-qkvo-1", "llama-qkvo-2", "llama-qkvo-3", "llama-qkvo-4"] * 2)
+            assert model.model.layers[0].mlp.forward.__func__ is apply_lora_mlp_swiglu
+
+    plugin = BNBAccelerationPlugin({"peft": {"quantization": {"bitsandbytes": {"quant_type": "nf4", "no_peft_model": False}}}})
+    with pytest.raises(NotImplementedError):
+        plugin.model_loader("mistralai/Mistral-7B-v0.1")
+
+
+def test_adapter_installer_follows_peft_matching(tmp_path):
+    """target_modules: list entries match by name or dotted suffix, a string is a regular expression, None takes the
+    model type's default (q_proj, v_proj for llama); a configuration that matches nothing raises and leaves the model as it was."""
+    import pytest
+    from transformers import LlamaForCausalLM
+
+    from fms_acceleration_peft import BNBAccelerationPlugin, Linear4bit, LoraLinear
+
+    _tiny_llama_dir(tmp_path)
+    plugin = BNBAccelerationPlugin({"peft": {"quantization": {"bitsandbytes": {"quant_type": "nf4", "no_peft_model": False}}}})
+    train_args = type("T", (), {"bf16": True, "fp16": False})()
+
+    def names(model):
+        return sorted(n for n, m in model.named_modules() if isinstance(m, LoraLinear))
+
+    def fresh():
+        return plugin.model_loader(str(tmp_path), torch_dtype=torch.bfloat16, device="cpu")
+
+    model = fresh()
+    with pytest.raises(ValueError, match="no Linear4bit module matches"):
+        plugin.augmentation(model, train_args, ({"r": 8, "lora_alpha": 16, "target_modules": ["nothing"]},))
+    assert not names(model) and any(p.requires_grad for p in model.parameters())  # untouched
+    with pytest.raises(AssertionError, match="mixed precision"):
+        plugin.augmentation(model, type("T", (), {"bf16": False, "fp16": False})(), ({"r": 8, "lora_alpha": 16},))
+    plugin.augmentation(model, train_args, ({"r": 8, "lora_alpha": 16, "target_modules": None},))
+    assert names(model) == sorted(f"model.layers.{i}.self_attn.{p}" for i in (0, 1) for p in ("q_proj", "v_proj"))
+    model = fresh()
+    plugin.augmentation(model, train_args, ({"r": 8, "lora_alpha": 16, "target_modules": ["layers.1.mlp.up_proj", "o_proj"]},))
+    assert names(model) == ["model.layers.0.self_attn.o_proj", "model.layers.1.mlp.up_proj", "model.layers.1.self_attn.o_proj"]
+    model = fresh()
+    plugin.augmentation(model, train_args, ({"r": 8, "lora_alpha": 16, "target_modules": r".*\.layers\.0\..*(gate|down)_proj"},))
+    assert names(model) == ["model.layers.0.mlp.down_proj", "model.layers.0.mlp.gate_proj"]
+    assert isinstance(model, LlamaForCausalLM) and model.quantization_method == "bitsandbytes"
+
+
 def test_bnb_plugin_shell_and_fused_ops_registry():
     import fms_acceleration  # noqa: F401  (registers the plugins)
     from fms_acceleration_foak.models.utils import FUSED_OPS, KEY_MLP, KEY_O, KEY_QKV
@@ -50,6 +170,14 @@ def test_bnb_plugin_shell_and_fused_ops_registry():
     class Args:
         bf16, fp16 = True, False
 
-    model = torch.nn.Linear(2, 2)
-    plugin.augmentation(model, Args(), (None,))
-    assert model.quantization_method == "bitsandbytes"
+    no_peft = BNBAccelerationPlugin({"peft": {"quantization": {"bitsandbytes": {"quant_type": "fp4", "no_peft_model": True}}}})
+    assert no_peft.requires_custom_loading and not no_peft.requires_augmentation
+    model = torch.nn.Sequential(Linear4bit_from(torch.randn(32, 64)))
+    out, args = plugin.augmentation(model, Args(), ({"r": 8, "lora_alpha": 8, "target_modules": ["0"]},))
+    assert out is model and args == (None,) and model.quantization_method == "bitsandbytes"
+
+
+def Linear4bit_from(W):
+    from fms_acceleration_peft import Linear4bit
+
+    return Linear4bit.from_dense(W * 0.02)

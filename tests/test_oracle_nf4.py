@@ -1,6 +1,8 @@
-"""NF4 oracle: closed forms and round trips (its parity with bitsandbytes itself is unpinned: the
-library is not available and the reference holds no NF4 vectors)."""
+"""NF4 oracle: the code book re-derived from its published construction (normal quantiles), closed
+forms and round trips.  Its parity with the bitsandbytes library itself stays unpinned: the library
+is not available and the reference holds no NF4 vectors."""
 import numpy as np
+import torch
 
 from oracle import nf4
 
@@ -48,3 +50,40 @@ def test_exact_codes_are_fixed_points():
     W = (nf4.NF4[idx] * np.float32(0.5)).astype(np.float32)
     q = nf4.quantize(W)
     assert np.array_equal(nf4.dequant(q, "fp32").numpy(), W)
+
+
+def test_nf4_table_is_the_normal_quantile_construction():
+    """The 16 NF4 values are not free constants: they are quantiles of N(0, 1) at evenly spaced probabilities
+    (8 on the positive side from 0.9677083 down to 0.5 exclusive, 7 on the negative side), an exact 0, sorted
+    and divided by the largest (QLoRA, appendix E; bitsandbytes `create_normal_map(offset=0.9677083)`).  A typo
+    in any entry of the oracle's table (and of the product's, which must equal it) fails this."""
+    from scipy.stats import norm
+
+    offset = 0.9677083
+    pos = norm.ppf(torch.linspace(offset, 0.5, 9)[:-1].numpy())
+    neg = -norm.ppf(torch.linspace(offset, 0.5, 8)[:-1].numpy())
+    table = torch.tensor(np.concatenate([pos, [0.0], neg])).sort().values
+    table = (table / table.max()).to(torch.float32).numpy()
+    assert table.shape == (16,)
+    assert np.array_equal(table, nf4.NF4), np.abs(table - nf4.NF4).max()
+    # asymmetric on purpose: 7 negative and 8 positive levels around an exact zero
+    assert (nf4.NF4 < 0).sum() == 7 and (nf4.NF4 > 0).sum() == 8
+    from fms_acceleration_peft.nf4 import NF4_CODE
+
+    assert np.array_equal(np.asarray(NF4_CODE, np.float32), nf4.NF4)
+
+
+def test_dynamic_map_known_entries():
+    """Entries of the signed 8-bit dynamic map that follow from its construction (7 exponent levels, level i holds
+    the 2**i midpoints of linspace(0.1, 1, 2**i + 1) scaled by 10**(i - 6), both signs, then 0 and 1)."""
+    m = nf4.dynamic_map_8bit()
+    assert np.unique(m).size == 256                     # 2 * (1 + 2 + ... + 64) + 2 distinct values
+    assert m[0] == np.float32(-(1.0 - 0.9 / 128))       # last midpoint of level 6: -(1 - 0.9 / 64 / 2)
+    assert m[m > 0][0] == np.float32(0.55e-6)           # level 0: the one midpoint of [0.1, 1] times 1e-6
+    assert m[m > 0][1] == np.float32(0.325e-5) and m[m > 0][2] == np.float32(0.775e-5)  # level 1
+    assert m[-2] == np.float32(1.0 - 0.9 / 128) and m[-1] == 1.0
+    assert (m < 0).sum() == 127 and (m > 0).sum() == 128
+    assert np.array_equal(np.sort(-m[m < 0]), m[(m > 0) & (m < 1)])  # symmetric apart from the extra 1.0
+    from fms_acceleration_peft.nf4 import dynamic_map_8bit
+
+    assert np.array_equal(dynamic_map_8bit().numpy(), m)
