@@ -535,6 +535,23 @@ def yardsticks(device):
         torch.cuda.synchronize()
         return s.elapsed_time(e) / n * 1e-3
 
+    # the MFMA-loop probe is a library of its own (fms-acceleration_amd/csrc/probe.hip -> lib/libfmsa_probe.so), not part of
+    # the product's C ABI
+    import ctypes
+
+    probe_path = os.path.join(os.path.dirname(os.path.abspath(fmsa_hip.__file__)), "..", "lib", "libfmsa_probe.so")
+    probe_lib = ctypes.CDLL(os.path.abspath(probe_path))
+    probe_lib.fmsa_probe_mfma.restype = ctypes.c_int
+    probe_lib.fmsa_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+
+    def probe_mfma(mode, iters, n_workgroups, dev):
+        out = torch.empty(n_workgroups * 256, dtype=torch.float32, device=dev)
+        # bf16 pairs in +-[1, 2), the kind of operand the loop keeps in registers (mode 3 feeds them to the MFMAs through LDS)
+        src = (torch.randint(0, 1 << 32, (1 << 18,), dtype=torch.int64, device=dev) & 0x807F807F | 0x3F803F80).to(torch.int32)
+        rc = probe_lib.fmsa_probe_mfma(mode, iters, n_workgroups, out.data_ptr(), src.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, f"fmsa_probe_mfma returned {rc}"
+        return float(n_workgroups) * 4 * iters * 16 * 32768.0
+
     gen = torch.Generator(device=device).manual_seed(0)
     x = torch.randn(M_TOKENS, HIDDEN, generator=gen, device=device).to(torch.bfloat16)
     w = (torch.randn(HIDDEN, 2 * INTER, generator=gen, device=device) * 0.02).to(torch.bfloat16)
@@ -548,7 +565,7 @@ def yardsticks(device):
         flop = [0.0]
 
         def run():
-            flop[0] = fmsa_hip.probe_mfma(mode, 20000, 1024, device)
+            flop[0] = probe_mfma(mode, 20000, 1024, device)
 
         t = ev_time(run, 5, 2)  # 5 x about 40 ms: long enough for the clocks to settle under the power limit
         out[name] = {"ms": t * 1e3, "tflops": flop[0] / t / 1e12}

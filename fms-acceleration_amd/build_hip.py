@@ -4,7 +4,9 @@
 
 hipcc cross-compiles for gfx950 without a GPU.  Each translation unit is compiled to an object
 in parallel and the objects are linked into ``lib/libfmsa_hip.so`` next to this file; the
-Python side loads that file with ctypes and never builds at import time.
+Python side loads that file with ctypes and never builds at import time.  The measurement probe
+(``csrc/probe.hip``, what ``bench.py --yardsticks`` times) is not part of the product: it becomes a
+library of its own, ``lib/libfmsa_probe.so``.
 """
 from __future__ import annotations
 
@@ -20,7 +22,9 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfmsa_hip.so")
 
-SOURCES = ["api.hip", "dequant.hip", "gemm_fwd.hip", "gemm_bwd.hip", "lora_skinny.hip", "elementwise.hip", "nf4.hip", "norm_rope.hip", "probe.hip"]
+SOURCES = ["api.hip", "dequant.hip", "gemm_fwd.hip", "gemm_bwd.hip", "lora_skinny.hip", "elementwise.hip", "nf4.hip", "norm_rope.hip"]
+PROBE_SOURCE = "probe.hip"
+PROBE_LIB_PATH = os.path.join(LIB_DIR, "libfmsa_probe.so")
 
 # -packed-fp32-ops is switched off on purpose: the packed fp32 VALU forms are not trusted on the
 # target machines, so fp32 math is emitted as scalar-per-lane instructions.
@@ -64,14 +68,16 @@ def build(verbose: bool = False, extra_flags=()) -> str:
             print(out)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
-        list(pool.map(compile_one, zip(SOURCES, objs)))
-    tmp = LIB_PATH + ".tmp"
-    # --no-undefined: a kernel whose host stub was not emitted must fail the link, not the first call
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--no-undefined", "-o", tmp, *objs])
-    os.replace(tmp, LIB_PATH)
-    if verbose:
-        print("built", LIB_PATH)
+    probe_obj = os.path.join(OBJ_DIR, PROBE_SOURCE.replace(".hip", ".o"))
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES) + 1)) as pool:
+        list(pool.map(compile_one, list(zip(SOURCES, objs)) + [(PROBE_SOURCE, probe_obj)]))
+    for path, members in ((LIB_PATH, objs), (PROBE_LIB_PATH, [probe_obj])):
+        tmp = path + ".tmp"
+        # --no-undefined: a kernel whose host stub was not emitted must fail the link, not the first call
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--no-undefined", "-o", tmp, *members])
+        os.replace(tmp, path)
+        if verbose:
+            print("built", path)
     return LIB_PATH
 
 

@@ -41,7 +41,6 @@ int launch_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64
 int launch_swiglu_bwd(const void* dh, int64_t lddh, void* e, void* g, void* h, int M, int I, int64_t ld, int act_dtype,
                       hipStream_t st);
 
-int launch_probe_mfma(int mode, int iters, int n_workgroups, float* out, const void* src, hipStream_t st);
 
 namespace {
 
@@ -114,11 +113,12 @@ const char* fmsa_strerror(int code) {
     case FMSA_ERR_UNSUPPORTED: return "configuration not covered by the gfx950 kernels";
     case FMSA_ERR_WORKSPACE: return "workspace missing or too small";
     case FMSA_ERR_LAUNCH: return "kernel launch failed";
+    case FMSA_ERR_DEVICE: return "tensors live on another GPU than the calling thread's current device";
     default: return "unknown error";
   }
 }
 
-int fmsa_abi_version(void) { return 7; }
+int fmsa_abi_version(void) { return 8; }
 
 int fmsa_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, void* stream) {
   if (!w || !out) return FMSA_ERR_NULL;
@@ -233,16 +233,21 @@ int fmsa_lora_grad_static(const void* L, int64_t ldl, const void* R, int64_t ldr
   if (C % 8 != 0 || ldr % 8 != 0 || ldl % 8 != 0 || r % 8 != 0 || r > 128) return FMSA_ERR_SHAPE;
   if (out_dtype != FMSA_F16 && out_dtype != FMSA_BF16 && out_dtype != FMSA_F32) return FMSA_ERR_DTYPE;
   if (!aligned16(R) || !aligned16(L)) return FMSA_ERR_ALIGN;
+  // the launch goes to the calling thread's current device, so that is whose copy of the buffer is used: the
+  // tensors (and the stream) must belong to it.  The query allocates nothing; a pointer the runtime does not
+  // know is left to the kernel's own addressing.
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return FMSA_ERR_LAUNCH;
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, out) == hipSuccess) {
+    if (attr.type == hipMemoryTypeDevice && attr.device != dev) return FMSA_ERR_DEVICE;
+  } else {
+    (void)hipGetLastError();
+  }
   void* ws = scratch_of_current_device();
   if (!ws) return FMSA_ERR_LAUNCH;
   // both passes write every partial sum they later read, so the buffer needs no clearing between calls
   return launch_lora_grad_batch(&job, 1, M, act_dtype, ws, (hipStream_t)stream);
-}
-
-int fmsa_probe_mfma(int mode, int iters, int n_workgroups, void* out, const void* src, void* stream) {
-  if (!out || (mode >= 2 && !src)) return FMSA_ERR_NULL;
-  if (mode < 0 || mode > 3 || iters <= 0 || (iters & 1) || n_workgroups <= 0 || n_workgroups > 65536) return FMSA_ERR_SHAPE;
-  return launch_probe_mfma(mode, iters, n_workgroups, (float*)out, src, (hipStream_t)stream);
 }
 
 static int check_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int64_t ldx, int M, int mode, const void* H,

@@ -461,13 +461,11 @@ __global__ __launch_bounds__(256) void lora_down_reduce_kernel(const float* __re
 // column walk.  Tiles of 32 tokens are staged through LDS (coalesced 16-byte global loads in, transposing
 // 8-byte reads out: column_frag below); token e of a tile is the MFMA's contraction index e, rows are padded
 // by 32 B.
-// Pass 1: workgroup = 128 (four waves) or 256 (eight waves: what the launcher uses) columns of R x one fixed range of
-// tokens (split); wave w owns columns
+// Pass 1: workgroup = 256 columns of R (eight waves) x one fixed range of tokens (split); wave w owns columns
 // 32w .. 32w+31 (two 16-wide MFMA tiles) and all r ranks.  Partial sums go to partial[split][r][C]
 // (fp32).  Pass 2 adds the splits in index order, so the result does not depend on scheduling.
 constexpr int LG_TM = 32;               // tokens per tile
-constexpr int LG_TC = 128;     // columns of R per workgroup of the 4-wave flavour; also the unit the number of splits is derived from
-constexpr int LG_TC_T = 256;   // ... of the flavour that also produces T (8 waves): half as many partial T's
+constexpr int LG_TC_T = 256;   // columns of R per workgroup (8 waves x 32)
 
 // Several gradients over the same M tokens go out as ONE launch of each pass (the dA of stacked
 // adapters and their dB's; a launch of a small gradient alone neither fills the chip nor hides its
@@ -511,11 +509,11 @@ FMSA_DEVI LoraGradJobDev select_job(const LoraGradArgs& a, int block) {
 // LDS and are summed in wave order by the whole workgroup one iteration later (behind the barrier the
 // loop has anyway), and leave as the column block's partial T[column block][token][rank] (fp32).  The
 // reduce pass adds the column blocks in index order and rounds once: deterministic like the rest.
-// WIDE: eight waves and 256 columns per workgroup without the T product: the L tile every workgroup re-reads is r / 128 of
-// the R bytes it consumes at 128 columns, half that at 256.
-template <typename T, int RT, bool WITH_T, bool WIDE = false>
-__global__ __launch_bounds__((WITH_T || WIDE) ? 512 : 256) void lora_grad_partial_kernel(const LoraGradArgs a) {
-  constexpr int NWV = (WITH_T || WIDE) ? 8 : 4;  // waves
+// Eight waves and 256 columns per workgroup: the L tile every workgroup re-reads is r / 256 of the R bytes it consumes
+// (a four-wave, 128-column workgroup measured slower at every rank: 44.6 vs 41.8 us over 235 MB at rank 16).
+template <typename T, int RT, bool WITH_T>
+__global__ __launch_bounds__(512) void lora_grad_partial_kernel(const LoraGradArgs a) {
+  constexpr int NWV = 8;  // waves
   constexpr int NTH = 64 * NWV;             // threads
   constexpr int TC = 32 * NWV;              // columns of R per workgroup
   constexpr int LG_RSTRIDE = TC + 16;       // elements: row + 32 B pad
@@ -744,10 +742,11 @@ __global__ __launch_bounds__(256) void lora_grad_reduce_kernel(const LoraGradArg
 }  // namespace
 
 int lora_grad_splits(int M, int C) {
-  const int ncb = (C + LG_TC - 1) / LG_TC;
-  // about four workgroups per CU, but at least 512 tokens (16 tiles) per split: shorter splits spend
-  // their time in the prologue and in writing / re-reading partial sums
-  int splits = 1024 / ncb;
+  const int ncb = (C + LG_TC_T - 1) / LG_TC_T;
+  // about two 512-thread workgroups per CU (16 waves), but at least 512 tokens (16 tiles) per split: shorter
+  // splits spend their time in the prologue and in writing / re-reading partial sums.  (The count equals what
+  // 1024 / number of 128-column blocks gave for widths that are multiples of 256; part of the workspace contract.)
+  int splits = 512 / ncb;
   const int max_splits = (M + 511) / 512;
   if (splits > max_splits) splits = max_splits;
   if (splits < 1) splits = 1;
@@ -921,10 +920,7 @@ int launch_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, in
   a.act_dtype = act_dtype;
   bool any_t = false;
   for (int q = 0; q < n_jobs; ++q) any_t = any_t || jobs[q].Wt != nullptr;
-  int r_all = 0;
-  for (int q = 0; q < n_jobs; ++q) r_all = jobs[q].r > r_all ? jobs[q].r : r_all;
-  const bool wide = true;  // measured better at every rank (235 MB, rank 16: 44.6 -> 41.8 us); the 128-column flavour is kept for reference
-  const int tc = wide ? LG_TC_T : LG_TC;  // the launch's flavour decides the column-block width of all its jobs
+  const int tc = LG_TC_T;
   int blocks = 0, rblocks = 0, r_max = 0;
   size_t ws_off = 0;
   for (int q = 0; q < n_jobs; ++q) {
@@ -959,15 +955,15 @@ int launch_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, in
     }
     r_max = s.r > r_max ? s.r : r_max;
   }
-  dim3 grid1(blocks), grid2(rblocks), block(256), block1(wide ? 512 : 256);
+  dim3 grid1(blocks), grid2(rblocks), block(256), block1(512);
   const int rt = (r_max + 15) / 16;
 #define LAUNCH(TT, RT, WT) hipLaunchKernelGGL((lora_grad_partial_kernel<TT, RT, WT>), grid1, block1, 0, st, a)
 #define DISPATCH(TT)                                                  \
   switch (rt) {                                                       \
-    case 1: if (any_t) LAUNCH(TT, 1, true); else hipLaunchKernelGGL((lora_grad_partial_kernel<TT, 1, false, true>), grid1, block1, 0, st, a); break; \
-    case 2: if (any_t) LAUNCH(TT, 2, true); else hipLaunchKernelGGL((lora_grad_partial_kernel<TT, 2, false, true>), grid1, block1, 0, st, a); break; \
-    case 3: case 4: hipLaunchKernelGGL((lora_grad_partial_kernel<TT, 4, false, true>), grid1, block1, 0, st, a); break; \
-    default: hipLaunchKernelGGL((lora_grad_partial_kernel<TT, 8, false, true>), grid1, block1, 0, st, a); break;         \
+    case 1: if (any_t) LAUNCH(TT, 1, true); else hipLaunchKernelGGL((lora_grad_partial_kernel<TT, 1, false>), grid1, block1, 0, st, a); break; \
+    case 2: if (any_t) LAUNCH(TT, 2, true); else hipLaunchKernelGGL((lora_grad_partial_kernel<TT, 2, false>), grid1, block1, 0, st, a); break; \
+    case 3: case 4: hipLaunchKernelGGL((lora_grad_partial_kernel<TT, 4, false>), grid1, block1, 0, st, a); break; \
+    default: hipLaunchKernelGGL((lora_grad_partial_kernel<TT, 8, false>), grid1, block1, 0, st, a); break;         \
   }
   if (act_dtype == FMSA_BF16) {
     DISPATCH(bf16_t)

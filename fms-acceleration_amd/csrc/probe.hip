@@ -85,12 +85,19 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float* out, const uint3
 
 }  // namespace
 
-int launch_probe_mfma(int mode, int iters, int n_workgroups, float* out, const void* src, hipStream_t st) {
+// The library's one entry point (bench.py --yardsticks binds it with ctypes).  iters even; `out`: n_workgroups * 256
+// floats; `src`: >= 1 MiB of bf16 operands for modes 2 and 3.  Returns 0, or a negative FMSA_ERR_* code for bad arguments
+// before any HIP call.  FLOP of a launch = n_workgroups * 4 * iters * 16 * 32768.
+extern "C" int fmsa_probe_mfma(int mode, int iters, int n_workgroups, void* out, const void* src, void* stream) {
+  if (!out || (mode >= 2 && !src)) return FMSA_ERR_NULL;
+  if (mode < 0 || mode > 3 || iters <= 0 || (iters & 1) || n_workgroups <= 0 || n_workgroups > 65536) return FMSA_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  float* o = (float*)out;
   dim3 grid(n_workgroups), block(256);
-  if (mode == 0) hipLaunchKernelGGL(probe_mfma_kernel<0>, grid, block, 0, st, out, (const uint32_t*)src, iters);
-  else if (mode == 1) hipLaunchKernelGGL(probe_mfma_kernel<1>, grid, block, 0, st, out, (const uint32_t*)src, iters);
-  else if (mode == 2) hipLaunchKernelGGL(probe_mfma_kernel<2>, grid, block, 0, st, out, (const uint32_t*)src, iters);
-  else hipLaunchKernelGGL(probe_mfma_kernel<3>, grid, block, 0, st, out, (const uint32_t*)src, iters);
+  if (mode == 0) hipLaunchKernelGGL(probe_mfma_kernel<0>, grid, block, 0, st, o, (const uint32_t*)src, iters);
+  else if (mode == 1) hipLaunchKernelGGL(probe_mfma_kernel<1>, grid, block, 0, st, o, (const uint32_t*)src, iters);
+  else if (mode == 2) hipLaunchKernelGGL(probe_mfma_kernel<2>, grid, block, 0, st, o, (const uint32_t*)src, iters);
+  else hipLaunchKernelGGL(probe_mfma_kernel<3>, grid, block, 0, st, o, (const uint32_t*)src, iters);
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }

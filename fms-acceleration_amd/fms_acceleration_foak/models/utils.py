@@ -58,7 +58,10 @@ def _build_fused_forwards(attn: torch.nn.Module, fused_operation: Callable, subm
     rope_operation (apply_lora_qkv_rope): a forward pre-hook of the attention keeps the `position_embeddings` it is
     called with; the fused call then returns Q and K already rotated and marks them, so that the attention's
     apply_rotary_pos_emb (fast_rope_embedding of the `<arch>-rope` rule) passes them through.  Without tables
-    (an attention called without `position_embeddings`) the plain fused operation runs."""
+    (an attention called without `position_embeddings`) the plain fused operation runs.  A forward hook that runs
+    whether or not the forward raised closes the protocol: a mark that is still there when the attention returns
+    means its rotation did not go through fast_rope_embedding (Q / K would leave rotated twice), which raises at
+    once; after an exception inside the forward the mark and the pending outputs are dropped, so a retry starts clean."""
     pending = {}
     tables = {}
 
@@ -68,18 +71,25 @@ def _build_fused_forwards(attn: torch.nn.Module, fused_operation: Callable, subm
         def _keep_tables(module, args, kwargs):
             tables["pe"] = kwargs.get("position_embeddings", args[1] if len(args) > 1 else None)
 
+        def _close_protocol(module, args, output):
+            key = tables.pop("marked", None)
+            tables.pop("pe", None)
+            unconsumed = key is not None and unmark_rotated(key)
+            if output is None:  # the forward raised: leave nothing behind for the next call
+                pending.clear()
+                return
+            if unconsumed:
+                raise RuntimeError("fused Q/K/V with rotary embedding: the attention returned without handing the rotated "
+                                   "Q / K to apply_rotary_pos_emb (fast_rope_embedding): its outputs are rotated twice; "
+                                   "enable fast_rope_embeddings for this model or switch the fused rotation off")
+
         attn.register_forward_pre_hook(_keep_tables, with_kwargs=True)
+        attn.register_forward_hook(_close_protocol, always_call=True)
 
     def _forward(self, X, name: str):
         if not any(n in pending for n in submodule_names):
             pe = tables.pop("pe", None)
             if rope_operation is not None and pe is not None and X.dim() == 3:
-                stale = tables.pop("marked", None)
-                if stale is not None and unmark_rotated(stale):
-                    # the Q / K of the previous call were never handed to apply_rotary_pos_emb: this attention does
-                    # not rotate what it is given position_embeddings for, and its outputs must not come rotated
-                    raise RuntimeError("fused Q/K/V with rotary embedding: the attention did not call apply_rotary_pos_emb "
-                                       "on the previous projections; use fast_rope_embeddings: true for this model")
                 outs = rope_operation(attn, X, pe[0], pe[1])
                 tables["marked"] = mark_rotated(outs[0], outs[1])
             else:

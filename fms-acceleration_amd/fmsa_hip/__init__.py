@@ -52,7 +52,6 @@ EXPORTED_SYMBOLS = (
     "fmsa_cross_entropy_fwd",
     "fmsa_cross_entropy_bwd",
     "fmsa_cross_entropy_fused",
-    "fmsa_probe_mfma",
 )
 
 
@@ -226,7 +225,6 @@ def lib() -> ctypes.CDLL:
                                       c_int, c_void_p]
     L.fmsa_cross_entropy_fwd.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.fmsa_cross_entropy_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]
-    L.fmsa_probe_mfma.argtypes = [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.fmsa_cross_entropy_fused.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int64, c_void_p, c_float, c_void_p, c_void_p]
     for name in EXPORTED_SYMBOLS:
         getattr(L, name)  # AttributeError here means the library is stale: rebuild it
@@ -380,9 +378,11 @@ def lora_grad_static(L, R, scale: float, transpose_out: bool, out):
     C = R.shape[1]
     assert R.shape[0] == M and L.stride(1) == 1 and R.stride(1) == 1 and L.dtype == R.dtype
     assert out.is_contiguous() and tuple(out.shape) == ((C, r) if transpose_out else (r, C))
-    _check("fmsa_lora_grad_static",
-           lib().fmsa_lora_grad_static(_ptr(L), L.stride(0), _ptr(R), R.stride(0), M, C, r, float(scale), int(transpose_out),
-                                       act_enum(R.dtype), _DTYPE_ENUM[out.dtype], _ptr(out), _stream(out)))
+    assert L.device == R.device == out.device
+    with torch.cuda.device(out.device):  # the library uses the buffer of the thread's current device
+        _check("fmsa_lora_grad_static",
+               lib().fmsa_lora_grad_static(_ptr(L), L.stride(0), _ptr(R), R.stride(0), M, C, r, float(scale), int(transpose_out),
+                                           act_enum(R.dtype), _DTYPE_ENUM[out.dtype], _ptr(out), _stream(out)))
     return out
 
 
@@ -646,12 +646,3 @@ def cross_entropy_fused_(logits2d, labels, scale=None, label_smoothing=0.0, igno
                                           int(ignore_index), _ptr(scale) if scale is not None else None, float(label_smoothing),
                                           _ptr(losses), _stream(logits2d)))
     return losses, logits2d
-
-
-def probe_mfma(mode: int, iters: int = 20000, n_workgroups: int = 1024, device="cuda"):
-    """Launches the register-only MFMA loop (see fmsa_probe_mfma in include/fmsa.h); returns its FLOP count."""
-    out = torch.empty(n_workgroups * 256, dtype=torch.float32, device=device)
-    # bf16 pairs in +-[1, 2), the kind of operand the loop keeps in registers (mode 3 feeds them to the MFMAs through LDS)
-    src = (torch.randint(0, 1 << 32, (1 << 18,), dtype=torch.int64, device=device) & 0x807F807F | 0x3F803F80).to(torch.int32)
-    _check("fmsa_probe_mfma", lib().fmsa_probe_mfma(mode, iters, n_workgroups, _ptr(out), _ptr(src), _stream(out)))
-    return float(n_workgroups) * 4 * iters * 16 * 32768.0

@@ -36,6 +36,7 @@ extern "C" {
 #define FMSA_ERR_UNSUPPORTED (-5) /* valid input the kernels do not cover            */
 #define FMSA_ERR_WORKSPACE (-6)   /* workspace missing or too small                  */
 #define FMSA_ERR_LAUNCH (-7)      /* hipGetLastError() after the launch was not success */
+#define FMSA_ERR_DEVICE (-8)      /* tensors on another GPU than the calling thread's current device */
 
 enum fmsa_dtype { FMSA_F16 = 0, FMSA_BF16 = 1, FMSA_F32 = 2 };
 
@@ -168,7 +169,9 @@ int fmsa_lora_grad_batch(const fmsa_lora_grad_job* jobs, int n_jobs, int M, int 
  * FMSA_ERR_WORKSPACE when fmsa_lora_grad_workspace(M, C, r) exceeds that size (16 MiB covers 8192 tokens x
  * 14336 columns at rank 16, or 4096 columns at rank 64).  All calls on one GPU share the buffer: calls that
  * overlap in time on one GPU (two streams, two threads) race on it; calls on one stream are ordered.  The very
- * first call on a device looks up the buffer's address (not an allocation); make that call outside a capture. */
+ * first call on a device looks up the buffer's address (not an allocation); make that call outside a capture.
+ * The buffer used is the copy of the calling thread's CURRENT device (hipGetDevice), which must be the GPU that
+ * owns L, R, out and the stream: an `out` the runtime places on another GPU returns FMSA_ERR_DEVICE. */
 #define FMSA_LORA_GRAD_STATIC_BYTES (16u << 20)
 int fmsa_lora_grad_static(const void* L, int64_t ldl, const void* R, int64_t ldr, int M, int C, int r, float scale,
                           int transpose_out, int act_dtype, int out_dtype, void* out, void* stream);
@@ -368,19 +371,6 @@ int fmsa_cross_entropy_bwd(void* logits, int64_t ld, const float* dloss, int64_t
 int fmsa_cross_entropy_fused(void* logits, int64_t ld, const int64_t* labels, int M, int V, int dtype,
                              int64_t ignore_index, const float* scale, float label_smoothing, float* losses,
                              void* stream);
-
-/* ------------------------------------------------------------------------------------------
- * Measurement support (no counterpart in the reference; used by bench.py --yardsticks).
- * A register-only loop of `iters` (even) x 16 MFMA 32x32x16 bf16 per wave, 4 waves per workgroup:
- *   mode 0  all-zero operands (what the clock allows),
- *   mode 1  random bf16 operands (what the power limit leaves),
- *   mode 2  as 1, plus one 1 KB direct-to-LDS load per wave and 8 MFMAs from `src` (>= 1 MiB), the
- *           ratio of the GEMM kernels' main loops,
- *   mode 3  as 2, with the A operands read from LDS (one 1 KB fragment read per wave and 2 MFMAs, a workgroup
- *           barrier per 64 MFMAs): the operand traffic of a main loop without the unpacking.
- * FLOP of a launch = n_workgroups * 4 * iters * 16 * 32768.  `out`: n_workgroups * 256 floats.
- * ------------------------------------------------------------------------------------------ */
-int fmsa_probe_mfma(int mode, int iters, int n_workgroups, void* out, const void* src, void* stream);
 
 #ifdef __cplusplus
 }

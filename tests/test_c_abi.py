@@ -27,6 +27,20 @@ def test_header_and_library_agree():
     assert lib.fmsa_strerror(0) == b"ok" and b"NULL" in lib.fmsa_strerror(-1)
 
 
+def test_probe_is_a_library_of_its_own():
+    """The MFMA-loop probe of `bench.py --yardsticks` is measurement support: the product library does not export it;
+    its own library does, and checks its arguments before any HIP call."""
+    assert not hasattr(fmsa_hip.lib(), "fmsa_probe_mfma")
+    path = os.path.join(ROOT, "fms-acceleration_amd", "lib", "libfmsa_probe.so")
+    f = ctypes.CDLL(path).fmsa_probe_mfma
+    f.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    assert f(0, 100, 16, None, None, None) == -1
+    assert f(2, 100, 16, 0x1000, None, None) == -1      # modes with direct loads need a source
+    assert f(4, 100, 16, 0x1000, 0x2000, None) == -2
+    assert f(1, 101, 16, 0x1000, None, None) == -2      # two fragment sets used in turn: an even number of iterations
+    assert f(1, 100, 0, 0x1000, None, None) == -2
+
+
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(fmsa_hip.GptqWeight) == 72
     assert ctypes.sizeof(fmsa_hip.FwdProj) == 128
@@ -67,17 +81,6 @@ def test_codebook_weight_validation():
     assert p(ctypes.byref(nf4(K=96)), 0x5000, 0x6000, None) == -2        # K % blocksize
     assert p(ctypes.byref(nf4(blocksize=0)), 0x5000, 0x6000, None) == -2
     assert p(ctypes.byref(nf4()), 0x5004, 0x6000, None) == -3
-
-
-def test_probe_validation():
-    """The measurement entry point checks its arguments before any HIP call too."""
-    f = fmsa_hip.lib().fmsa_probe_mfma
-    assert f(0, 100, 16, None, None, None) == -1
-    assert f(2, 100, 16, 0x1000, None, None) == -1      # modes with direct loads need a source
-    assert f(4, 100, 16, 0x1000, 0x2000, None) == -2
-    assert f(1, 0, 16, 0x1000, None, None) == -2
-    assert f(1, 101, 16, 0x1000, None, None) == -2      # two fragment sets used in turn: an even number of iterations
-    assert f(1, 100, 0, 0x1000, None, None) == -2
 
 
 def test_dequant_validation():

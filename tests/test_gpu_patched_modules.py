@@ -1,8 +1,10 @@
-"""Patched (fused) versus unpatched (unfused QuantLinear + LoRA) transformers modules, the
+"""Patched (fused) versus unpatched (unfused base linear + LoRA) transformers modules, the
 reference's own parity test design (plugins/fused-ops-and-kernels/tests/test_fused_ops.py:355-438):
-deep-copy a Llama attention / MLP whose projections are LoRA-wrapped GPTQ linears, patch one copy
+deep-copy an attention / MLP whose projections are LoRA-wrapped quantised linears, patch one copy
 through the ModelPatcher rules, run both under autocast, loss = out.norm(), compare the loss and
-the adapter gradients -- plus the input gradient, which the reference computes but never asserts."""
+the adapter gradients -- plus the input gradient, which the reference computes but never asserts.
+The reference runs this for a bitsandbytes Llama attention; here every architecture with a rule set
+(llama, mistral, granite: attention + MLP; mixtral: attention only) runs with both base types."""
 import copy
 
 import pytest
@@ -11,7 +13,7 @@ import torch
 from fms_acceleration.model_patcher import ModelPatcher, patch_model
 from fms_acceleration.utils.test_utils import instantiate_model_patcher
 from tests.helpers import randn
-from tests.model_utils import MaskDropout, make_lora_gptq_linear
+from tests.model_utils import MaskDropout, make_lora_gptq_linear, make_lora_nf4_linear
 
 pytestmark = pytest.mark.gpu
 
@@ -20,36 +22,58 @@ SIZES = [(1, 128, 2048), (2, 256, 2048)]
 R, ALPHA = 8, 1.0
 
 
-def _llama_cfg(hidden):
-    from transformers import LlamaConfig
+def _arch(name, hidden):
+    """(config, attention class, MLP class or None, rotary class, rules module) of one architecture, built from a config."""
+    import importlib
 
-    cfg = LlamaConfig(hidden_size=hidden, intermediate_size=2 * hidden, num_attention_heads=16, num_key_value_heads=4,
-                      num_hidden_layers=1, vocab_size=64, hidden_act="silu", attention_dropout=0.0)
+    kw = dict(hidden_size=hidden, intermediate_size=2 * hidden, num_attention_heads=16, num_key_value_heads=4,
+              num_hidden_layers=1, vocab_size=64, hidden_act="silu", attention_dropout=0.0)
+    tf = importlib.import_module(f"transformers.models.{name}.modeling_{name}")
+    cap = {"llama": "Llama", "mistral": "Mistral", "granite": "Granite", "mixtral": "Mixtral"}[name]
+    if name == "mixtral":
+        kw.update(num_local_experts=2, num_experts_per_tok=1)
+    if name == "mistral":
+        kw.update(sliding_window=None)
+    cfg = getattr(importlib.import_module(f"transformers.models.{name}.configuration_{name}"), cap + "Config")(**kw)
     cfg._attn_implementation = "eager"
-    return cfg
+    rules = importlib.import_module(f"fms_acceleration_foak.models.{name}")
+    return cfg, getattr(tf, cap + "Attention"), getattr(tf, cap + "MLP", None) if name != "mixtral" else None, \
+        getattr(tf, cap + "RotaryEmbedding"), rules
 
 
-def _wrap(mod, names, seed, dropout_p=0.0, tokens=None, act_order=False, dropout_on=None):
+def _llama_cfg(hidden):
+    return _arch("llama", hidden)[0]
+
+
+def _wrap(mod, names, seed, dropout_p=0.0, tokens=None, act_order=False, dropout_on=None, base_type="auto_gptq",
+          compute_dtype=torch.bfloat16):
     for i, name in enumerate(names):
         lin = getattr(mod, name)
         dropped = dropout_p is not None and (dropout_on is None or name in dropout_on) and (dropout_p or dropout_on)
         drop = MaskDropout(dropout_p, (tokens, lin.in_features), seed=seed + 50 + i) if dropped else None
-        wrapped, _, _, _ = make_lora_gptq_linear(lin.in_features, lin.out_features, R, ALPHA, seed=seed + i, dropout=drop,
-                                                 act_order=act_order)
+        if base_type == "bitsandbytes":
+            wrapped, _, _, _ = make_lora_nf4_linear(lin.in_features, lin.out_features, R, ALPHA, seed=seed + i, dropout=drop,
+                                                    compute_dtype=compute_dtype)
+        else:
+            wrapped, _, _, _ = make_lora_gptq_linear(lin.in_features, lin.out_features, R, ALPHA, seed=seed + i, dropout=drop,
+                                                     act_order=act_order)
         setattr(mod, name, wrapped)
 
 
-def _patched_copy(module, cfg):
-    from fms_acceleration_foak.models import llama
+def _patched_copy(module, cfg, rules=None, base_type="auto_gptq", arch="llama"):
+    if rules is None:
+        from fms_acceleration_foak.models import llama as rules
 
     twin = copy.deepcopy(module)
     with instantiate_model_patcher():
-        for rule in llama.get_mp_rules("auto_gptq", cfg):
+        for rule in rules.get_mp_rules(base_type, cfg):
             ModelPatcher.register(rule)
         patch_model(twin)
         # the rope rule swaps a function of the modeling module: it is not one of the twin's patched forwards
-        n_patched = sum(1 for h in ModelPatcher.history if not h.rule_id.endswith("-rope"))
-    return twin, n_patched
+        fired = sorted(h.rule_id for h in ModelPatcher.history if not h.rule_id.endswith("-rope"))
+    assert all(f.startswith(arch + "-") for f in fired), fired
+    twin._fired = fired
+    return twin, len(fired)
 
 
 def _lora_grads(module):
@@ -79,21 +103,27 @@ def _compare(ref_mod, fused_mod, run, x, dtype):
         assert torch.allclose(g0[name], g1[name], rtol=1e-3 * k, atol=1e-4 * k), name
 
 
+# (architecture, base type): every rule set with both base types; the reference's own case is (llama, bitsandbytes)
+ARCH_BASE = [(a, b) for a in ("llama", "mistral", "granite", "mixtral") for b in ("auto_gptq", "bitsandbytes")]
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("dropout_p", [0.0, 0.1, 0.5])
 @pytest.mark.parametrize("bsz,seq,hidden", SIZES)
-def test_attention_qkvo(bsz, seq, hidden, dropout_p, dtype):
-    from transformers.models.llama.modeling_llama import LlamaAttention, LlamaRotaryEmbedding
-
-    cfg = _llama_cfg(hidden)
-    attn = LlamaAttention(cfg, layer_idx=0)
-    _wrap(attn, ("q_proj", "k_proj", "v_proj", "o_proj"), seed=3, dropout_p=dropout_p, tokens=bsz * seq)
+@pytest.mark.parametrize("arch,base_type", ARCH_BASE)
+def test_attention_qkvo(arch, base_type, bsz, seq, hidden, dropout_p, dtype):
+    if arch != "llama" and (bsz, seq) != SIZES[0][:2] and dropout_p == 0.1:
+        pytest.skip("the other architectures run the larger size with dropout 0 and 0.5 only")
+    cfg, attn_cls, _, rotary_cls, rules = _arch(arch, hidden)
+    attn = attn_cls(cfg, layer_idx=0)
+    _wrap(attn, ("q_proj", "k_proj", "v_proj", "o_proj"), seed=3, dropout_p=dropout_p, tokens=bsz * seq, base_type=base_type,
+          compute_dtype=dtype)
     attn = attn.cuda()
-    fused, n_patched = _patched_copy(attn, cfg)
-    assert n_patched == 4
+    fused, n_patched = _patched_copy(attn, cfg, rules, base_type, arch)
+    assert fused._fired == [f"{arch}-qkvo-{i}" for i in (1, 2, 3, 4)]
     x = randn((bsz, seq, hidden), 2, dtype).cuda()
     pos = torch.arange(seq, device="cuda")[None].expand(bsz, -1)
-    cos, sin = LlamaRotaryEmbedding(cfg).cuda()(x, pos)
+    cos, sin = rotary_cls(cfg).cuda()(x, pos)
 
     def run(mod, xi):
         return mod(xi, position_embeddings=(cos, sin), attention_mask=None)[0]
@@ -106,16 +136,19 @@ def test_attention_qkvo(bsz, seq, hidden, dropout_p, dtype):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("act_order,dropout_p", [(False, 0.0), (True, 0.0), (True, 0.5), (False, 0.5)])
 @pytest.mark.parametrize("bsz,seq,hidden", SIZES)
-def test_mlp(bsz, seq, hidden, dtype, act_order, dropout_p):
-    from transformers.models.llama.modeling_llama import LlamaMLP
-
-    cfg = _llama_cfg(hidden)
-    mlp = LlamaMLP(cfg)
+@pytest.mark.parametrize("arch,base_type", [ab for ab in ARCH_BASE if ab[0] != "mixtral"])
+def test_mlp(arch, base_type, bsz, seq, hidden, dtype, act_order, dropout_p):
+    if act_order and base_type == "bitsandbytes":
+        pytest.skip("act-order is a GPTQ notion")
+    if arch != "llama" and (bsz, seq) != SIZES[0][:2]:
+        pytest.skip("the other architectures run the reference's first size")
+    cfg, _, mlp_cls, _, rules = _arch(arch, hidden)
+    mlp = mlp_cls(cfg)
     _wrap(mlp, ("gate_proj", "up_proj", "down_proj"), seed=9, dropout_p=dropout_p, tokens=bsz * seq, act_order=act_order,
-          dropout_on=("gate_proj", "up_proj") if dropout_p else None)
+          dropout_on=("gate_proj", "up_proj") if dropout_p else None, base_type=base_type, compute_dtype=dtype)
     mlp = mlp.cuda()
-    fused, n_patched = _patched_copy(mlp, cfg)
-    assert n_patched == 1
+    fused, n_patched = _patched_copy(mlp, cfg, rules, base_type, arch)
+    assert fused._fired == [f"{arch}-mlp"]
     x = randn((bsz, seq, hidden), 2, dtype).cuda()
     _compare(mlp, fused, lambda mod, xi: mod(xi), x, dtype)
 

@@ -260,21 +260,32 @@ def test_qkv_wrapper_with_rope_tables():
     with pytest.raises(RuntimeError, match="K does not"):
         re_mod.fast_rope_embedding(q, k.clone(), None, None)
     assert not re_mod._ROTATED
-    # an attention that is given tables but never rotates: the second call finds the first mark unconsumed and refuses
+    # an attention that is given tables but never rotates: refused when that very forward returns, not a call later
     class NoRope(torch.nn.Module):
+        boom = False
+
         def forward(self, hidden_states, position_embeddings=None):
-            return [fwd2[n](None, hidden_states) for n in names]
+            q = fwd2["q_proj"](None, hidden_states)
+            if self.boom:
+                raise MemoryError("inside the forward")
+            return [q] + [fwd2[n](None, hidden_states) for n in names[1:]]
 
     lazy = NoRope()
     fwd2 = dict(_build_fused_forwards(lazy, plain, names, with_rope))
-    lazy(x, position_embeddings=("c", "s"))
-    with pytest.raises(RuntimeError, match="did not call apply_rotary_pos_emb"):
+    with pytest.raises(RuntimeError, match="rotated twice"):
         lazy(x, position_embeddings=("c", "s"))
     assert not re_mod._ROTATED
+    # an exception between the fused call and the rotation leaves neither a mark nor pending outputs: the retry is clean
+    lazy.boom = True
+    with pytest.raises(MemoryError):
+        lazy(x, position_embeddings=("c", "s"))
+    assert not re_mod._ROTATED
+    lazy.boom = False
+    assert [o.flatten()[0].item() for o in lazy(x)] == [1, 2, 3]  # no tables: the plain operation, protocol intact
     # without tables the plain fused operation runs and nothing is marked
     for n in names:
         out = fwd[n](None, x)
-    assert out.flatten()[0] == 3 and not re_mod._ROTATED and len(seen) == 2  # (the two calls with tables above)
+    assert out.flatten()[0] == 3 and not re_mod._ROTATED and len(seen) == 3  # (the three calls with tables above)
 
 
 def test_fast_rope_embeddings_fused_qkv_is_accepted():

@@ -12,7 +12,7 @@ from tests.helpers import randn
 pytestmark = pytest.mark.gpu
 
 
-def _both(M, C, r, transpose_out, out_dtype, dtype, seed):
+def _both(M, C, r, transpose_out, out_dtype, dtype, seed, check_allocations=False):
     import fmsa_hip
 
     L = randn((M, r), seed, dtype).cuda()
@@ -21,12 +21,21 @@ def _both(M, C, r, transpose_out, out_dtype, dtype, seed):
     out = torch.full_like(ref, float("nan"))
     # straight through the C ABI: the caller owns inputs and output, the library brings its own scratch
     lib = fmsa_hip.lib()
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    allocs_before = torch.cuda.memory_stats()["allocation.all.allocated"]
     rc = lib.fmsa_lora_grad_static(ctypes.c_void_p(L.data_ptr()), L.stride(0), ctypes.c_void_p(R.data_ptr()), R.stride(0), M, C, r,
                                    ctypes.c_float(0.5), int(transpose_out), fmsa_hip.act_enum(dtype),
                                    {torch.float32: fmsa_hip.F32, torch.bfloat16: fmsa_hip.BF16, torch.float16: fmsa_hip.F16}[out_dtype],
                                    ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     assert rc == 0, fmsa_hip.lib().fmsa_strerror(rc)
     torch.cuda.synchronize()
+    if check_allocations:
+        # what the entry point exists for: neither the device's free memory (driver-level allocations: hipMalloc, module
+        # loads) nor torch's allocation count moves across the call, and a second query agrees
+        assert torch.cuda.memory_stats()["allocation.all.allocated"] == allocs_before
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert torch.cuda.mem_get_info()[0] == free_before
     return out, ref
 
 
@@ -35,9 +44,10 @@ def test_static_scratch_matches_workspace_entry_point_twice():
     out, ref = _both(8192, 14336, 16, False, torch.float32, torch.bfloat16, 1)
     assert torch.equal(out, ref)
     # second call, smaller and ragged (fewer splits, fewer columns, other rank): stale partial sums must not leak in
-    out, ref = _both(1000, 1024 + 32, 8, True, torch.bfloat16, torch.bfloat16, 3)
+    # (from here on the code object is loaded and the buffer's address known: the calls must not allocate)
+    out, ref = _both(1000, 1024 + 32, 8, True, torch.bfloat16, torch.bfloat16, 3, check_allocations=True)
     assert torch.equal(out, ref)
-    out, ref = _both(4096, 4096, 64, True, torch.float32, torch.float16, 5)
+    out, ref = _both(4096, 4096, 64, True, torch.float32, torch.float16, 5, check_allocations=True)
     assert torch.equal(out, ref)
 
 
