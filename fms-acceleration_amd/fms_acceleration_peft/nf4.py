@@ -107,6 +107,14 @@ class Params4bit(nn.Parameter):
         self.quant_state = quant_state
         return self
 
+    def __deepcopy__(self, memo):
+        import copy  # pylint: disable=import-outside-toplevel
+
+        # nn.Parameter's own __deepcopy__ would call the constructor with (data, requires_grad)
+        twin = type(self)(self.data.clone(memory_format=torch.preserve_format), copy.deepcopy(self.quant_state, memo))
+        memo[id(self)] = twin
+        return twin
+
 
 class Linear4bitFunction(torch.autograd.Function):
     """y = x @ deq(W)^T, dx = dy @ deq(W) for a frozen 4-bit weight (what bitsandbytes' MatMul4Bit computes:

@@ -35,6 +35,12 @@ def test_linear4bit_container_and_parameter_scrape():
     assert A.shape == (8, 128) and B.shape == (64, 8) and s == 2.0
     lin.enable_adapters(False)
     assert get_lora_parameters(lin)[3:] == (None, None, None, None)
+    import copy
+
+    twin = copy.deepcopy(lin)  # the quant state travels with the parameter through a deep copy
+    qs2 = twin.base_layer.weight.quant_state
+    assert qs2 is not qs and torch.equal(qs2.absmax, qs.absmax) and torch.equal(qs2.state2.absmax, qs.state2.absmax)
+    assert torch.equal(twin.base_layer.weight.data, base.weight.data) and twin.base_layer.weight.data_ptr() != base.weight.data_ptr()
 
 
 def test_fp4_book_and_unsorted_nearest():
@@ -97,7 +103,8 @@ def test_bnb_plugin_loader_augmentation_and_fused_rules(tmp_path, monkeypatch):
         monkeypatch.setattr(AccelerationFramework, "active_plugins", [])  # class-level state, as in the reference
         monkeypatch.setattr(AccelerationFramework, "plugins_require_custom_loading", [])
         fw = AccelerationFramework(str(cfg_file))
-        assert [type(p).__name__ for _, p in fw.active_plugins] == ["BNBAccelerationPlugin", "FastKernelsAccelerationPlugin"]
+        # (activation follows registration order, which follows import order)
+        assert sorted(type(p).__name__ for _, p in fw.active_plugins) == ["BNBAccelerationPlugin", "FastKernelsAccelerationPlugin"]
         model = fw.model_loader(str(tmp_path), torch_dtype=torch.bfloat16, device="cpu")
         quantised = [m for m in model.modules() if isinstance(m, Linear4bit)]
         assert len(quantised) == 14 and isinstance(model.lm_head, torch.nn.Linear)
