@@ -22,7 +22,7 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfmsa_hip.so")
 
-SOURCES = ["api.hip", "dequant.hip", "gemm_fwd.hip", "gemm_bwd.hip", "lora_skinny.hip", "elementwise.hip", "nf4.hip", "norm_rope.hip"]
+SOURCES = ["api.hip", "dequant.hip", "gemm_fwd.hip", "gemm_bwd.hip", "gemm_bwd_t.hip", "lora_skinny.hip", "elementwise.hip", "nf4.hip", "norm_rope.hip"]
 PROBE_SOURCE = "probe.hip"
 PROBE_LIB_PATH = os.path.join(LIB_DIR, "libfmsa_probe.so")
 

@@ -21,6 +21,10 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
 int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx, void* e,
                             void* g, void* h_out, int64_t ldeg, int act_dtype, hipStream_t st);
 
+int launch_gptq_lora_bwd_dx_t(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx, void* e,
+                              void* g, void* h_out, int64_t ldeg, int act_dtype, hipStream_t st);
+bool bwd_dx_twin_applies(const fmsa_bwd_proj* projs, int n_proj);
+int launch_gptq_transpose(const int32_t* qweight, int K, int N, int32_t* out, hipStream_t st);
 int launch_gptq_nsz(const fmsa_gptq_weight* w, float* out, hipStream_t st);
 int launch_lora_pack_batch(const fmsa_lora_pack_job* jobs, int n_jobs, int act_dtype, hipStream_t st);
 int launch_rms_fwd(const void* X, int64_t ldx, const void* W, int M, int C, float eps, int gemma, int x_dtype, int w_dtype, void* Y,
@@ -331,6 +335,7 @@ int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mod
     if (!s.dY || (!s.nsz && s.w.format != FMSA_WEIGHT_CODEBOOK)) return FMSA_ERR_NULL;
     if (s.lddy < s.w.N) return FMSA_ERR_SHAPE;
     if (s.nsz && !aligned16(s.nsz)) return FMSA_ERR_ALIGN;
+    if ((s.qweight_t && !aligned16(s.qweight_t)) || (s.scale_f32 && !aligned16(s.scale_f32))) return FMSA_ERR_ALIGN;
     if (!aligned16(s.dY) || s.lddy % 8 != 0) return FMSA_ERR_ALIGN;
     if (int rc = check_rank(s.r)) return rc;
     if (s.r > 0) {
@@ -357,7 +362,16 @@ int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mod
     if (lddx < K) return FMSA_ERR_SHAPE;
     if (!aligned16(dX) || lddx % 8 != 0) return FMSA_ERR_ALIGN;
   }
+  if (bwd_dx_twin_applies(projs, n_proj))
+    return launch_gptq_lora_bwd_dx_t(projs, n_proj, M, mode, dX, lddx, e, g, h_out, ldeg, act_dtype, (hipStream_t)stream);
   return launch_gptq_lora_bwd_dx(projs, n_proj, M, mode, dX, lddx, e, g, h_out, ldeg, act_dtype, (hipStream_t)stream);
+}
+
+int fmsa_gptq_transpose(const int32_t* qweight, int K, int N, int32_t* qweight_t_out, void* stream) {
+  if (!qweight || !qweight_t_out) return FMSA_ERR_NULL;
+  if (K <= 0 || N <= 0 || K % 8 != 0 || N % 8 != 0) return FMSA_ERR_SHAPE;
+  if (!aligned16(qweight) || !aligned16(qweight_t_out)) return FMSA_ERR_ALIGN;
+  return launch_gptq_transpose(qweight, K, N, qweight_t_out, (hipStream_t)stream);
 }
 
 int fmsa_swiglu_fwd(const void* e, const void* g, void* h, int M, int I, int64_t ld, int act_dtype, void* stream) {

@@ -137,8 +137,9 @@ class _Proj:
                         if permuted is not None:
                             permuted[key] = (mask_src, pm)  # holds the source too: its id stays taken
                         mask_src = pm
+        qweight_t, scale_f32 = self.w.twin
         return {"w": self.w.struct, "nsz": self.w.nsz, "dY": dY2, "T": T, "At": At, "mask_src": mask_src if self.r else None,
-                "r": self.r, "s": self.s}
+                "r": self.r, "s": self.s, "qweight_t": qweight_t, "scale_f32": scale_f32}
 
     def lora_grads(self, T, Xd, U, dY2):
         """dA [r, K] = s T^T Xd and dB [N, r] = s dY^T U, in the dtypes of the parameters."""

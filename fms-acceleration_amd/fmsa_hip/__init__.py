@@ -42,6 +42,7 @@ EXPORTED_SYMBOLS = (
     "fmsa_swiglu_fwd",
     "fmsa_swiglu_bwd",
     "fmsa_gptq_make_nsz",
+    "fmsa_gptq_transpose",
     "fmsa_nf4_dequant",
     "fmsa_nf4_prepare",
     "fmsa_lora_pack",
@@ -167,6 +168,8 @@ class BwdProj(Structure):
         ("ldmask", c_int64),
         ("r", c_int32),
         ("s", c_float),
+        ("qweight_t", c_void_p),
+        ("scale_f32", c_void_p),
     ]
 
 
@@ -212,6 +215,7 @@ def lib() -> ctypes.CDLL:
     L.fmsa_swiglu_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
     L.fmsa_swiglu_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
     L.fmsa_gptq_make_nsz.argtypes = [POINTER(GptqWeight), c_void_p, c_void_p]
+    L.fmsa_gptq_transpose.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p]
     L.fmsa_nf4_dequant.argtypes = [POINTER(Nf4Weight), c_int, c_void_p, c_void_p]
     L.fmsa_nf4_prepare.argtypes = [POINTER(Nf4Weight), c_void_p, c_void_p, c_void_p]
     L.fmsa_lora_pack.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -461,8 +465,9 @@ def gptq_lora_fwd(x2d, projs: Sequence[dict], mode: int = FWD_LINEAR, rope=None)
 
 
 def gptq_lora_bwd_dx(projs: Sequence[dict], M: int, K: int, mode: int = BWD_LINEAR, e=None, g=None):
-    """projs: dicts with keys w, nsz, dY, T, At, mask_src, r, s.  LINEAR mode returns dX [M, K];
-    SWIGLU mode overwrites e <- d_g, g <- d_e and returns h."""
+    """projs: dicts with keys w, nsz, dY, T, At, mask_src, r, s and optionally qweight_t, scale_f32 (the weight's
+    transposed twin, see gptq_transpose).  LINEAR mode returns dX [M, K]; SWIGLU mode overwrites e <- d_g,
+    g <- d_e and returns h."""
     arr = (BwdProj * len(projs))()
     ref = projs[0]["dY"]
     for i, p in enumerate(projs):
@@ -473,7 +478,7 @@ def gptq_lora_bwd_dx(projs: Sequence[dict], M: int, K: int, mode: int = BWD_LINE
         assert T is None or T.stride(1) == 1
         arr[i] = BwdProj(p["w"], _ptr(p["nsz"]), _ptr(dy), dy.stride(0), _ptr(T), 0 if T is None else T.stride(0),
                          _ptr(p.get("At")) if p["r"] else None, _ptr(ms), 0 if ms is None else ms.stride(0),
-                         int(p["r"]), float(p["s"] or 0.0))
+                         int(p["r"]), float(p["s"] or 0.0), _ptr(p.get("qweight_t")), _ptr(p.get("scale_f32")))
     if mode == BWD_SWIGLU:
         h = torch.empty_like(e)
         _check("fmsa_gptq_lora_bwd_dx",
@@ -485,6 +490,21 @@ def gptq_lora_bwd_dx(projs: Sequence[dict], M: int, K: int, mode: int = BWD_LINE
            lib().fmsa_gptq_lora_bwd_dx(arr, len(projs), M, mode, _ptr(dx), dx.stride(0), None, None, None, 0,
                                        act_enum(ref.dtype), _stream(ref)))
     return dx
+
+
+def dx_twin_enabled() -> bool:
+    """Whether prepared weights build the transposed twin the input-gradient kernel prefers (one more packed copy
+    of every frozen weight, 4 bits per weight, plus fp32 scales).  FMSA_DX_TWIN=0 keeps the checkpoint layout only."""
+    return os.environ.get("FMSA_DX_TWIN", "1") != "0"
+
+
+def gptq_transpose(qweight):
+    """The transposed twin [N/8, K] of a packed weight [K/8, N]: nibble j of word [n8, k] = q[k, 8 n8 + j]."""
+    K8, N = qweight.shape
+    assert qweight.dtype == torch.int32 and qweight.is_contiguous() and N % 8 == 0
+    out = torch.empty((N // 8, K8 * 8), dtype=torch.int32, device=qweight.device)
+    _check("fmsa_gptq_transpose", lib().fmsa_gptq_transpose(_ptr(qweight), K8 * 8, N, _ptr(out), _stream(qweight)))
+    return out
 
 
 def swiglu_fwd(e, g):

@@ -16,7 +16,8 @@ class PreparedWeight:
     same order from act-order GPTQ (it sorts by the diagonal of the input's Hessian): `perm_key`
     lets their callers see that and keep them in one launch."""
 
-    __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep", "_zero_offset", "_columns", "col_inv", "_row_inv")
+    __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep", "_zero_offset", "_columns", "col_inv", "_row_inv",
+                 "_twin")
 
     def __init__(self, qweight, scales, qzeros, g_idx, bits):
         if bits != 4:
@@ -50,10 +51,25 @@ class PreparedWeight:
 
     def _finish(self, qweight, scales, qzeros):
         self._keep = (qweight, scales, qzeros)
+        self._twin = None
         self.struct = fmsa_hip.make_weight(qweight, scales, qzeros, None, self.group_size, self._zero_offset)
         # -scale * zero per (group, column), fp32: read by the input-gradient kernel (frozen weight,
         # so it is built once)
         self.nsz = fmsa_hip.gptq_make_nsz(self.struct, qweight.device)
+
+    @property
+    def twin(self):
+        """(qweight_t int32 [N/8, K], scale_f32 [G, N]) for the input-gradient kernel, built on first use (the weight
+        is frozen): the nibbles packed along N, so that a lane's word is its MFMA fragment as in the forward kernel,
+        and the scales widened once.  (None, None) when switched off or when a group does not hold whole 64-column
+        wave tiles (the kernel then reads the checkpoint layout)."""
+        if self._twin is None:
+            if fmsa_hip.dx_twin_enabled() and self.group_size % 64 == 0:
+                qweight, scales, _ = self._keep
+                self._twin = (fmsa_hip.gptq_transpose(qweight), scales.to(torch.float32).contiguous())
+            else:
+                self._twin = (None, None)
+        return self._twin
 
     @property
     def row_inv(self):

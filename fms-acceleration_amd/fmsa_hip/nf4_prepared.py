@@ -52,7 +52,7 @@ def _shared_code_book(code, device):
 class PreparedNf4Weight:
     """The C-ABI view (`struct`, code-book format) of one NF4 linear of shape [N, K]."""
 
-    __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep")
+    __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep", "_twin")
 
     def __init__(self, W, quant_state):
         quant_state = normalize_quant_state(quant_state)
@@ -75,7 +75,22 @@ class PreparedNf4Weight:
         self.perm = self.perm_key = None  # no act-order for NF4
         self.nsz = None   # the input-gradient kernel reads block_scale through the struct
         self._keep = (qweight, block_scale, code)
+        self._twin = None
         self.struct = fmsa_hip.make_codebook_weight(qweight, code, block_scale, bs)
+
+
+def _twin(self):
+    """(qweight_t int32 [N/8, K], None): the codes packed along N for the input-gradient kernel, built on first use
+    (see gptq_prepared.PreparedWeight.twin; the block scales are fp32 already)."""
+    if self._twin is None:
+        if fmsa_hip.dx_twin_enabled() and self.group_size % 64 == 0:
+            self._twin = (fmsa_hip.gptq_transpose(self._keep[0]), None)
+        else:
+            self._twin = (None, None)
+    return self._twin
+
+
+PreparedNf4Weight.twin = property(_twin)
 
 
 def prepare(W, quant_state) -> PreparedNf4Weight:

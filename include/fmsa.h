@@ -267,6 +267,14 @@ typedef struct fmsa_bwd_proj {
   int64_t ldmask;
   int32_t r;
   float s;
+  /* Optional per-weight twin for this kernel, built once (the base weight is frozen): the nibbles packed along N,
+   * qweight_t int32 [N/8, K] from fmsa_gptq_transpose, and for the affine format the scales widened to fp32,
+   * scale_f32 [G, N].  When every projection of a call carries them (and every group_size % 64 == 0) the kernel
+   * reads the twin: a lane's word is then its MFMA fragment, as in the forward kernel, instead of an 8 x 8 block of
+   * nibbles that has to be transposed with byte shuffles.  Same values, same contraction order: bit-identical
+   * results.  NULL: the checkpoint layout in `w` is read. */
+  const int32_t* qweight_t;
+  const float* scale_f32;
 } fmsa_bwd_proj;
 
 enum fmsa_bwd_mode { FMSA_BWD_LINEAR = 0, FMSA_BWD_SWIGLU = 1 };
@@ -275,6 +283,11 @@ enum fmsa_bwd_mode { FMSA_BWD_LINEAR = 0, FMSA_BWD_SWIGLU = 1 };
  * (z[g, n] + zero_offset), fp32 [G, N] (exact: 11-bit x 5-bit).  The base weight is frozen, so a
  * caller builds it once per weight. */
 int fmsa_gptq_make_nsz(const fmsa_gptq_weight* w /*host*/, float* out, void* stream);
+
+/* The transposed twin of a packed weight for fmsa_bwd_proj.qweight_t: out int32 [N/8, K], nibble j of word
+ * [n8, k] = q[k, 8*n8 + j], from qweight int32 [K/8, N] (pack() of qlinear_tritonv2.py:132-147 packs along K).
+ * For an act-order weight pass the row-repacked qweight (fmsa_gptq_permute_rows).  K % 8 == 0, N % 8 == 0. */
+int fmsa_gptq_transpose(const int32_t* qweight, int K, int N, int32_t* qweight_t_out, void* stream);
 
 int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs /*host*/, int n_proj, int M, int mode,
                           void* dX, int64_t lddx, void* e, void* g, void* h_out, int64_t ldeg,

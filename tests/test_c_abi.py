@@ -44,7 +44,7 @@ def test_probe_is_a_library_of_its_own():
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(fmsa_hip.GptqWeight) == 72
     assert ctypes.sizeof(fmsa_hip.FwdProj) == 128
-    assert ctypes.sizeof(fmsa_hip.BwdProj) == 144
+    assert ctypes.sizeof(fmsa_hip.BwdProj) == 160
     assert ctypes.sizeof(fmsa_hip.LoraGradJob) == 88
     assert ctypes.sizeof(fmsa_hip.LoraPackJob) == 64
 

@@ -18,8 +18,10 @@ def dev(t):
 def gweight(w, identity=True):
     import fmsa_hip
 
-    t = {k: dev(v) for k, v in w["t"].items()}
-    w["dev"] = t
+    t = w.get("dev")  # the C struct holds raw pointers: one device copy per weight, kept alive by the dict
+    if t is None:
+        t = {k: dev(v) for k, v in w["t"].items()}
+        w["dev"] = t
     return fmsa_hip.make_weight(t["qweight"], t["scales"], t["qzeros"], None if identity else t["g_idx"],
                                 w["group_size"], w["zero_offset"])
 
@@ -321,12 +323,24 @@ def test_fwd_swiglu(M, H, I, dtype):
     assert olora.max_rel_err(h.cpu(), torch.nn.functional.silu(e_ref) * g_ref) < TOL
 
 
-def _proj_bwd(w, dy_dev, A, B, s, dtype, mask_src=None):
+def _twin(w):
+    """The weight's transposed twin for the input-gradient kernel (packed along N, fp32 scales); None, None when a
+    group does not hold whole 64-column tiles (the kernel then reads the checkpoint layout)."""
+    import fmsa_hip
+
+    if w["group_size"] % 64 != 0:
+        return {"qweight_t": None, "scale_f32": None}
+    return {"qweight_t": fmsa_hip.gptq_transpose(w["dev"]["qweight"]), "scale_f32": w["dev"]["scales"].float().contiguous()}
+
+
+def _proj_bwd(w, dy_dev, A, B, s, dtype, mask_src=None, twin=False):
     import fmsa_hip
 
     gw = gweight(w)
     p = {"w": gw, "nsz": fmsa_hip.gptq_make_nsz(gw, dy_dev.device), "r": A.shape[0], "s": s, "dY": dy_dev,
          "mask_src": mask_src}
+    if twin:
+        p.update(_twin(w))
     p["T"] = fmsa_hip.lora_down(dy_dev, dev(B.to(dtype).t().contiguous()))
     p["At"] = dev(A.to(dtype).t().contiguous())
     return p
@@ -338,7 +352,8 @@ def _proj_bwd(w, dy_dev, A, B, s, dtype, mask_src=None):
     (200, 1056, 1024, 64, 8),   # ragged M; K not a multiple of the 256-wide output tile
     (256, 256, 96, 128, 64),    # N not a multiple of the 64-wide stage
 ])
-def test_bwd_dx_linear(M, K, N, gs, r, dtype):
+@pytest.mark.parametrize("twin", [False, True])
+def test_bwd_dx_linear(M, K, N, gs, r, dtype, twin):
     import fmsa_hip
 
     s = 2.0
@@ -348,11 +363,11 @@ def test_bwd_dx_linear(M, K, N, gs, r, dtype):
     x[::7, ::5] = 0  # exact zeros: the LoRA part of dX is masked there
     dy = randn((M, N), 3, dtype)
     dyd = dev(dy)
-    dx = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(w, dyd, A, B, s, dtype, mask_src=dev(x))], M, K)
+    dx = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(w, dyd, A, B, s, dtype, mask_src=dev(x), twin=twin)], M, K)
     ref, _, _ = olora.lora_w_manual(x.float(), w["dense"], A.to(dtype).float(), B.to(dtype).float(), s, dy.float())
     assert olora.max_rel_err(dx.cpu(), ref) < TOL
     # without the mask source the LoRA term is applied everywhere
-    dx2 = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(w, dyd, A, B, s, dtype)], M, K)
+    dx2 = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(w, dyd, A, B, s, dtype, twin=twin)], M, K)
     ref2 = dy.float() @ w["dense"].t() + (dy.float() @ B.to(dtype).float()) @ (s * A.to(dtype).float())
     assert olora.max_rel_err(dx2.cpu(), ref2) < TOL
 
@@ -396,13 +411,18 @@ def test_fwd_and_bwd_random_shapes(M, K, N, gs, r, bias, dtype):
     dyd = dev(dy)
     if r:
         dx = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(w, dyd, A, B, s, dtype, mask_src=xd)], M, K)
+        # the kernel flavour that reads the transposed twin: same values in the same order, so the same bits
+        dx_t = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(w, dyd, A, B, s, dtype, mask_src=xd, twin=True)], M, K)
+        assert torch.equal(dx, dx_t)
         dx_ref, dA_ref, dB_ref = olora.lora_w_manual(x.float(), w["dense"], Aq, Bq, s, dy.float())
         T = fmsa_hip.lora_down(dyd, dev(B.to(dtype).t().contiguous()))
         dA, dB = fmsa_hip.lora_grad_batch([(T, xd, s, False, torch.float32), (p["U"], dyd, s, True, torch.float32)])
         assert olora.max_rel_err(dA.cpu(), dA_ref) < TOL and olora.max_rel_err(dB.cpu(), dB_ref) < TOL
     else:
-        dx = fmsa_hip.gptq_lora_bwd_dx([{"w": gw, "nsz": fmsa_hip.gptq_make_nsz(gw, dyd.device), "dY": dyd, "T": None, "At": None,
-                                         "mask_src": None, "r": 0, "s": 0.0}], M, K)
+        base = {"w": gw, "nsz": fmsa_hip.gptq_make_nsz(gw, dyd.device), "dY": dyd, "T": None, "At": None,
+                "mask_src": None, "r": 0, "s": 0.0}
+        dx = fmsa_hip.gptq_lora_bwd_dx([base], M, K)
+        assert torch.equal(dx, fmsa_hip.gptq_lora_bwd_dx([{**base, **_twin(w)}], M, K))
         dx_ref = dy.float() @ w["dense"].t()
     assert olora.max_rel_err(dx.cpu(), dx_ref) < TOL
 
@@ -421,14 +441,19 @@ def test_bwd_dx_three_projections(dtype):
     xd = dev(x)  # one mask source for the whole call
     projs = [_proj_bwd(w, dev(dy), A, B, s, dtype, mask_src=xd) for w, (A, B), dy in zip(ws, ABs, dys)]
     dx = fmsa_hip.gptq_lora_bwd_dx(projs, M, K)
+    twins = [_proj_bwd(w, dev(dy), A, B, s, dtype, mask_src=xd, twin=True) for w, (A, B), dy in zip(ws, ABs, dys)]
+    assert torch.equal(dx, fmsa_hip.gptq_lora_bwd_dx(twins, M, K))
+    # a call in which one projection comes without its twin takes the checkpoint-layout kernel for all of them
+    assert torch.equal(dx, fmsa_hip.gptq_lora_bwd_dx([twins[0], projs[1], twins[2]], M, K))
     ref, _ = olora.lora_qkv_manual(x.float(), [(w["dense"], A.to(dtype).float(), B.to(dtype).float(), s)
                                                  for w, (A, B) in zip(ws, ABs)], [d.float() for d in dys])
     assert olora.max_rel_err(dx.cpu(), ref) < TOL
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,H,I", [(256, 512, 1024), (200, 256, 352)])
-def test_bwd_swiglu(M, H, I, dtype):
+@pytest.mark.parametrize("M,H,I", [(256, 512, 1024), (200, 256, 352), (300, 288, 640)])
+@pytest.mark.parametrize("twin", [False, True])
+def test_bwd_swiglu(M, H, I, dtype, twin):
     """Down-projection backward: dh = dY Wd^T + LoRA, then the in-place SwiGLU backward."""
     import fmsa_hip
 
@@ -440,7 +465,7 @@ def test_bwd_swiglu(M, H, I, dtype):
     g = randn((M, I), 8, dtype)
     dy = randn((M, H), 9, dtype)
     e_d, g_d = dev(e).clone(), dev(g).clone()
-    h = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(wd, dev(dy), Ad, Bd, s, dtype)], M, I, fmsa_hip.BWD_SWIGLU, e=e_d, g=g_d)
+    h = fmsa_hip.gptq_lora_bwd_dx([_proj_bwd(wd, dev(dy), Ad, Bd, s, dtype, twin=twin)], M, I, fmsa_hip.BWD_SWIGLU, e=e_d, g=g_d)
     h_mask = (olora.swiglu_fwd(e, g) != 0).float()
     dh_ref = dy.float() @ wd["dense"].t() + h_mask * ((dy.float() @ Bd.to(dtype).float()) @ (s * Ad.to(dtype).float()))
     # h does not depend on the GEMM: it must match the reference's rounding points closely
@@ -454,3 +479,20 @@ def test_bwd_swiglu(M, H, I, dtype):
     de_ref = dh_ref * g32 * se * (1.0 + e32 * (1.0 - se))
     assert olora.max_rel_err(e_d.cpu(), dg_ref) < TOL
     assert olora.max_rel_err(g_d.cpu(), de_ref) < TOL
+
+
+@pytest.mark.parametrize("K,N", [(32, 32), (256, 96), (1056, 1024)])
+def test_gptq_transpose_bit_exact(K, N):
+    """The twin's packing: nibble j of word [n8, k] = q[k, 8 n8 + j], against a plain numpy re-packing of the
+    unpacked 4-bit values (the unpack is the oracle's, which the layout tests pin bit by bit)."""
+    import numpy as np
+
+    import fmsa_hip
+
+    w = make_gptq(K, N, 32, seed=K + 3 * N)
+    q = ogptq.unpack_rows(w["np"]["qweight"]).astype(np.uint32)  # [K, N]
+    want = np.zeros((N // 8, K), dtype=np.uint32)
+    for j in range(8):
+        want |= q[:, j::8].T << np.uint32(4 * j)
+    got = fmsa_hip.gptq_transpose(dev(w["t"]["qweight"])).cpu().numpy().view(np.uint32)
+    assert np.array_equal(got, want)
