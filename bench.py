@@ -41,7 +41,7 @@ TOL_OUT, TOL_GRAD = 1e-2, 2e-2  # max |out - ref| / max |ref| per tensor: output
 # WRITE_SIZE, scaled by a device copy of known size): lines `roofline_traffic_bytes <kernel label> = <bytes>`,
 # and `kernel_sources_sha256 = <digest>` of the two GEMM sources the counters were taken with.
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gptq_lora_gemms_llama3_8b_hbm_traffic_pmc.txt")
-GEMM_SOURCES = [os.path.join(ROOT, "fms-acceleration_amd", "csrc", f) for f in ("gemm_fwd.hip", "gemm_bwd.hip", "common.h")]
+GEMM_SOURCES = [os.path.join(ROOT, "fms-acceleration_amd", "csrc", f) for f in ("gemm_fwd.hip", "gemm_bwd.hip", "gemm_bwd_t.hip", "common.h")]
 
 _W_BYTES = HIDDEN * INTER // 2 + (HIDDEN // GROUP) * INTER * 2 + (HIDDEN // GROUP) * INTER // 2  # packed + scales + zeros
 # algorithmic bytes of the launches that can be the dominant one
@@ -49,10 +49,11 @@ ALGORITHMIC_BYTES = {
     # X once, gate and up weights once, U and B, the three outputs e, g, h
     "gptq_lora_fwd<swiglu> K=4096 N=14336+14336":
         M_TOKENS * HIDDEN * 2 + 2 * _W_BYTES + 2 * (M_TOKENS * RANK * 2 + INTER * RANK * 2) + 3 * M_TOKENS * INTER * 2,
-    # d_g and d_e once, up and gate weights + fp32 offset tables once, T and A^T, the mask source X, dX
+    # d_g and d_e once, the transposed twins of the up and gate weights + their fp32 scale and offset tables once, T and
+    # A^T, the mask source X, dX
     "gptq_lora_bwd_dx<linear> K=4096 N=14336+14336":
-        2 * M_TOKENS * INTER * 2 + 2 * (_W_BYTES + (HIDDEN // GROUP) * INTER * 4) + 2 * (M_TOKENS * RANK * 2 + HIDDEN * RANK * 2)
-        + 2 * M_TOKENS * HIDDEN * 2,
+        2 * M_TOKENS * INTER * 2 + 2 * (HIDDEN * INTER // 2 + 2 * (HIDDEN // GROUP) * INTER * 4)
+        + 2 * (M_TOKENS * RANK * 2 + HIDDEN * RANK * 2) + 2 * M_TOKENS * HIDDEN * 2,
 }
 
 
@@ -515,6 +516,43 @@ def attention_config(device, dtype, attn, steps=20, warmup=5):
             "workload": "LoRA_QKV + LoRA_W(o_proj) fwd+bwd, 8192 tokens, 32 + 8 heads of 128, GPTQ g128, r=16"}
 
 
+def fp16_layer_config(device, attn, mlp, M, steps, warmup):
+    """The same layer step in float16, the reference's own arithmetic for the GPTQ path (its dequantisation always emits
+    fp16 and its GPTQ-LoRA benchmarks run in fp16: scripts/benchmarks/scenarios.yaml:111-112): outputs and dX of one step
+    on 128 sampled token rows against the fp32 oracle first, then the timed steps and the per-launch figures."""
+    import torch
+
+    dtype = torch.float16
+    io = {}
+    step = make_step(attn, mlp, M, device, dtype, io)
+    step()
+    torch.cuda.synchronize()
+    rows = torch.randperm(M, generator=torch.Generator().manual_seed(11))[:128].sort().values
+    torch.set_num_threads(cpu_threads())
+    ref = oracle_step(attn, mlp, io, dtype, rows)()
+    got = gpu_results(attn, mlp, io, rows)
+    keep = [k for k in ref if not k.startswith(("dA_", "dB_"))]
+    parity = parity_report({k: got[k] for k in keep}, {k: ref[k] for k in keep},
+                           "outputs and dX of one float16 step on 128 sampled token rows against the fp32 oracle")
+    del got, ref, io
+    out = {"workload": "the headline layer step in float16 (LoRA_QKV + LoRA_W(o_proj) + LoRA_MLP fwd+bwd, 8192 tokens)",
+           "dtype": "f16", "parity": {k: parity[k] for k in ("ok", "checked", "max_rel_err", "max_rel_err_tensor", "tolerance")}}
+    if not parity["ok"]:
+        out["error"] = "parity check failed, not timed"
+        return out
+    step = make_step(attn, mlp, M, device, dtype)
+    dt = time_steps(step, steps, warmup)
+    fl = layer_flops(M)
+    out.update({"ms_per_step": dt * 1e3, "tokens_per_s": M / dt, "tflops": fl / dt / 1e12,
+                "frac_f16_mfma_peak": fl / dt / 1e12 / PEAK_BF16_TFLOPS})  # fp16 and bf16 dense MFMA peaks are equal
+    with LaunchTimer(M) as timer:
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+    out["kernels"] = {k: {"ms": v[0], "tflops": v[1] / v[0] / 1e9} for k, v in timer.summary().items()}
+    return out
+
+
 def yardsticks(device):
     """What the machine at hand sustains, next to the fused kernels' figures: the vendor library's plain bf16 GEMM of
     the gate/up shape (no dequantisation, no LoRA, no SwiGLU), and the register-only MFMA loop of the library with
@@ -706,6 +744,7 @@ def main():
         result["cpu_baseline"] = cpu_base
     if not args.no_other_configs:
         del step
+        fp16_cfg = fp16_layer_config(device, attn, mlp, M, args.steps, args.warmup)
         rope_cfg = qkv_rope_config(device, dtype, attn)
         attn_cfg = attention_config(device, dtype, attn)
         attn = None
@@ -713,6 +752,7 @@ def main():
         result["other_configs"] = other_configs(device, dtype, mlp)
         result["other_configs"]["config3_llama3_8b_attention"] = attn_cfg
         result["other_configs"]["qkv_with_rope_llama3_8b"] = rope_cfg
+        result["other_configs"]["llama3_8b_layer_fp16"] = fp16_cfg
     print(json.dumps(result))
 
 
