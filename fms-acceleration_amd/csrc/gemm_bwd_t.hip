@@ -260,51 +260,6 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
           wf[par][j][b] = pack2<T>(__uint_as_float(gath[j][b]) * __uint_as_float(bsv[b >> 1][2 * (b & 1)]),
                                    __uint_as_float(gath[j][4 + b]) * __uint_as_float(bsv[b >> 1][2 * (b & 1) + 1]));
     };
-    auto mfma_step = [&](auto par_c) {
-      constexpr int par = decltype(par_c)::value;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[par][j], xf[par][mt], acc[mt][j]);
-    };
-    auto mfma_half = [&](auto par_c, auto h_c) {
-      constexpr int par = decltype(par_c)::value;
-      constexpr int h = decltype(h_c)::value;
-#pragma unroll
-      for (int mt = h * (MT / 2); mt < (h + 1) * (MT / 2); ++mt)
-#pragma unroll
-        for (int j = 0; j < NT; ++j) acc[mt][j] = mfma32<T>(wf[par][j], xf[par][mt], acc[mt][j]);
-    };
-    // code-book halves: (a) 8 MFMAs with the address arithmetic and the LDS-pipe instructions (8 fragment reads, 2 table
-    // reads, 16 gathers); (b) 8 MFMAs with the 24 multiplies / conversions and, in the last step of a stage, the loads
-    // of a later stage
-    auto interleave_a = [&]() {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-        if (i < 2)
-          __builtin_amdgcn_sched_group_barrier(0x080, 4, 0);
-        else
-          __builtin_amdgcn_sched_group_barrier(0x080, 3, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    auto interleave_b = [&](auto with_vmem_c) {
-      constexpr bool with_vmem = decltype(with_vmem_c)::value;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
-        if (with_vmem) {
-          if (i == 0)
-            __builtin_amdgcn_sched_group_barrier(0x020, 3, 0);
-          else
-            __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    };
     using WithVmem = std::integral_constant<bool, true>;
     using NoVmem = std::integral_constant<bool, false>;
     // The affine step written slot by slot: the 16 MFMAs of parity `cur`, each followed by its share of the work that
@@ -388,14 +343,125 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
         fence();
       });
     };
+    // The code-book step slot by slot.  The LDS pipe carries 26 instructions per step here (8 fragment reads, 2 table
+    // reads, 16 gathers) next to the other waves' share, so they are spread as evenly as the dependencies allow: the
+    // gathers of a fragment register's two weights go out first, its product follows about four MFMAs later.
+    auto step_codebook = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c, int st_next, auto lb_c) {
+      constexpr int SB = decltype(nb_c)::value;
+      constexpr int t = decltype(nt_c)::value;
+      constexpr int par = decltype(nx_c)::value;
+      constexpr int cur = decltype(cur_c)::value;
+      constexpr bool with_vmem = decltype(vmem_c)::value;
+      const char* lt = tb_buf(nb_c);
+      const char* lr = dy_buf(nb_c) + dy_r[t];
+      const int li = (int)__float_as_uint(lut);
+      auto mfma_slot = [&](int slot) { acc[slot >> 1][slot & 1] = mfma32<T>(wf[cur][slot & 1], xf[cur][slot >> 1], acc[slot >> 1][slot & 1]); };
+      auto frag = [&](int mt) { xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2); };
+      auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+      auto dma = [&](auto idx_c) {
+        if constexpr (with_vmem) load_piece(st_next, lb_c, idx_c);
+      };
+      uint32_t ad[NT][2];  // [tile][0]: byte b = 4 * nibble 2b (a lane's byte address in the table); [1]: nibble 2b + 1
+      uint32_t ga[NT][8];  // code of nibble 2b in [b], of nibble 2b + 1 in [4 + b]
+      u32x4 bs[2];
+      // the two gathers of fragment register `reg` of tile `j`
+      auto gather2 = [&](auto j_c, auto reg_c) {
+        constexpr int j = decltype(j_c)::value;
+        constexpr int reg = decltype(reg_c)::value;
+        ga[j][reg] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((ad[j][0] >> (8 * reg)) & 0xffu), li);
+        ga[j][4 + reg] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((ad[j][1] >> (8 * reg)) & 0xffu), li);
+      };
+      auto piece = [&](auto j_c, auto reg_c) {
+        constexpr int j = decltype(j_c)::value;
+        constexpr int reg = decltype(reg_c)::value;
+        wf[par][j][reg] = pack2<T>(__uint_as_float(ga[j][reg]) * __uint_as_float(bs[reg >> 1][2 * (reg & 1)]),
+                                   __uint_as_float(ga[j][4 + reg]) * __uint_as_float(bs[reg >> 1][2 * (reg & 1) + 1]));
+      };
+      using J0 = std::integral_constant<int, 0>;
+      using J1 = std::integral_constant<int, 1>;
+      mfma_slot(0);
+      bs[0] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * 64);
+      bs[1] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * 64 + 16);
+      ad[0][0] = opaque((qw[SB][0][t] << 2) & 0x3C3C3C3Cu);
+      ad[0][1] = opaque((qw[SB][0][t] >> 2) & 0x3C3C3C3Cu);
+      gather2(J0{}, I0{});
+      dma(std::integral_constant<int, 0>{});
+      fence();
+      mfma_slot(1);
+      ad[1][0] = opaque((qw[SB][1][t] << 2) & 0x3C3C3C3Cu);
+      ad[1][1] = opaque((qw[SB][1][t] >> 2) & 0x3C3C3C3Cu);
+      gather2(J1{}, I0{});
+      dma(std::integral_constant<int, 1>{});
+      fence();
+      mfma_slot(2);
+      gather2(J0{}, I1{});
+      dma(std::integral_constant<int, 2>{});
+      fence();
+      mfma_slot(3);
+      gather2(J1{}, I1{});
+      dma(std::integral_constant<int, 3>{});
+      fence();
+      mfma_slot(4);
+      frag(0);
+      frag(1);
+      dma(std::integral_constant<int, 4>{});
+      fence();
+      mfma_slot(5);
+      frag(2);
+      gather2(J0{}, I2{});
+      piece(J0{}, I0{});
+      dma(std::integral_constant<int, 5>{});
+      fence();
+      mfma_slot(6);
+      frag(3);
+      gather2(J1{}, I2{});
+      piece(J1{}, I0{});
+      dma(std::integral_constant<int, 6>{});
+      fence();
+      mfma_slot(7);
+      frag(4);
+      piece(J0{}, I1{});
+      dma(std::integral_constant<int, 7>{});
+      fence();
+      mfma_slot(8);
+      frag(5);
+      gather2(J0{}, I3{});
+      piece(J1{}, I1{});
+      dma(std::integral_constant<int, 8>{});
+      fence();
+      mfma_slot(9);
+      frag(6);
+      gather2(J1{}, I3{});
+      dma(std::integral_constant<int, 9>{});
+      fence();
+      mfma_slot(10);
+      frag(7);
+      piece(J0{}, I2{});
+      dma(std::integral_constant<int, 10>{});
+      fence();
+      mfma_slot(11);
+      piece(J1{}, I2{});
+      dma(std::integral_constant<int, 11>{});
+      fence();
+      mfma_slot(12);
+      dma(std::integral_constant<int, 12>{});
+      dma(std::integral_constant<int, 13>{});
+      fence();
+      mfma_slot(13);
+      dma(std::integral_constant<int, 14>{});
+      dma(std::integral_constant<int, 15>{});
+      fence();
+      mfma_slot(14);
+      piece(J0{}, I3{});
+      dma(std::integral_constant<int, 16>{});
+      fence();
+      mfma_slot(15);
+      piece(J1{}, I3{});
+      fence();
+    };
     auto step = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c, int st_next, auto lb_c) {
       if constexpr (CODEBOOK) {
-        prefetch_a(nb_c, nt_c, nx_c);
-        mfma_half(cur_c, I0{});
-        interleave_a();
-        prefetch_b(nx_c);
-        mfma_half(cur_c, I1{});
-        interleave_b(vmem_c);
+        step_codebook(nb_c, nt_c, nx_c, cur_c, vmem_c, st_next, lb_c);
       } else {
         step_affine(nb_c, nt_c, nx_c, cur_c, vmem_c, st_next, lb_c);
       }
@@ -414,7 +480,6 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
       __builtin_amdgcn_s_waitcnt(WAIT_VM0);
       __syncthreads();
       const int st_next = min(s + 2, n_stages - 1);
-      if constexpr (CODEBOOK) load_stage(st_next, sb_c);  // spread under phase b by the group barriers
       step(S1{}, I0{}, I0{}, I1{}, WithVmem{}, st_next, sb_c);
     };
 
