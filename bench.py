@@ -394,51 +394,59 @@ def time_steps(step, steps, warmup):
 # --------------------------------------------------------------------------------------------------
 # the other configurations of the baseline description: MLP forward + backward only, timed for reference
 # --------------------------------------------------------------------------------------------------
-def other_configs(device, dtype, mlp_layer, steps=10, warmup=3):
+def _timed_mlp(op, mlp, M, H, I, r, note, device, dtype, steps, warmup, launch_timing=False):
+    import torch
+
+    gen = torch.Generator(device=device).manual_seed(2)
+    x = torch.randn(M, H, generator=gen, device=device).to(dtype).requires_grad_(True)
+    dy = torch.randn(M, H, generator=gen, device=device).to(dtype)
+    params = [p for p in mlp.parameters() if p.requires_grad]
+
+    def step():
+        for t in (x, *params):
+            t.grad = None
+        op(mlp, x).backward(dy)
+
+    dt = time_steps(step, steps, warmup)
+    fl = mlp_flops(M, H, I, r)
+    out = {"ms_per_step": dt * 1e3, "tokens_per_s": M / dt, "tflops": fl / dt / 1e12,
+           "frac_bf16_mfma_peak": fl / dt / 1e12 / PEAK_BF16_TFLOPS, "workload": note}
+    if launch_timing:
+        with LaunchTimer(M) as timer:
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+        out["kernels"] = {k: {"ms": v[0], "tflops": v[1] / v[0] / 1e9} for k, v in timer.summary().items()}
+    return out
+
+
+def build_act_order_mlp(device, shared):
+    """Config 4: Llama-2-70B MLP shape, desc_act GPTQ: g_idx is a seeded random permutation of the group assignments
+    along K; act-order GPTQ gives projections quantised on the same input one permutation (`shared`), the description
+    draws one each."""
+    import torch
+
+    from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_mlp
+
+    H, I, r, alpha = 8192, 28672, 64, 128.0
+    gen = torch.Generator(device=device).manual_seed(0)
+    mlp = torch.nn.Module()
+    for i, (name, K, N) in enumerate((("gate_proj", H, I), ("up_proj", H, I), ("down_proj", I, H))):
+        pseed = 1234 + K if shared else 40 + i
+        perm = torch.randperm(K, generator=torch.Generator().manual_seed(pseed))
+        g_idx = (torch.arange(K) // GROUP)[perm].to(torch.int32).to(device)
+        setattr(mlp, name, _lora_gptq(K, N, r, alpha, gen, device, 20 + i, g_idx=g_idx))
+    note = ("LoRA_MLP fwd+bwd, 4096 tokens, 8192<->28672, GPTQ g128 desc_act, r=64, "
+            + ("gate and up share their permutation" if shared else "one random permutation per projection"))
+    return apply_lora_mlp, mlp, 4096, H, I, r, note
+
+
+def build_nf4_mlp(device, dtype):
+    """Config 5: Mistral-7B MLP shape, NF4 with double-quantised statistics, 16384 packed tokens."""
     import torch
 
     from fms_acceleration_foak.fused_ops.unsloth_lora.bnb.fast_lora import apply_lora_mlp_swiglu
-    from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_mlp
     from fms_acceleration_peft import Linear4bit, LoraLinear
-
-    def timed(op, mlp, M, H, I, r, note):
-        gen = torch.Generator(device=device).manual_seed(2)
-        x = torch.randn(M, H, generator=gen, device=device).to(dtype).requires_grad_(True)
-        dy = torch.randn(M, H, generator=gen, device=device).to(dtype)
-        params = [p for p in mlp.parameters() if p.requires_grad]
-
-        def step():
-            for t in (x, *params):
-                t.grad = None
-            op(mlp, x).backward(dy)
-
-        dt = time_steps(step, steps, warmup)
-        fl = mlp_flops(M, H, I, r)
-        return {"ms_per_step": dt * 1e3, "tokens_per_s": M / dt, "tflops": fl / dt / 1e12,
-                "frac_bf16_mfma_peak": fl / dt / 1e12 / PEAK_BF16_TFLOPS, "workload": note}
-
-    out = {"config2_llama3_8b_mlp": timed(apply_lora_mlp, mlp_layer, M_TOKENS, HIDDEN, INTER, RANK,
-                                           "LoRA_MLP fwd+bwd, 8192 tokens, 4096<->14336, GPTQ g128, r=16")}
-
-    def act_order_mlp(shared):
-        H, I, r, alpha = 8192, 28672, 64, 128.0
-        gen = torch.Generator(device=device).manual_seed(0)
-        mlp = torch.nn.Module()
-        for i, (name, K, N) in enumerate((("gate_proj", H, I), ("up_proj", H, I), ("down_proj", I, H))):
-            # desc_act: g_idx is a seeded random permutation of the group assignments along K; act-order GPTQ gives
-            # projections quantised on the same input one permutation (`shared`), the description draws one each
-            pseed = 1234 + K if shared else 40 + i
-            perm = torch.randperm(K, generator=torch.Generator().manual_seed(pseed))
-            g_idx = (torch.arange(K) // GROUP)[perm].to(torch.int32).to(device)
-            setattr(mlp, name, _lora_gptq(K, N, r, alpha, gen, device, 20 + i, g_idx=g_idx))
-        return timed(apply_lora_mlp, mlp, 4096, H, I, r,
-                     "LoRA_MLP fwd+bwd, 4096 tokens, 8192<->28672, GPTQ g128 desc_act, r=64, "
-                     + ("gate and up share their permutation" if shared else "one random permutation per projection"))
-
-    out["config4_llama2_70b_mlp_act_order"] = act_order_mlp(False)
-    torch.cuda.empty_cache()
-    out["config4_shared_permutation"] = act_order_mlp(True)
-    torch.cuda.empty_cache()
 
     H, I, r, alpha = 4096, 14336, 8, 16.0
     gen = torch.Generator(device=device).manual_seed(0)
@@ -449,8 +457,23 @@ def other_configs(device, dtype, mlp_layer, steps=10, warmup=3):
         lin.lora_B["default"].weight.data.copy_(torch.randn(N, r, generator=torch.Generator().manual_seed(30 + i)) * 0.02)
         setattr(mlp, name, lin)
         del W
-    out["config5_mistral_7b_mlp_nf4"] = timed(apply_lora_mlp_swiglu, mlp, 16384, H, I, r,
-                                              "LoRA_MLP fwd+bwd, 16384 packed tokens, 4096<->14336, NF4 b64 + 8-bit absmax b256, r=8")
+    return (apply_lora_mlp_swiglu, mlp, 16384, H, I, r,
+            "LoRA_MLP fwd+bwd, 16384 packed tokens, 4096<->14336, NF4 b64 + 8-bit absmax b256, r=8")
+
+
+def other_configs(device, dtype, mlp_layer, steps=10, warmup=3):
+    import torch
+
+    from fms_acceleration_foak.fused_ops.unsloth_lora.gptq.fast_lora import apply_lora_mlp
+
+    out = {"config2_llama3_8b_mlp": _timed_mlp(apply_lora_mlp, mlp_layer, M_TOKENS, HIDDEN, INTER, RANK,
+                                               "LoRA_MLP fwd+bwd, 8192 tokens, 4096<->14336, GPTQ g128, r=16",
+                                               device, dtype, steps, warmup)}
+    out["config4_llama2_70b_mlp_act_order"] = _timed_mlp(*build_act_order_mlp(device, False), device, dtype, steps, warmup)
+    torch.cuda.empty_cache()
+    out["config4_shared_permutation"] = _timed_mlp(*build_act_order_mlp(device, True), device, dtype, steps, warmup)
+    torch.cuda.empty_cache()
+    out["config5_mistral_7b_mlp_nf4"] = _timed_mlp(*build_nf4_mlp(device, dtype), device, dtype, steps, warmup)
     return out
 
 
@@ -620,6 +643,9 @@ def main():
                     help="skip the CPU baseline; the parity gate then checks a sample of token rows instead of every token")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true")
+    ap.add_argument("--workload", default="layer", choices=["layer", "layer_fp16", "config4", "config4_shared", "config5"],
+                    help="profiling runs: time ONE of the other workloads (its own JSON line: step time and per-launch figures; "
+                         "parity of these is the business of tests/test_gpu_full_size.py) instead of the headline layer")
     ap.add_argument("--no-parity", action="store_true", help="profiling runs only: skip the parity gate (the line says so)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one device copy of 1 GiB (a kernel of known traffic, for scaling "
@@ -641,6 +667,17 @@ def main():
     device, dtype, M = torch.device("cuda:0"), torch.bfloat16, args.tokens
     if args.yardsticks:
         print(json.dumps({"yardsticks": yardsticks(device), "peak_bf16_tflops": PEAK_BF16_TFLOPS}))
+        return
+
+    if args.workload != "layer":
+        if args.workload == "layer_fp16":
+            attn, mlp = build_layer(device)
+            out = fp16_layer_config(device, attn, mlp, M, args.steps, args.warmup)
+        else:
+            built = (build_nf4_mlp(device, dtype) if args.workload == "config5"
+                     else build_act_order_mlp(device, args.workload == "config4_shared"))
+            out = _timed_mlp(*built, device, dtype, args.steps, args.warmup, launch_timing=not args.no_kernel_timing)
+        print(json.dumps({"workload_only": args.workload, **out}))
         return
 
     attn, mlp = build_layer(device)
