@@ -475,17 +475,115 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
       interleave(vmem_c);
     }
   };
+  // The affine step (one scale group per stage) written slot by slot, as the input-gradient kernel on the transposed
+  // twin does: the 16 MFMAs of parity `cur`, behind each one its share of the work that produces step (nb, nt) into
+  // parity `nx` -- a fragment read behind the first eight, one unpacked fragment register (2 conversions, 2
+  // multiply-adds, 1 packed conversion) behind every even one -- and, in the last step of a stage, the 20 loads of
+  // stage `st_next` into buffer / slot `lb`.  A scheduling fence closes every slot: the order below is the schedule
+  // (about 1 % faster than what the group-barrier matcher makes of the same step; the fragment reads spread over the
+  // odd slots instead measured no gain).
+  constexpr bool HAND = CODEBOOK == 0 && GPS == 1;
+  // load number `idx` of stage `st` into slot SB (GPS == 1, affine): 0-7 the X tile (direct loads), 8-15 the weight
+  // words (idx - 8 = 4 j + t), 16-17 scale and zero word of column tile 0, 18-19 of column tile 1
+  auto load_piece = [&](int st, auto sb_c, auto idx_c) {
+    constexpr int SB = decltype(sb_c)::value;
+    constexpr int idx = decltype(idx_c)::value;
+    if constexpr (idx < 8) {
+      uint32_t poison = 0u;
+      if constexpr (KTAIL) poison = ((st * BK + 8 * (chunk_even ^ (4 * (idx & 1)))) < K) ? 0u : 0x80000000u;
+      char* lw = lds_buf(sb_c) + uwave * (64 * BK * 2);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (__attribute__((address_space(3))) void*)(lw + idx * (8 * BK * 2)), 16,
+                                               x_off[idx] | poison, (uint32_t)st * (BK * 2), 0, 0);
+    } else if constexpr (idx < 16) {
+      constexpr int j = (idx - 8) >> 2, t = (idx - 8) & 3;
+      uint32_t so = (uint32_t)st * q_stage_bytes[j] + t * q_step_bytes[j];
+      if constexpr (KTAIL) so = min(so, q_last[j]);
+      qw[SB][j][t] = __builtin_amdgcn_raw_buffer_load_b32(q_rsrc[j], q_off[j], so, 0);
+    } else {
+      constexpr int j = (idx - 16) >> 1;
+      const int gu = __builtin_amdgcn_readfirstlane(min(g_ld[j], n_groups_j[j] - 1));
+      if constexpr (((idx - 16) & 1) == 0) {
+        sc_raw[SB][j][0] = __builtin_amdgcn_raw_buffer_load_b16(sc_rsrc[j], sc_off[j], (uint32_t)gu * Np[j] * 2, 0);
+      } else {
+        zw_raw[SB][j][0] = __builtin_amdgcn_raw_buffer_load_b32(z_rsrc[j], z_off[j], (uint32_t)gu * (Np[j] >> 3) * 4, 0);
+        k_in_g[j] += BK;  // uniform scalar bookkeeping, no division
+        const bool wrap = k_in_g[j] >= gs[j];
+        k_in_g[j] -= wrap ? gs[j] : 0;
+        g_ld[j] += wrap ? 1 : 0;
+      }
+    }
+  };
+  auto step_affine = [&](auto nb_c, auto nt_c, auto nx_c, auto cur_c, auto vmem_c, int st_next, auto lb_c) {
+    constexpr int SB = decltype(nb_c)::value;
+    constexpr int t = decltype(nt_c)::value;
+    constexpr int par = decltype(nx_c)::value;
+    constexpr int cur = decltype(cur_c)::value;
+    constexpr bool with_vmem = decltype(vmem_c)::value;
+    const char* lr = lds_buf(nb_c) + lds_r_off[t];
+    auto mfma_slot = [&](int slot) { acc[slot >> 1][slot & 1] = mfma32<T>(wf[cur][slot & 1], xf[cur][slot >> 1], acc[slot >> 1][slot & 1]); };
+    auto frag = [&](int mt) { xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2); };
+    auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+    auto dma = [&](auto idx_c) {
+      if constexpr (with_vmem) load_piece(st_next, lb_c, idx_c);
+    };
+    uint32_t nib[NT][2];  // [tile][0]: nibbles 0, 2, 4, 6 in bytes 0..3; [1]: 16 * nibbles 1, 3, 5, 7 (the scale is pre-divided)
+    auto masks = [&](auto j_c) {
+      constexpr int j = decltype(j_c)::value;
+      nib[j][0] = opaque(qw[SB][j][t] & 0x0F0F0F0Fu);
+      nib[j][1] = opaque(qw[SB][j][t] & 0xF0F0F0F0u);
+    };
+    auto piece = [&](auto j_c, auto reg_c) {
+      constexpr int j = decltype(j_c)::value;
+      constexpr int reg = decltype(reg_c)::value;
+      float b0, b1;
+      if constexpr (reg == 0) {
+        b0 = ubyte0(nib[j][0]);
+        b1 = ubyte0(nib[j][1]);
+      } else if constexpr (reg == 1) {
+        b0 = ubyte1(nib[j][0]);
+        b1 = ubyte1(nib[j][1]);
+      } else if constexpr (reg == 2) {
+        b0 = ubyte2(nib[j][0]);
+        b1 = ubyte2(nib[j][1]);
+      } else {
+        b0 = ubyte3(nib[j][0]);
+        b1 = ubyte3(nib[j][1]);
+      }
+      wf[par][j][reg] = pack2<T>(__builtin_fmaf(sf[j][0], b0, nsz[j][0]), __builtin_fmaf(sf16[j][0], b1, nsz[j][0]));
+    };
+    static_for<0, 16>([&](auto u_c) {
+      constexpr int u = decltype(u_c)::value;
+      mfma_slot(u);
+      if constexpr (u == 0) masks(std::integral_constant<int, 0>{});
+      if constexpr (u == 8) masks(std::integral_constant<int, 1>{});
+      if constexpr ((u & 1) == 0) piece(std::integral_constant<int, (u >> 3)>{}, std::integral_constant<int, ((u >> 1) & 3)>{});
+      if constexpr (u < 8) frag(u);
+      dma(std::integral_constant<int, u>{});
+      if constexpr (u >= 12) dma(std::integral_constant<int, 4 + u>{});  // loads 16-19: scales and zero words
+      fence();
+    });
+  };
   auto stage = [&](int s, auto sb_c) {
     constexpr int SB = decltype(sb_c)::value;
     using S1 = std::integral_constant<int, SB ^ 1>;
-    step(sb_c, I1{}, I1{}, I0{}, NoVmem{});
-    step(sb_c, I2{}, I0{}, I1{}, NoVmem{});
-    step(sb_c, I3{}, I1{}, I0{}, NoVmem{});
+    if constexpr (HAND) {
+      step_affine(sb_c, I1{}, I1{}, I0{}, NoVmem{}, 0, sb_c);
+      step_affine(sb_c, I2{}, I0{}, I1{}, NoVmem{}, 0, sb_c);
+      step_affine(sb_c, I3{}, I1{}, I0{}, NoVmem{}, 0, sb_c);
+    } else {
+      step(sb_c, I1{}, I1{}, I0{}, NoVmem{});
+      step(sb_c, I2{}, I0{}, I1{}, NoVmem{});
+      step(sb_c, I3{}, I1{}, I0{}, NoVmem{});
+    }
     __builtin_amdgcn_s_waitcnt(WAIT_VM0);
     commit_stage(S1{});
     __syncthreads();
-    load_stage(min(s + 2, n_stages - 1), sb_c);
-    step(S1{}, I0{}, I0{}, I1{}, WithVmem{});
+    if constexpr (HAND) {
+      step_affine(S1{}, I0{}, I0{}, I1{}, WithVmem{}, min(s + 2, n_stages - 1), sb_c);
+    } else {
+      load_stage(min(s + 2, n_stages - 1), sb_c);
+      step(S1{}, I0{}, I0{}, I1{}, WithVmem{});
+    }
   };
 
   // LoRA operands of ranks 0..15 (the whole adapter up to rank 16): direct loads into the epilogue planes,
