@@ -1,7 +1,7 @@
 """Collects the rocprofv3 evidence for the fused kernels and reduces it to the short summaries under profiles/.
 
-    python bench_profiles.py collect      (on the MI355X box; raw output under gpurun_out/prof_*)
-    python bench_profiles.py summarize    (reads gpurun_out/prof_*, writes profiles/*.txt)
+    python bench_profiles.py collect      (on the MI355X; raw profiler output goes to RAW/prof_*)
+    python bench_profiles.py summarize    (reads RAW/prof_*, writes profiles/*.txt)
 
 Every profiler run is a child process of its own (`rocprofv3 ... -- python3 bench.py ...`), one counter set per run;
 the commands are repeated at the top of each summary.  Summaries are named for the kernels and workload they cover.
