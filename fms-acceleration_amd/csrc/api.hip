@@ -23,8 +23,9 @@ int launch_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int m
 
 int launch_gptq_lora_bwd_dx_t(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx, void* e,
                               void* g, void* h_out, int64_t ldeg, int act_dtype, hipStream_t st);
-bool bwd_dx_twin_applies(const fmsa_bwd_proj* projs, int n_proj);
+int bwd_dx_twin_flavour(const fmsa_bwd_proj* projs, int n_proj, int act_dtype);
 int launch_gptq_transpose(const int32_t* qweight, int K, int N, int32_t* out, hipStream_t st);
+int launch_gptq_interleave(const int32_t* qweight, int K, int N, int32_t* out, hipStream_t st);
 int launch_gptq_nsz(const fmsa_gptq_weight* w, float* out, hipStream_t st);
 int launch_lora_pack_batch(const fmsa_lora_pack_job* jobs, int n_jobs, int act_dtype, hipStream_t st);
 int launch_rms_fwd(const void* X, int64_t ldx, const void* W, int M, int C, float eps, int gemma, int x_dtype, int w_dtype, void* Y,
@@ -51,8 +52,10 @@ namespace {
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool is_act(int d) { return d == FMSA_BF16 || d == FMSA_F16; }
 
-int check_weight(const fmsa_gptq_weight* w, int group_multiple) {
+int check_weight(const fmsa_gptq_weight* w, int group_multiple, bool interleaved_ok = false) {
   if (w->format != FMSA_WEIGHT_AFFINE && w->format != FMSA_WEIGHT_CODEBOOK) return FMSA_ERR_SHAPE;
+  if (w->nibble_order != 0 && w->nibble_order != 1) return FMSA_ERR_SHAPE;
+  if (w->nibble_order == 1 && (!interleaved_ok || w->format != FMSA_WEIGHT_AFFINE || w->group_size % 64 != 0)) return FMSA_ERR_UNSUPPORTED;
   if (!w->qweight) return FMSA_ERR_NULL;
   if (w->K <= 0 || w->N <= 0 || w->group_size <= 0) return FMSA_ERR_SHAPE;
   if (w->K % 32 != 0 || w->N % 32 != 0) return FMSA_ERR_SHAPE;  // qlinear_tritonv2.py:57-60
@@ -265,8 +268,10 @@ static int check_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, int6
   if (!aligned16(X) || ldx % 8 != 0) return FMSA_ERR_ALIGN;
   for (int p = 0; p < n_proj; ++p) {
     const fmsa_fwd_proj& s = projs[p];
-    if (int rc = check_weight(&s.w, 16)) return rc;
-    if (s.w.format != projs[0].w.format) return FMSA_ERR_UNSUPPORTED;  // one kernel flavour per launch
+    // the interleaved nibble order belongs to the packed-half unpack: fp16 activations (and no rotary epilogue, which
+    // fmsa_gptq_lora_fwd_rope checks)
+    if (int rc = check_weight(&s.w, 16, act_dtype == FMSA_F16)) return rc;
+    if (s.w.format != projs[0].w.format || s.w.nibble_order != projs[0].w.nibble_order) return FMSA_ERR_UNSUPPORTED;  // one kernel flavour per launch
     if (s.w.K != K) return FMSA_ERR_SHAPE;
     if (!s.Y) return FMSA_ERR_NULL;
     if (s.ldy < s.w.N) return FMSA_ERR_SHAPE;
@@ -312,6 +317,7 @@ int fmsa_gptq_lora_fwd_rope(const fmsa_fwd_proj* projs, int n_proj, const void* 
   for (int p = 0; p < n_proj; ++p) {
     if (((rope->proj_mask >> p) & 1) && projs[p].w.N % hd != 0) return FMSA_ERR_SHAPE;
     if (projs[p].w.group_size <= 0 || projs[p].w.group_size % 64 != 0) return FMSA_ERR_UNSUPPORTED;
+    if (projs[p].w.nibble_order != 0) return FMSA_ERR_UNSUPPORTED;  // the rotating flavours read the checkpoint's order
   }
   if (K % 64 != 0) return FMSA_ERR_UNSUPPORTED;
   return launch_gptq_lora_fwd(projs, n_proj, X, ldx, M, FMSA_FWD_LINEAR, nullptr, 0, rope, act_dtype, (hipStream_t)stream);
@@ -332,7 +338,9 @@ int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mod
     if (s.w.format != projs[0].w.format) return FMSA_ERR_UNSUPPORTED;  // one kernel flavour per launch
     if (s.w.group_size < 32) return FMSA_ERR_UNSUPPORTED;  // at most 8 groups per 256 output columns
     if (s.w.K != K) return FMSA_ERR_SHAPE;
-    if (!s.dY || (!s.nsz && s.w.format != FMSA_WEIGHT_CODEBOOK)) return FMSA_ERR_NULL;
+    // the offset table: fp32 -s*z, or (fp16 activations on the transposed twin) the fp16 -(1024 + z) table alone
+    if (!s.dY) return FMSA_ERR_NULL;
+    if (s.negzp_f16 && !aligned16(s.negzp_f16)) return FMSA_ERR_ALIGN;
     if (s.lddy < s.w.N) return FMSA_ERR_SHAPE;
     if (s.nsz && !aligned16(s.nsz)) return FMSA_ERR_ALIGN;
     if ((s.qweight_t && !aligned16(s.qweight_t)) || (s.scale_f32 && !aligned16(s.scale_f32))) return FMSA_ERR_ALIGN;
@@ -362,9 +370,21 @@ int fmsa_gptq_lora_bwd_dx(const fmsa_bwd_proj* projs, int n_proj, int M, int mod
     if (lddx < K) return FMSA_ERR_SHAPE;
     if (!aligned16(dX) || lddx % 8 != 0) return FMSA_ERR_ALIGN;
   }
-  if (bwd_dx_twin_applies(projs, n_proj))
+  const int twin = bwd_dx_twin_flavour(projs, n_proj, act_dtype);
+  // the checkpoint-layout kernel needs every affine projection's fp32 offset table
+  if (!twin)
+    for (int p = 0; p < n_proj; ++p)
+      if (!projs[p].nsz && projs[p].w.format != FMSA_WEIGHT_CODEBOOK) return FMSA_ERR_NULL;
+  if (twin)
     return launch_gptq_lora_bwd_dx_t(projs, n_proj, M, mode, dX, lddx, e, g, h_out, ldeg, act_dtype, (hipStream_t)stream);
   return launch_gptq_lora_bwd_dx(projs, n_proj, M, mode, dX, lddx, e, g, h_out, ldeg, act_dtype, (hipStream_t)stream);
+}
+
+int fmsa_gptq_interleave(const int32_t* qweight, int K, int N, int32_t* qweight_out, void* stream) {
+  if (!qweight || !qweight_out) return FMSA_ERR_NULL;
+  if (K <= 0 || N <= 0 || K % 8 != 0 || N % 4 != 0) return FMSA_ERR_SHAPE;
+  if (!aligned16(qweight) || !aligned16(qweight_out)) return FMSA_ERR_ALIGN;
+  return launch_gptq_interleave(qweight, K, N, qweight_out, (hipStream_t)stream);
 }
 
 int fmsa_gptq_transpose(const int32_t* qweight, int K, int N, int32_t* qweight_t_out, void* stream) {

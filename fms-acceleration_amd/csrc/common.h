@@ -63,6 +63,12 @@ FMSA_DEVI float ubyte0(uint32_t x) { return (float)(x & 0xffu); }
 FMSA_DEVI float ubyte1(uint32_t x) { return (float)((x >> 8) & 0xffu); }
 FMSA_DEVI float ubyte2(uint32_t x) { return (float)((x >> 16) & 0xffu); }
 FMSA_DEVI float ubyte3(uint32_t x) { return (float)(x >> 24); }
+template <int B> FMSA_DEVI float ubyte_n(uint32_t x) {
+  if constexpr (B == 0) return ubyte0(x);
+  else if constexpr (B == 1) return ubyte1(x);
+  else if constexpr (B == 2) return ubyte2(x);
+  else return ubyte3(x);
+}
 // Stops the optimiser from narrowing the byte masks above back into nibble masks (which would
 // cost a shift + and + convert per value instead of one convert).  Emits no instruction.
 FMSA_DEVI uint32_t opaque(uint32_t x) {
@@ -85,6 +91,15 @@ template <typename T> FMSA_DEVI u32x4 dequant8(uint32_t w, float sf, float sf16,
   r[2] = pack2<T>(__builtin_fmaf(sf, ubyte2(lo), nsz), __builtin_fmaf(sf16, ubyte2(hi), nsz));
   r[3] = pack2<T>(__builtin_fmaf(sf, ubyte3(lo), nsz), __builtin_fmaf(sf16, ubyte3(hi), nsz));
   return r;
+}
+
+// ---- packed half arithmetic (fp16 only: v_pk_add_f16 / v_pk_mul_f16; fp32 packed forms stay switched off) ----------
+// (1024 + q) - (1024 + z) is exact in fp16 and the product with the fp16 scale rounds once: RNE_fp16(s * (q - z)), the
+// value of UL/gptq/triton/kernels.py:118-122 bit for bit, two weights per instruction.
+FMSA_DEVI uint32_t pk_sub_mul_f16(uint32_t q_plus_1024, uint32_t neg_z_plus_1024, uint32_t scale) {
+  const f16x2 a = __builtin_bit_cast(f16x2, q_plus_1024), b = __builtin_bit_cast(f16x2, neg_z_plus_1024);
+  const f16x2 d = a + b;
+  return __builtin_bit_cast(uint32_t, d * __builtin_bit_cast(f16x2, scale));
 }
 
 // ---- MFMA 32x32x16: D[i][j] += sum_k A[i][k] * B[k][j] ---------------------------------------

@@ -3,8 +3,11 @@
 //
 // The checkpoint packs 8 nibbles along K into one word, which is the forward's contraction axis; the input
 // gradient contracts over N.  The twin (built once per frozen weight by gptq_transpose below) packs along N:
-//   qweight_t int32 [N/8, K]   nibble j of word [n8, k] = q[k, 8*n8 + j]
-// so one word is again exactly the 8-element MFMA fragment of the lane that owns output column k, and this
+//   qweight_t int32 [N/8, K]   word [n8, k] holds q[k, 8*n8 + e], e = 0..7, with the even elements in its low half
+//                              (element 2p at nibble position p) and the odd ones in its high half (2p + 1 at 4 + p)
+// so one word is again exactly the 8-element MFMA fragment of the lane that owns output column k (the interleaved
+// order costs the byte-wise unpack nothing and lets (w >> 4r) & 0x000F000F pick the pair of fragment register r for
+// the packed-half unpack of the fp16 flavour), and this
 // kernel is the forward kernel with the roles of K and N exchanged: every lane loads its own words into
 // registers and unpacks them there (no byte shuffles, no words staged through LDS), and an accumulator quad
 // holds 4 ADJACENT output columns, so the epilogue's dump is the forward's (8-byte LDS writes).
@@ -13,6 +16,9 @@
 // for all lanes of a half wave (group_size % 64 == 0: the wave's 64 columns lie in one group), and come from a
 // per-stage table in LDS (fp32 scale [groups of the tile][64], fp32 -scale*zero likewise; filled by direct loads,
 // one per wave and stage) by broadcast reads: 4 reads of 16 bytes per 16-wide step.
+// PK16 (fp16 activations, affine weights): the tables are the checkpoint's fp16 scales and fp16 -(1024 + zero), and a
+// fragment register is (((w >> 4r) & 0x000F000F) | 0x64006400) + (-(1024 + z)) [exact] times the scale [one rounding]
+// in packed half arithmetic: 15 instead of 23 instructions per word, 2 table reads per step instead of 4, same bits.
 //
 // Tiling as in the forward: workgroup = 4 waves = 256 tokens x 256 output columns, wave = 256 x 64 (8 x 2 MFMA
 // 32x32x16 tiles), contraction walked in stages of 64 with the dY tile loaded global -> LDS directly, one stage
@@ -34,6 +40,8 @@ struct BwdTProjDev {
   const int32_t* qt;   // [N/8, K]
   const float* sc;     // [G, N] fp32 scales (affine) / block scales (code book)
   const float* nsz;    // [G, N] fp32 -scale * (zero + zero_offset) (affine only)
+  const uint16_t* sc16;  // PK16: [G, N] fp16 scales (the checkpoint's own)
+  const uint16_t* nz16;  // PK16: [G, N] fp16 -(1024 + zero + zero_offset)
   const float* code;   // code-book format: 16 entries
   const uint16_t* dY;
   int64_t lddy;
@@ -60,13 +68,14 @@ struct BwdTArgs {
 FMSA_DEVI BwdTProjDev select_proj(const BwdTArgs& a, int p) { return p == 0 ? a.p[0] : (p == 1 ? a.p[1] : a.p[2]); }
 
 // CODEBOOK: W = code[q] * block_scale[group, n] instead of the affine scale * q + (-scale * zero).
-template <typename T, bool NTAIL, int MODE, bool CODEBOOK>
+template <typename T, bool NTAIL, int MODE, bool CODEBOOK, bool PK16 = false>
 __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs a) {
+  static_assert(!PK16 || (std::is_same<T, f16_t>::value && !CODEBOOK), "packed half unpack: fp16 activations, affine weights");
   // separate arrays per stage buffer: every access names its buffer statically, so the compiler can tell fragment
   // reads of one buffer from the direct loads in flight into the other
   __shared__ __attribute__((aligned(1024))) uint16_t dy0[BM * BK];
   __shared__ __attribute__((aligned(1024))) uint16_t dy1[BM * BK];
-  // per buffer 4 KB: scales [8][64] fp32 | offsets [8][64] fp32
+  // per buffer 4 KB: scales [8][64] fp32 | offsets [8][64] fp32 (PK16: fp16 scales [8][64] | fp16 offsets [8][64], 2 KB used)
   __shared__ __attribute__((aligned(1024))) uint32_t tb0[1024];
   __shared__ __attribute__((aligned(1024))) uint32_t tb1[1024];
   __shared__ __attribute__((aligned(16))) uint16_t ep_planes[2 * EP_ROWS * EP_STRIDE];
@@ -141,13 +150,20 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
     // tables: waves 0, 1 load the scales of groups 0-3 / 4-7 of the tile, waves 2, 3 the offsets (lane q: group
     // q >> 4, 4-column chunk q & 15): one load per wave and stage.  The code-book format has no offsets (its
     // resource is empty: no traffic).
+    // PK16: 1 KB each, wave 0 loads the scales, wave 1 the offsets (lane q: group q >> 3, 8-column chunk q & 7), waves
+    // 2 and 3 issue the same instruction on an empty resource.
     const int g0 = k_tile0 / gs;
-    const int tb_g = 4 * (wave & 1) + (lane >> 4);
-    const int tb_col = 4 * (lane & 15);
-    const __amdgpu_buffer_rsrc_t sc_rsrc = make_rsrc(P.sc, (size_t)n_groups * N * 4);
-    const __amdgpu_buffer_rsrc_t nz_rsrc = make_rsrc(P.nsz, CODEBOOK ? 0 : (size_t)n_groups * N * 4);
-    const __amdgpu_buffer_rsrc_t tb_rsrc = (wave < 2) ? sc_rsrc : nz_rsrc;
-    const uint32_t tb_off = (uint32_t)(((g0 + tb_g) * N + tb_col) * 4) | ((g0 + tb_g) < n_groups ? 0u : 0x80000000u);
+    constexpr int TB_ELEM = PK16 ? 2 : 4;  // bytes per table element
+    const int tb_g = PK16 ? (lane >> 3) : 4 * (wave & 1) + (lane >> 4);
+    const int tb_col = PK16 ? 8 * (lane & 7) : 4 * (lane & 15);
+    const __amdgpu_buffer_rsrc_t sc_rsrc = PK16 ? make_rsrc(P.sc16, wave == 0 ? (size_t)n_groups * N * 2 : 0)
+                                                : make_rsrc(P.sc, (size_t)n_groups * N * 4);
+    const __amdgpu_buffer_rsrc_t nz_rsrc = PK16 ? make_rsrc(P.nz16, wave == 1 ? (size_t)n_groups * N * 2 : 0)
+                                                : make_rsrc(P.nsz, CODEBOOK ? 0 : (size_t)n_groups * N * 4);
+    const __amdgpu_buffer_rsrc_t tb_rsrc = PK16 ? ((wave == 0) ? sc_rsrc : nz_rsrc) : ((wave < 2) ? sc_rsrc : nz_rsrc);
+    const uint32_t tb_off = (uint32_t)(((g0 + tb_g) * N + tb_col) * TB_ELEM) | ((g0 + tb_g) < n_groups ? 0u : 0x80000000u);
+    constexpr int TB_ZOFF = PK16 ? 1024 : 2048;   // byte offset of the offsets inside a table buffer
+    constexpr int TB_STEP = 16 * TB_ELEM;         // bytes of one group's row per 16-wide step
     // weights: word (n8, k) at (n8 * K + k) * 4; the lane part is (half * K + k) * 4
     const __amdgpu_buffer_rsrc_t q_rsrc = make_rsrc(P.qt, (size_t)(N >> 3) * K * 4);
     uint32_t q_off[NT];
@@ -156,7 +172,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
     // the wave's group inside the tile (its 64 columns lie in one group: group_size % 64 == 0), and the table read
     // offset (bytes): [group][16 t + 8 half ..]
     const int gl = min(max(col0[0] / gs - g0, 0), TB_GROUPS - 1);
-    const uint32_t tb_r = (uint32_t)(gl * (BK * 4) + 8 * half * 4);
+    const uint32_t tb_r = (uint32_t)(gl * (BK * TB_ELEM) + 8 * half * TB_ELEM);
     const uint32_t q_step_bytes = (uint32_t)K * 8;    // two packed rows per 16-wide step
     const uint32_t q_stage_bytes = (uint32_t)K * 32;  // eight packed rows per stage
     const uint32_t q_last = (uint32_t)((N >> 3) - 2) * K * 4;
@@ -181,7 +197,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
         uint32_t poison = 0u;
         if constexpr (NTAIL) poison = ((int)n0 + tb_col < N) ? 0u : 0x80000000u;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(tb_rsrc, (__attribute__((address_space(3))) void*)(tb_buf(sb_c) + wave * 1024), 16,
-                                                 tb_off | poison, n0 * 4, 0, 0);
+                                                 tb_off | poison, n0 * TB_ELEM, 0, 0);
       } else {
         constexpr int j = (idx - 9) >> 2, t = (idx - 9) & 3;
         uint32_t so = (uint32_t)st * q_stage_bytes + t * q_step_bytes;
@@ -195,37 +211,60 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
 
     // ---- affine: LDS -> registers for step t of buffer SB (8 dY fragments, the step's 8 scales and 8 offsets of each
     // column tile's group) and the two unpacked weight fragments, into parity `par`
+    // fragment register `reg` (contraction elements 2 reg, 2 reg + 1 = columns n + 2 reg, + 1) of a word whose byte
+    // planes are p0 = w & 0x0F0F0F0F (elements 0, 4, 1, 5) and p1 = (w >> 4) & 0x0F0F0F0F (elements 2, 6, 3, 7): bytes
+    // reg >> 1 and (reg >> 1) + 2 of plane reg & 1; value = scale * nibble + (-scale * zero), exact in fp32, one rounding
+    auto unpack_reg = [&](uint32_t p0, uint32_t p1, const u32x4 (&sv)[2], const u32x4 (&zv)[2], auto reg_c) -> uint32_t {
+      constexpr int reg = decltype(reg_c)::value;
+      const uint32_t pl = (reg & 1) ? p1 : p0;
+      const float b0 = ubyte_n<(reg >> 1)>(pl), b1 = ubyte_n<(reg >> 1) + 2>(pl);
+      const float s0 = __uint_as_float(sv[reg >> 1][2 * (reg & 1)]), s1 = __uint_as_float(sv[reg >> 1][2 * (reg & 1) + 1]);
+      const float z0 = __uint_as_float(zv[reg >> 1][2 * (reg & 1)]), z1 = __uint_as_float(zv[reg >> 1][2 * (reg & 1) + 1]);
+      return pack2<T>(__builtin_fmaf(s0, b0, z0), __builtin_fmaf(s1, b1, z1));
+    };
+    // PK16: the pair (1024 + element 2 reg, 1024 + element 2 reg + 1) in packed half precision straight out of the word
+    // (mask and bias sit in vector registers: the three-operand and-or takes no literal and one scalar at most)
+    const uint32_t pk_mask = opaque(0x000F000Fu), pk_bias = opaque(0x64006400u);
+    auto pair16 = [&](uint32_t w, auto reg_c) -> uint32_t {
+      constexpr int reg = decltype(reg_c)::value;
+      return ((w >> (4 * reg)) & pk_mask) | pk_bias;
+    };
+    // ---- affine: LDS -> registers for step t of buffer SB (8 dY fragments, the step's 8 scales and 8 offsets of the
+    // wave's group) and the two unpacked weight fragments, into parity `par` (the very first step of a projection)
     auto prefetch = [&](auto sb_c, auto t_c, auto par_c) {
       constexpr int SB = decltype(sb_c)::value;
       constexpr int t = decltype(t_c)::value;
       constexpr int par = decltype(par_c)::value;
       const char* lt = tb_buf(sb_c);
       const char* lr = dy_buf(sb_c) + dy_r[t];
-      u32x4 sv[2], zv[2];
-      sv[0] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * 64);
-      sv[1] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * 64 + 16);
-      zv[0] = *reinterpret_cast<const u32x4*>(lt + 2048 + tb_r + t * 64);
-      zv[1] = *reinterpret_cast<const u32x4*>(lt + 2048 + tb_r + t * 64 + 16);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2);
+      if constexpr (PK16) {
+        const u32x4 s16 = *reinterpret_cast<const u32x4*>(lt + tb_r + t * TB_STEP);
+        const u32x4 z16 = *reinterpret_cast<const u32x4*>(lt + TB_ZOFF + tb_r + t * TB_STEP);
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        const uint32_t w = qw[SB][j][t];
-        const uint32_t lo = opaque(w & 0x0F0F0F0Fu);         // nibbles 0, 2, 4, 6 in bytes 0..3
-        const uint32_t hi = opaque((w >> 4) & 0x0F0F0F0Fu);  // nibbles 1, 3, 5, 7
-        // fragment register i: contraction elements 2i, 2i+1 = columns n + 2i, n + 2i + 1; value = scale * nibble +
-        // (-scale * zero), exact in fp32, one rounding
-        auto sf = [&](int e) { return __uint_as_float(sv[e >> 2][e & 3]); };
-        auto zf = [&](int e) { return __uint_as_float(zv[e >> 2][e & 3]); };
-        wf[par][j][0] = pack2<T>(__builtin_fmaf(sf(0), ubyte0(lo), zf(0)), __builtin_fmaf(sf(1), ubyte0(hi), zf(1)));
-        wf[par][j][1] = pack2<T>(__builtin_fmaf(sf(2), ubyte1(lo), zf(2)), __builtin_fmaf(sf(3), ubyte1(hi), zf(3)));
-        wf[par][j][2] = pack2<T>(__builtin_fmaf(sf(4), ubyte2(lo), zf(4)), __builtin_fmaf(sf(5), ubyte2(hi), zf(5)));
-        wf[par][j][3] = pack2<T>(__builtin_fmaf(sf(6), ubyte3(lo), zf(6)), __builtin_fmaf(sf(7), ubyte3(hi), zf(7)));
+        for (int j = 0; j < NT; ++j)
+          static_for<0, 4>([&](auto r_c) {
+            constexpr int r = decltype(r_c)::value;
+            wf[par][j][r] = pk_sub_mul_f16(pair16(qw[SB][j][t], r_c), z16[r], s16[r]);
+          });
+      } else {
+        u32x4 sv[2], zv[2];
+        sv[0] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * TB_STEP);
+        sv[1] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * TB_STEP + 16);
+        zv[0] = *reinterpret_cast<const u32x4*>(lt + TB_ZOFF + tb_r + t * TB_STEP);
+        zv[1] = *reinterpret_cast<const u32x4*>(lt + TB_ZOFF + tb_r + t * TB_STEP + 16);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const uint32_t w = qw[SB][j][t];
+          const uint32_t p0 = opaque(w & 0x0F0F0F0Fu), p1 = opaque((w >> 4) & 0x0F0F0F0Fu);
+          static_for<0, 4>([&](auto r_c) { wf[par][j][decltype(r_c)::value] = unpack_reg(p0, p1, sv, zv, r_c); });
+        }
       }
     };
     // ---- code book, two phases so that no gather is waited for right after its issue.  Phase a: fragment reads,
-    // the block scales of the step, and the 16 gathers from the lane-resident table (ds_bpermute; element 2b / 2b+1
-    // of a word in gath[j][b] / [4 + b]); phase b: code * block scale in fp32, one rounding.
+    // the block scales of the step, and the 16 gathers from the lane-resident table (ds_bpermute; the codes of
+    // elements 2b / 2b+1 of a word in gath[j][b] / [4 + b]); phase b: code * block scale in fp32, one rounding.
     uint32_t gath[NT][8];
     u32x4 bsv[2];
     auto prefetch_a = [&](auto sb_c, auto t_c, auto par_c) {
@@ -234,20 +273,22 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
       constexpr int par = decltype(par_c)::value;
       const char* lt = tb_buf(sb_c);
       const char* lr = dy_buf(sb_c) + dy_r[t];
-      bsv[0] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * 64);
-      bsv[1] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * 64 + 16);
+      bsv[0] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * TB_STEP);
+      bsv[1] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * TB_STEP + 16);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) xf[par][mt] = *reinterpret_cast<const u32x4*>(lr + mt * 32 * BK * 2);
       const int li = (int)__float_as_uint(lut);
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
         const uint32_t w = qw[SB][j][t];
-        const uint32_t e = opaque((w << 2) & 0x3C3C3C3Cu);  // byte b: 4 * nibble 2b (a lane's byte address)
-        const uint32_t o = opaque((w >> 2) & 0x3C3C3C3Cu);  // byte b: 4 * nibble 2b+1
+        // byte planes of table addresses (4 * code): a0 = elements 0, 4, 1, 5, a1 = elements 2, 6, 3, 7; fragment
+        // register b takes bytes b >> 1 and (b >> 1) + 2 of plane b & 1
+        const uint32_t a0 = opaque((w << 2) & 0x3C3C3C3Cu), a1 = opaque((w >> 2) & 0x3C3C3C3Cu);
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
-          gath[j][b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((e >> (8 * b)) & 0xffu), li);
-          gath[j][4 + b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((o >> (8 * b)) & 0xffu), li);
+          const uint32_t pl = (b & 1) ? a1 : a0;
+          gath[j][b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((pl >> (8 * (b >> 1))) & 0xffu), li);
+          gath[j][4 + b] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((pl >> (8 * ((b >> 1) + 2))) & 0xffu), li);
         }
       }
     };
@@ -283,20 +324,24 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
       auto dma = [&](auto idx_c) {
         if constexpr (with_vmem) load_piece(st_next, lb_c, idx_c);
       };
-      u32x4 sv[2], zv[2];
-      uint32_t nib[NT][2];  // [tile][0]: nibbles 0, 2, 4, 6 in bytes 0..3; [1]: nibbles 1, 3, 5, 7
+      u32x4 sv[2], zv[2];   // PK16: sv[0] / zv[0] hold the 8 fp16 scales / offsets of the step
+      uint32_t nib[NT][2];  // byte planes of a word: [tile][0] elements 0, 4, 1, 5; [1] elements 2, 6, 3, 7 (unused by PK16)
       mfma_slot(0);
-      sv[0] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * 64);
-      sv[1] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * 64 + 16);
-      nib[0][0] = opaque(qw[SB][0][t] & 0x0F0F0F0Fu);
-      nib[0][1] = opaque((qw[SB][0][t] >> 4) & 0x0F0F0F0Fu);
+      sv[0] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * TB_STEP);
+      if constexpr (!PK16) {
+        sv[1] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * TB_STEP + 16);
+        nib[0][0] = opaque(qw[SB][0][t] & 0x0F0F0F0Fu);
+        nib[0][1] = opaque((qw[SB][0][t] >> 4) & 0x0F0F0F0Fu);
+      }
       dma(std::integral_constant<int, 0>{});
       fence();
       mfma_slot(1);
-      zv[0] = *reinterpret_cast<const u32x4*>(lt + 2048 + tb_r + t * 64);
-      zv[1] = *reinterpret_cast<const u32x4*>(lt + 2048 + tb_r + t * 64 + 16);
-      nib[1][0] = opaque(qw[SB][1][t] & 0x0F0F0F0Fu);
-      nib[1][1] = opaque((qw[SB][1][t] >> 4) & 0x0F0F0F0Fu);
+      zv[0] = *reinterpret_cast<const u32x4*>(lt + TB_ZOFF + tb_r + t * TB_STEP);
+      if constexpr (!PK16) {
+        zv[1] = *reinterpret_cast<const u32x4*>(lt + TB_ZOFF + tb_r + t * TB_STEP + 16);
+        nib[1][0] = opaque(qw[SB][1][t] & 0x0F0F0F0Fu);
+        nib[1][1] = opaque((qw[SB][1][t] >> 4) & 0x0F0F0F0Fu);
+      }
       dma(std::integral_constant<int, 1>{});
       fence();
       mfma_slot(2);
@@ -309,28 +354,14 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
       frag(3);
       dma(std::integral_constant<int, 3>{});
       fence();
-      // fragment register `reg` of tile `j`: contraction elements 2 reg, 2 reg + 1 (columns n + 2 reg, + 1); value =
-      // scale * nibble + (-scale * zero), exact in fp32, one rounding
+      // fragment register `reg` of tile `j` (5 instructions; PK16: 4, the pair straight out of the word)
       auto piece = [&](auto j_c, auto reg_c) {
         constexpr int j = decltype(j_c)::value;
         constexpr int reg = decltype(reg_c)::value;
-        const float s0 = __uint_as_float(sv[reg >> 1][2 * (reg & 1)]), s1 = __uint_as_float(sv[reg >> 1][2 * (reg & 1) + 1]);
-        const float z0 = __uint_as_float(zv[reg >> 1][2 * (reg & 1)]), z1 = __uint_as_float(zv[reg >> 1][2 * (reg & 1) + 1]);
-        float b0, b1;
-        if constexpr (reg == 0) {
-          b0 = ubyte0(nib[j][0]);
-          b1 = ubyte0(nib[j][1]);
-        } else if constexpr (reg == 1) {
-          b0 = ubyte1(nib[j][0]);
-          b1 = ubyte1(nib[j][1]);
-        } else if constexpr (reg == 2) {
-          b0 = ubyte2(nib[j][0]);
-          b1 = ubyte2(nib[j][1]);
-        } else {
-          b0 = ubyte3(nib[j][0]);
-          b1 = ubyte3(nib[j][1]);
-        }
-        wf[par][j][reg] = pack2<T>(__builtin_fmaf(s0, b0, z0), __builtin_fmaf(s1, b1, z1));
+        if constexpr (PK16)
+          wf[par][j][reg] = pk_sub_mul_f16(pair16(qw[SB][j][t], reg_c), zv[0][reg], sv[0][reg]);
+        else
+          wf[par][j][reg] = unpack_reg(nib[j][0], nib[j][1], sv, zv, reg_c);
       };
       static_for<0, 12>([&](auto u_c) {
         constexpr int u = decltype(u_c)::value;  // slots 4 .. 15
@@ -361,15 +392,15 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
       auto dma = [&](auto idx_c) {
         if constexpr (with_vmem) load_piece(st_next, lb_c, idx_c);
       };
-      uint32_t ad[NT][2];  // [tile][0]: byte b = 4 * nibble 2b (a lane's byte address in the table); [1]: nibble 2b + 1
-      uint32_t ga[NT][8];  // code of nibble 2b in [b], of nibble 2b + 1 in [4 + b]
+      uint32_t ad[NT][2];  // byte planes of table addresses (4 * code): [tile][0] elements 0, 4, 1, 5; [1] elements 2, 6, 3, 7
+      uint32_t ga[NT][8];  // code of element 2b in [b], of element 2b + 1 in [4 + b]
       u32x4 bs[2];
       // the two gathers of fragment register `reg` of tile `j`
       auto gather2 = [&](auto j_c, auto reg_c) {
         constexpr int j = decltype(j_c)::value;
         constexpr int reg = decltype(reg_c)::value;
-        ga[j][reg] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((ad[j][0] >> (8 * reg)) & 0xffu), li);
-        ga[j][4 + reg] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((ad[j][1] >> (8 * reg)) & 0xffu), li);
+        ga[j][reg] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((ad[j][reg & 1] >> (8 * (reg >> 1))) & 0xffu), li);
+        ga[j][4 + reg] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((ad[j][reg & 1] >> (8 * ((reg >> 1) + 2))) & 0xffu), li);
       };
       auto piece = [&](auto j_c, auto reg_c) {
         constexpr int j = decltype(j_c)::value;
@@ -380,8 +411,8 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
       using J0 = std::integral_constant<int, 0>;
       using J1 = std::integral_constant<int, 1>;
       mfma_slot(0);
-      bs[0] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * 64);
-      bs[1] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * 64 + 16);
+      bs[0] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * TB_STEP);
+      bs[1] = *reinterpret_cast<const u32x4*>(lt + tb_r + t * TB_STEP + 16);
       ad[0][0] = opaque((qw[SB][0][t] << 2) & 0x3C3C3C3Cu);
       ad[0][1] = opaque((qw[SB][0][t] >> 2) & 0x3C3C3C3Cu);
       gather2(J0{}, I0{});
@@ -717,9 +748,9 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
   }
 }
 
-// qweight [K/8, N] (nibble j of word [k8, n] = q[8 k8 + j, n]) -> qweight_t [N/8, K] (nibble j of word [n8, k] =
-// q[k, 8 n8 + j]).  One thread per 8 x 8 block of nibbles: 8 adjacent words in, 8 adjacent words out.  Runs once per
-// frozen weight.
+// qweight [K/8, N] (nibble j of word [k8, n] = q[8 k8 + j, n]) -> qweight_t [N/8, K]: word [n8, k] holds q[k, 8 n8 + e]
+// with element e = 2p at nibble position p and e = 2p + 1 at position 4 + p.  One thread per 8 x 8 block of nibbles:
+// 8 adjacent words in, 8 adjacent words out.  Runs once per frozen weight.
 __global__ __launch_bounds__(256) void gptq_transpose_kernel(const uint32_t* __restrict__ qweight, int K8, int N8,
                                                              uint32_t* __restrict__ out) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -733,10 +764,10 @@ __global__ __launch_bounds__(256) void gptq_transpose_kernel(const uint32_t* __r
   in[0] = a[0]; in[1] = a[1]; in[2] = a[2]; in[3] = a[3];
   in[4] = b[0]; in[5] = b[1]; in[6] = b[2]; in[7] = b[3];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {  // output word i: row k = 8 k8 + i, nibble j from input word j (column 8 n8 + j)
+  for (int i = 0; i < 8; ++i) {  // output word i: row k = 8 k8 + i; element j comes from input word j (column 8 n8 + j)
     uint32_t w = 0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) w |= ((in[j] >> (4 * i)) & 0xFu) << (4 * j);
+    for (int j = 0; j < 8; ++j) w |= ((in[j] >> (4 * i)) & 0xFu) << (4 * ((j >> 1) + 4 * (j & 1)));
     o[i] = w;
   }
   u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)n8 * K + 8 * k8);
@@ -744,7 +775,32 @@ __global__ __launch_bounds__(256) void gptq_transpose_kernel(const uint32_t* __r
   dst[1] = u32x4{o[4], o[5], o[6], o[7]};
 }
 
+// The same re-ordering inside the words of the checkpoint layout itself (no transpose): out word [k8, n] holds
+// q[8 k8 + e, n] with element 2p at nibble position p and element 2p + 1 at position 4 + p.  Four words per thread.
+__global__ __launch_bounds__(256) void gptq_interleave_kernel(const u32x4* __restrict__ in, int64_t quads, u32x4* __restrict__ out) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= quads) return;
+  const u32x4 w = in[idx];
+  u32x4 o;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    uint32_t v = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v |= ((w[c] >> (4 * e)) & 0xFu) << (4 * ((e >> 1) + 4 * (e & 1)));
+    o[c] = v;
+  }
+  out[idx] = o;
+}
+
 }  // namespace
+
+int launch_gptq_interleave(const int32_t* qweight, int K, int N, int32_t* out, hipStream_t st) {
+  const int64_t quads = (int64_t)(K / 8) * N / 4;
+  dim3 grid((unsigned)((quads + 255) / 256)), block(256);
+  hipLaunchKernelGGL(gptq_interleave_kernel, grid, block, 0, st, (const u32x4*)qweight, quads, (u32x4*)out);
+  FMSA_CHECK_LAUNCH();
+  return FMSA_OK;
+}
 
 int launch_gptq_transpose(const int32_t* qweight, int K, int N, int32_t* out, hipStream_t st) {
   const int64_t total = (int64_t)(K / 8) * (N / 8);
@@ -754,15 +810,19 @@ int launch_gptq_transpose(const int32_t* qweight, int K, int N, int32_t* out, hi
   return FMSA_OK;
 }
 
-// every projection carries its twin, and every group holds a whole number of 64-column wave tiles
-bool bwd_dx_twin_applies(const fmsa_bwd_proj* projs, int n_proj) {
+// Which flavour of the twin kernel a call can take: 0 none (a projection without its twin, or a group that does not hold
+// whole 64-column wave tiles), 1 the fp32 scale / offset tables, 2 the packed-half unpack (fp16 activations, affine
+// weights, every projection with its fp16 offset table).
+int bwd_dx_twin_flavour(const fmsa_bwd_proj* projs, int n_proj, int act_dtype) {
+  bool fp32_tables = true, pk16 = act_dtype == FMSA_F16;
   for (int p = 0; p < n_proj; ++p) {
     const fmsa_bwd_proj& s = projs[p];
-    if (!s.qweight_t) return false;
-    if (s.w.format != FMSA_WEIGHT_CODEBOOK && !s.scale_f32) return false;
-    if (s.w.group_size % 64 != 0) return false;
+    if (!s.qweight_t || s.w.group_size % 64 != 0) return 0;
+    const bool cb = s.w.format == FMSA_WEIGHT_CODEBOOK;
+    fp32_tables = fp32_tables && (cb || (s.scale_f32 && s.nsz));
+    pk16 = pk16 && !cb && s.negzp_f16 && s.w.scales;
   }
-  return true;
+  return pk16 ? 2 : (fp32_tables ? 1 : 0);
 }
 
 int launch_gptq_lora_bwd_dx_t(const fmsa_bwd_proj* projs, int n_proj, int M, int mode, void* dX, int64_t lddx,
@@ -785,6 +845,8 @@ int launch_gptq_lora_bwd_dx_t(const fmsa_bwd_proj* projs, int n_proj, int M, int
     d.qt = s.qweight_t;
     d.sc = cb ? s.w.block_scale : s.scale_f32;
     d.nsz = cb ? nullptr : s.nsz;
+    d.sc16 = s.w.scales;
+    d.nz16 = (const uint16_t*)s.negzp_f16;
     d.code = s.w.code;
     d.dY = (const uint16_t*)s.dY;
     d.lddy = s.lddy;
@@ -805,6 +867,12 @@ int launch_gptq_lora_bwd_dx_t(const fmsa_bwd_proj* projs, int n_proj, int M, int
   a.nbk = (a.K + 255) / 256;
   dim3 grid(a.nbm * a.nbk), block(256);
   const bool codebook = projs[0].w.format == FMSA_WEIGHT_CODEBOOK;  // api.hip: all projections of a launch share the format
+  const bool pk16 = bwd_dx_twin_flavour(projs, n_proj, act_dtype) == 2;
+#define LAUNCH_PK(MD)                                                                                          \
+  do {                                                                                                         \
+    if (ntail) hipLaunchKernelGGL((gptq_lora_bwd_dx_t_kernel<f16_t, true, MD, false, true>), grid, block, 0, st, a);  \
+    else hipLaunchKernelGGL((gptq_lora_bwd_dx_t_kernel<f16_t, false, MD, false, true>), grid, block, 0, st, a);       \
+  } while (0)
 #define LAUNCH_C(TT, MD, CB)                                                                             \
   do {                                                                                                   \
     if (ntail) hipLaunchKernelGGL((gptq_lora_bwd_dx_t_kernel<TT, true, MD, CB>), grid, block, 0, st, a);  \
@@ -820,13 +888,18 @@ int launch_gptq_lora_bwd_dx_t(const fmsa_bwd_proj* projs, int n_proj, int M, int
     if (mode == FMSA_BWD_SWIGLU) LAUNCH_M(TT, FMSA_BWD_SWIGLU); \
     else LAUNCH_M(TT, FMSA_BWD_LINEAR);                         \
   } while (0)
-  if (act_dtype == FMSA_BF16)
+  if (pk16) {
+    if (mode == FMSA_BWD_SWIGLU) LAUNCH_PK(FMSA_BWD_SWIGLU);
+    else LAUNCH_PK(FMSA_BWD_LINEAR);
+  } else if (act_dtype == FMSA_BF16) {
     LAUNCH(bf16_t);
-  else
+  } else {
     LAUNCH(f16_t);
+  }
 #undef LAUNCH
 #undef LAUNCH_M
 #undef LAUNCH_C
+#undef LAUNCH_PK
   FMSA_CHECK_LAUNCH();
   return FMSA_OK;
 }

@@ -75,8 +75,13 @@ FMSA_DEVI FwdProjDev select_proj(const FwdArgs& a, int p) { return p == 0 ? a.p[
 // leave the kernel with the rotary embedding applied
 // (kernels/unsloth/rope_embedding.py:36-65 of the reference: (q1, q2) <- (q1 cos - q2 sin, q2 cos + q1 sin) on the two
 // halves of every head, on the projection output ROUNDED to the storage type, fp32 arithmetic, one more rounding).
-template <typename T, int GPS, bool KTAIL, int CODEBOOK, int ROPE = 0>
+// PK16 (fp16 activations, affine weights whose words hold their nibbles interleaved -- element 2p at position p, element
+// 2p + 1 at position 4 + p --, one scale group per stage): a fragment register is (((w >> 4p) & 0x000F000F) | 0x64006400)
+// + (-(1024 + z)) [exact] times the fp16 scale [one rounding] in packed half arithmetic: RNE_fp16(s * (q - z)) bit for bit
+// in 15 instead of 22 instructions per word.
+template <typename T, int GPS, bool KTAIL, int CODEBOOK, int ROPE = 0, bool PK16 = false>
 __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
+  static_assert(!PK16 || (std::is_same<T, f16_t>::value && CODEBOOK == 0 && GPS == 1 && ROPE == 0), "packed half unpack");
   // two separate arrays (not one 2-D array): every access names its buffer statically, which is
   // what lets the compiler see that fragment reads of one buffer do not depend on the direct loads
   // in flight into the other
@@ -219,6 +224,8 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
   uint16_t sc_raw[NBUF][NT][GPS];
   uint32_t zw_raw[NBUF][NT][GPS];  // code-book format: the fp32 block scale
   float sf[NT][GPS], sf16[NT][GPS], nsz[NT][GPS];
+  uint32_t sp16[NT], nz16[NT];  // PK16: the stage's scale and -(1024 + zero) as fp16 pairs (both halves equal)
+  const uint32_t pk_mask = opaque(0x000F000Fu), pk_bias = opaque(0x64006400u);  // in vector registers: the and-or takes no literal
   // group index of the stage being loaded, advanced without a division when GPS == 1
   int g_ld[NT], k_in_g[NT];
 #pragma unroll
@@ -288,6 +295,10 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
           // (the tables are built step by step in prefetch)
         } else if constexpr (CODEBOOK == 1) {
           sf[j][u] = __uint_as_float(zw_raw[SB][j][u]);
+        } else if constexpr (PK16) {
+          sp16[j] = (uint32_t)sc_raw[SB][j][u] * 0x00010001u;
+          const float nz = -(1024.0f + (float)((zw_raw[SB][j][u] >> zshift[j]) & 0xFu) + zoff[j]);  // exact in fp16
+          nz16[j] = pack2<f16_t>(nz, nz);
         } else {
           sf[j][u] = fp16_bits_to_f32(sc_raw[SB][j][u]);
           sf16[j][u] = sf[j][u] * 0.0625f;
@@ -342,6 +353,11 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
         wf[par][j][1] = __builtin_amdgcn_perm(o01, e01, 0x07060302u);
         wf[par][j][2] = __builtin_amdgcn_perm(o23, e23, 0x05040100u);
         wf[par][j][3] = __builtin_amdgcn_perm(o23, e23, 0x07060302u);
+      } else if constexpr (PK16) {
+        static_for<0, 4>([&](auto r_c) {
+          constexpr int r = decltype(r_c)::value;
+          wf[par][j][r] = pk_sub_mul_f16(((qw[SB][j][t] >> (4 * r)) & pk_mask) | pk_bias, nz16[j], sp16[j]);
+        });
       } else {
         wf[par][j] = dequant8<T>(qw[SB][j][t], sf[j][t * GPS / 4], sf16[j][t * GPS / 4], nsz[j][t * GPS / 4]);
       }
@@ -529,12 +545,18 @@ __global__ __launch_bounds__(256) void gptq_lora_fwd_kernel(const FwdArgs a) {
     uint32_t nib[NT][2];  // [tile][0]: nibbles 0, 2, 4, 6 in bytes 0..3; [1]: 16 * nibbles 1, 3, 5, 7 (the scale is pre-divided)
     auto masks = [&](auto j_c) {
       constexpr int j = decltype(j_c)::value;
-      nib[j][0] = opaque(qw[SB][j][t] & 0x0F0F0F0Fu);
-      nib[j][1] = opaque(qw[SB][j][t] & 0xF0F0F0F0u);
+      if constexpr (!PK16) {
+        nib[j][0] = opaque(qw[SB][j][t] & 0x0F0F0F0Fu);
+        nib[j][1] = opaque(qw[SB][j][t] & 0xF0F0F0F0u);
+      }
     };
     auto piece = [&](auto j_c, auto reg_c) {
       constexpr int j = decltype(j_c)::value;
       constexpr int reg = decltype(reg_c)::value;
+      if constexpr (PK16) {
+        wf[par][j][reg] = pk_sub_mul_f16(((qw[SB][j][t] >> (4 * reg)) & pk_mask) | pk_bias, nz16[j], sp16[j]);
+        return;
+      }
       float b0, b1;
       if constexpr (reg == 0) {
         b0 = ubyte0(nib[j][0]);
@@ -951,6 +973,9 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
   const bool ktail = (a.K % BK) != 0;
   const bool codebook = projs[0].w.format == FMSA_WEIGHT_CODEBOOK;  // api.hip: all projections of a launch share the format
   // table flavour: one code book for the launch, one block per 64-wide stage
+  // packed-half unpack: fp16 activations and interleaved words (api.hip: then every projection is affine, interleaved, with
+  // group_size % 64 == 0, and there is no rotary epilogue)
+  const bool pk16 = act_dtype == FMSA_F16 && !codebook && projs[0].w.nibble_order == 1;
   bool table = codebook && gps == 1;
   for (int p = 0; p < n_proj; ++p)
     table = table && projs[p].w.code == projs[0].w.code && (projs[p].w.group_size & (projs[p].w.group_size - 1)) == 0;
@@ -975,10 +1000,14 @@ int launch_gptq_lora_fwd(const fmsa_fwd_proj* projs, int n_proj, const void* X, 
     if (ktail) LAUNCH2(TT, true); \
     else LAUNCH2(TT, false);  \
   } while (0)
-  if (act_dtype == FMSA_BF16)
+  if (pk16) {
+    if (ktail) hipLaunchKernelGGL((gptq_lora_fwd_kernel<f16_t, 1, true, 0, 0, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((gptq_lora_fwd_kernel<f16_t, 1, false, 0, 0, true>), grid, block, 0, st, a);
+  } else if (act_dtype == FMSA_BF16) {
     LAUNCH(bf16_t);
-  else
+  } else {
     LAUNCH(f16_t);
+  }
 #undef LAUNCH
 #undef LAUNCH2
 #undef LAUNCH3

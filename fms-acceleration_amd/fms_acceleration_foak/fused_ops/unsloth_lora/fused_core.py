@@ -117,8 +117,9 @@ class _Proj:
     def from_kernel_order(self, dXp):
         return dXp if self.w.perm is None or self.input_ordered else fmsa_hip.permute_cols(dXp, self.w.perm, gather=False)
 
-    def fwd_dict(self, U):
-        return {"w": self.w.struct, "U": U, "B": self.B, "bias": self.bias, "r": self.r, "s": self.s}
+    def fwd_dict(self, U, interleaved=False):
+        return {"w": self.w.struct_interleaved if interleaved else self.w.struct, "U": U, "B": self.B, "bias": self.bias,
+                "r": self.r, "s": self.s}
 
     def bwd_dict(self, dY2, T, mask_src, permuted=None):
         """`permuted`: dict shared by the projections of one launch, so that a mask source they have in common
@@ -137,9 +138,9 @@ class _Proj:
                         if permuted is not None:
                             permuted[key] = (mask_src, pm)  # holds the source too: its id stays taken
                         mask_src = pm
-        qweight_t, scale_f32 = self.w.twin
+        qweight_t, scale_f32, negzp_f16 = self.w.twin
         return {"w": self.w.struct, "nsz": self.w.nsz, "dY": dY2, "T": T, "At": At, "mask_src": mask_src if self.r else None,
-                "r": self.r, "s": self.s, "qweight_t": qweight_t, "scale_f32": scale_f32}
+                "r": self.r, "s": self.s, "qweight_t": qweight_t, "scale_f32": scale_f32, "negzp_f16": negzp_f16}
 
     def lora_grads(self, T, Xd, U, dY2):
         """dA [r, K] = s T^T Xd and dB [N, r] = s dY^T U, in the dtypes of the parameters."""
@@ -245,6 +246,12 @@ def _rope_in_epilogue(projs, rope, dtype):
             and all(p.w.N % head_dim == 0 for i, p in enumerate(projs) if (mask >> i) & 1))
 
 
+def _interleaved(projs, dtype):
+    """Whether a forward launch over these projections reads the interleaved copies of their weights (the kernel's
+    packed-half unpack: fp16 activations, GPTQ weights with groups in whole stages; all projections or none)."""
+    return all(getattr(p.w, "interleaved_ok", lambda _: False)(dtype) for p in projs)
+
+
 def _linear_forward(projs, X2, Xds, stack=None, rope=None):
     """Y_p = X deq(W_p) + s U_p B_p^T for projections sharing X2.  One launch when the weights walk K in one
     order (on X in that order); otherwise one launch per projection on its own column-permuted copy of X.
@@ -253,13 +260,15 @@ def _linear_forward(projs, X2, Xds, stack=None, rope=None):
     Us = _lora_down_all(projs, Xds, stack)
     fused_rope = rope is not None and _rope_in_epilogue(projs, rope, X2.dtype)
     if _one_order(projs):
-        outs = fmsa_hip.gptq_lora_fwd(projs[0].to_kernel_order(X2), [p.fwd_dict(U) for p, U in zip(projs, Us)],
+        il = not fused_rope and _interleaved(projs, X2.dtype)  # the rotating flavours read the checkpoint's nibble order
+        outs = fmsa_hip.gptq_lora_fwd(projs[0].to_kernel_order(X2), [p.fwd_dict(U, il) for p, U in zip(projs, Us)],
                                       rope=rope if fused_rope else None)
     else:
         outs = []
         for i, (p, U) in enumerate(zip(projs, Us)):
             r1 = (rope[0], rope[1], rope[2], 1) if fused_rope and (rope[3] >> i) & 1 else None
-            outs.append(fmsa_hip.gptq_lora_fwd(p.to_kernel_order(X2), [p.fwd_dict(U)], rope=r1)[0])
+            il = r1 is None and _interleaved([p], X2.dtype)
+            outs.append(fmsa_hip.gptq_lora_fwd(p.to_kernel_order(X2), [p.fwd_dict(U, il)], rope=r1)[0])
     if rope is not None and not fused_rope:
         cos2d, sin2d, head_dim, mask = rope
         for i, (p, y) in enumerate(zip(projs, outs)):
@@ -411,7 +420,8 @@ def mlp_forward(ctx, X, gate, up, down, dropouts, dtype):
     fused = _one_order([gate, up])
     if fused:
         Ug, Uu = _lora_down_all([gate, up], [Xg, Xu], stack)
-        e, g, h = fmsa_hip.gptq_lora_fwd(gate.to_kernel_order(X2), [gate.fwd_dict(Ug), up.fwd_dict(Uu)], fmsa_hip.FWD_SWIGLU)
+        il = _interleaved([gate, up], X2.dtype)
+        e, g, h = fmsa_hip.gptq_lora_fwd(gate.to_kernel_order(X2), [gate.fwd_dict(Ug, il), up.fwd_dict(Uu, il)], fmsa_hip.FWD_SWIGLU)
     else:
         (e, g), (Ug, Uu) = _linear_forward([gate, up], X2, [Xg, Xu], stack)
         h = fmsa_hip.swiglu_fwd(e, g)

@@ -141,7 +141,7 @@ class Linear4bitFunction(torch.autograd.Function):
         dy2 = dy if dy.is_contiguous() else dy.contiguous()
         dx = fmsa_hip.gptq_lora_bwd_dx(
             [{"w": w.struct, "nsz": w.nsz, "dY": dy2, "T": None, "At": None, "mask_src": None, "r": 0, "s": 0.0,
-              "qweight_t": w.twin[0], "scale_f32": w.twin[1]}], dy2.shape[0], w.K)
+              "qweight_t": w.twin[0], "scale_f32": w.twin[1], "negzp_f16": w.twin[2]}], dy2.shape[0], w.K)
         return dx, None, None
 
 

@@ -41,7 +41,8 @@ class QuantLinearFunction(torch.autograd.Function):
         x2 = x if x.is_contiguous() else x.contiguous()
         if w.perm is not None:  # act-order: the repacked weight walks K in sorted-group order
             x2 = fmsa_hip.permute_cols(x2, w.perm, gather=True)
-        (y,) = fmsa_hip.gptq_lora_fwd(x2, [{"w": w.struct, "U": None, "B": None, "bias": None, "r": 0, "s": 0.0}])
+        struct = w.struct_interleaved if w.interleaved_ok(x2.dtype) else w.struct
+        (y,) = fmsa_hip.gptq_lora_fwd(x2, [{"w": struct, "U": None, "B": None, "bias": None, "r": 0, "s": 0.0}])
         return y
 
     @staticmethod
@@ -59,7 +60,7 @@ class QuantLinearFunction(torch.autograd.Function):
         dy2 = dy if dy.is_contiguous() else dy.contiguous()
         dx = fmsa_hip.gptq_lora_bwd_dx(
             [{"w": w.struct, "nsz": w.nsz, "dY": dy2, "T": None, "At": None, "mask_src": None, "r": 0, "s": 0.0,
-              "qweight_t": w.twin[0], "scale_f32": w.twin[1]}], dy2.shape[0], w.K)
+              "qweight_t": w.twin[0], "scale_f32": w.twin[1], "negzp_f16": w.twin[2]}], dy2.shape[0], w.K)
         if w.perm is not None:
             dx = fmsa_hip.permute_cols(dx, w.perm, gather=False)
         return dx, None, None, None, None, None, None, None

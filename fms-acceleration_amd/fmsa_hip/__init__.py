@@ -43,6 +43,7 @@ EXPORTED_SYMBOLS = (
     "fmsa_swiglu_bwd",
     "fmsa_gptq_make_nsz",
     "fmsa_gptq_transpose",
+    "fmsa_gptq_interleave",
     "fmsa_nf4_dequant",
     "fmsa_nf4_prepare",
     "fmsa_lora_pack",
@@ -67,7 +68,7 @@ class GptqWeight(Structure):
         ("group_size", c_int32),
         ("zero_offset", c_int32),
         ("format", c_int32),
-        ("reserved", c_int32),
+        ("nibble_order", c_int32),
         ("code", c_void_p),
         ("block_scale", c_void_p),
     ]
@@ -170,6 +171,7 @@ class BwdProj(Structure):
         ("s", c_float),
         ("qweight_t", c_void_p),
         ("scale_f32", c_void_p),
+        ("negzp_f16", c_void_p),
     ]
 
 
@@ -216,6 +218,7 @@ def lib() -> ctypes.CDLL:
     L.fmsa_swiglu_bwd.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p]
     L.fmsa_gptq_make_nsz.argtypes = [POINTER(GptqWeight), c_void_p, c_void_p]
     L.fmsa_gptq_transpose.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p]
+    L.fmsa_gptq_interleave.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p]
     L.fmsa_nf4_dequant.argtypes = [POINTER(Nf4Weight), c_int, c_void_p, c_void_p]
     L.fmsa_nf4_prepare.argtypes = [POINTER(Nf4Weight), c_void_p, c_void_p, c_void_p]
     L.fmsa_lora_pack.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -264,15 +267,16 @@ def act_enum(dtype: torch.dtype) -> int:
     return _DTYPE_ENUM[dtype]
 
 
-def make_weight(qweight, scales, qzeros, g_idx, group_size: int, zero_offset: int = 0) -> GptqWeight:
-    """GptqWeight from QuantLinear buffers.  g_idx=None declares the identity assignment."""
+def make_weight(qweight, scales, qzeros, g_idx, group_size: int, zero_offset: int = 0, nibble_order: int = 0) -> GptqWeight:
+    """GptqWeight from QuantLinear buffers.  g_idx=None declares the identity assignment.  nibble_order=1 declares
+    that qweight is gptq_interleave's output (forward entry point, fp16 activations, group_size % 64 == 0 only)."""
     K = qweight.shape[0] * 8
     N = qweight.shape[1]
     assert qweight.dtype == torch.int32 and qzeros.dtype == torch.int32 and scales.dtype == torch.float16
     assert qweight.is_contiguous() and qzeros.is_contiguous() and scales.is_contiguous()
     return GptqWeight(
         qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
-        None if g_idx is None else g_idx.data_ptr(), K, N, int(group_size), int(zero_offset), WEIGHT_AFFINE, 0, None, None,
+        None if g_idx is None else g_idx.data_ptr(), K, N, int(group_size), int(zero_offset), WEIGHT_AFFINE, int(nibble_order), None, None,
     )
 
 
@@ -465,8 +469,8 @@ def gptq_lora_fwd(x2d, projs: Sequence[dict], mode: int = FWD_LINEAR, rope=None)
 
 
 def gptq_lora_bwd_dx(projs: Sequence[dict], M: int, K: int, mode: int = BWD_LINEAR, e=None, g=None):
-    """projs: dicts with keys w, nsz, dY, T, At, mask_src, r, s and optionally qweight_t, scale_f32 (the weight's
-    transposed twin, see gptq_transpose).  LINEAR mode returns dX [M, K]; SWIGLU mode overwrites e <- d_g,
+    """projs: dicts with keys w, nsz, dY, T, At, mask_src, r, s and optionally qweight_t, scale_f32, negzp_f16 (the
+    weight's transposed twin and its tables, see gptq_transpose and gptq_negzp_f16).  LINEAR mode returns dX [M, K]; SWIGLU mode overwrites e <- d_g,
     g <- d_e and returns h."""
     arr = (BwdProj * len(projs))()
     ref = projs[0]["dY"]
@@ -478,7 +482,8 @@ def gptq_lora_bwd_dx(projs: Sequence[dict], M: int, K: int, mode: int = BWD_LINE
         assert T is None or T.stride(1) == 1
         arr[i] = BwdProj(p["w"], _ptr(p["nsz"]), _ptr(dy), dy.stride(0), _ptr(T), 0 if T is None else T.stride(0),
                          _ptr(p.get("At")) if p["r"] else None, _ptr(ms), 0 if ms is None else ms.stride(0),
-                         int(p["r"]), float(p["s"] or 0.0), _ptr(p.get("qweight_t")), _ptr(p.get("scale_f32")))
+                         int(p["r"]), float(p["s"] or 0.0), _ptr(p.get("qweight_t")), _ptr(p.get("scale_f32")),
+                         _ptr(p.get("negzp_f16")))
     if mode == BWD_SWIGLU:
         h = torch.empty_like(e)
         _check("fmsa_gptq_lora_bwd_dx",
@@ -498,8 +503,34 @@ def dx_twin_enabled() -> bool:
     return os.environ.get("FMSA_DX_TWIN", "1") != "0"
 
 
+def fwd_interleaved_enabled() -> bool:
+    """Whether prepared weights build the interleaved copy the forward kernel's packed-half unpack reads for fp16
+    activations (one more packed copy of every frozen weight, 4 bits per weight).  FMSA_FWD_INTERLEAVED=0 keeps the
+    checkpoint layout only."""
+    return os.environ.get("FMSA_FWD_INTERLEAVED", "1") != "0"
+
+
+def gptq_negzp_f16(qzeros, N: int, zero_offset: int = 0):
+    """fp16 [G, N] = -(1024 + zero point + zero_offset), exact in fp16: the offset table of the packed-half unpack
+    (fmsa_bwd_proj.negzp_f16)."""
+    shifts = torch.arange(0, 32, 4, device=qzeros.device, dtype=torch.int64)
+    z = ((qzeros.to(torch.int64).unsqueeze(-1) >> shifts) & 0xF).reshape(qzeros.shape[0], -1)[:, :N]
+    return (-(1024 + z + int(zero_offset))).to(torch.float16).contiguous()
+
+
+def gptq_interleave(qweight):
+    """The packed weight [K/8, N] with the nibbles of every word interleaved (element 2p at position p, element 2p + 1 at
+    position 4 + p): what the forward kernel's packed-half unpack reads (GptqWeight.nibble_order = 1, fp16 activations)."""
+    K8, N = qweight.shape
+    assert qweight.dtype == torch.int32 and qweight.is_contiguous() and N % 4 == 0
+    out = torch.empty_like(qweight)
+    _check("fmsa_gptq_interleave", lib().fmsa_gptq_interleave(_ptr(qweight), K8 * 8, N, _ptr(out), _stream(qweight)))
+    return out
+
+
 def gptq_transpose(qweight):
-    """The transposed twin [N/8, K] of a packed weight [K/8, N]: nibble j of word [n8, k] = q[k, 8 n8 + j]."""
+    """The transposed twin [N/8, K] of a packed weight [K/8, N]: word [n8, k] holds q[k, 8 n8 + e], element 2p at nibble
+    position p, element 2p + 1 at position 4 + p."""
     K8, N = qweight.shape
     assert qweight.dtype == torch.int32 and qweight.is_contiguous() and N % 8 == 0
     out = torch.empty((N // 8, K8 * 8), dtype=torch.int32, device=qweight.device)

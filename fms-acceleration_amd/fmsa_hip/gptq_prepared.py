@@ -17,7 +17,7 @@ class PreparedWeight:
     lets their callers see that and keep them in one launch."""
 
     __slots__ = ("struct", "K", "N", "group_size", "perm", "perm_key", "nsz", "_keep", "_zero_offset", "_columns", "col_inv", "_row_inv",
-                 "_twin")
+                 "_twin", "_interleaved")
 
     def __init__(self, qweight, scales, qzeros, g_idx, bits):
         if bits != 4:
@@ -52,6 +52,7 @@ class PreparedWeight:
     def _finish(self, qweight, scales, qzeros):
         self._keep = (qweight, scales, qzeros)
         self._twin = None
+        self._interleaved = None
         self.struct = fmsa_hip.make_weight(qweight, scales, qzeros, None, self.group_size, self._zero_offset)
         # -scale * zero per (group, column), fp32: read by the input-gradient kernel (frozen weight,
         # so it is built once)
@@ -59,17 +60,34 @@ class PreparedWeight:
 
     @property
     def twin(self):
-        """(qweight_t int32 [N/8, K], scale_f32 [G, N]) for the input-gradient kernel, built on first use (the weight
-        is frozen): the nibbles packed along N, so that a lane's word is its MFMA fragment as in the forward kernel,
-        and the scales widened once.  (None, None) when switched off or when a group does not hold whole 64-column
-        wave tiles (the kernel then reads the checkpoint layout)."""
+        """(qweight_t int32 [N/8, K], scale_f32 [G, N], negzp_f16 [G, N]) for the input-gradient kernel, built on first
+        use (the weight is frozen): the nibbles packed along N, so that a lane's word is its MFMA fragment as in the
+        forward kernel, the scales widened once, and the fp16 offsets of the packed-half unpack (fp16 activations).
+        (None, None, None) when switched off or when a group does not hold whole 64-column wave tiles (the kernel then
+        reads the checkpoint layout)."""
         if self._twin is None:
             if fmsa_hip.dx_twin_enabled() and self.group_size % 64 == 0:
-                qweight, scales, _ = self._keep
-                self._twin = (fmsa_hip.gptq_transpose(qweight), scales.to(torch.float32).contiguous())
+                qweight, scales, qzeros = self._keep
+                self._twin = (fmsa_hip.gptq_transpose(qweight), scales.to(torch.float32).contiguous(),
+                              fmsa_hip.gptq_negzp_f16(qzeros, self.N, self._zero_offset))
             else:
-                self._twin = (None, None)
+                self._twin = (None, None, None)
         return self._twin
+
+    def interleaved_ok(self, dtype) -> bool:
+        """Whether the forward kernel's packed-half unpack applies: fp16 activations, groups in whole 64-row stages."""
+        return dtype == torch.float16 and self.group_size % 64 == 0 and fmsa_hip.fwd_interleaved_enabled()
+
+    @property
+    def struct_interleaved(self):
+        """The C-ABI view of a copy of the packed weight whose words hold their nibbles interleaved (nibble_order 1),
+        built on first use: the forward kernel unpacks it with packed-half arithmetic (fp16 activations only)."""
+        if self._interleaved is None:
+            qweight, scales, qzeros = self._keep
+            q_il = fmsa_hip.gptq_interleave(qweight)
+            struct = fmsa_hip.make_weight(q_il, scales, qzeros, None, self.group_size, self._zero_offset, nibble_order=1)
+            self._interleaved = (struct, q_il)
+        return self._interleaved[0]
 
     @property
     def row_inv(self):

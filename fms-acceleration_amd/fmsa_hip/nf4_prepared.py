@@ -80,13 +80,13 @@ class PreparedNf4Weight:
 
 
 def _twin(self):
-    """(qweight_t int32 [N/8, K], None): the codes packed along N for the input-gradient kernel, built on first use
+    """(qweight_t int32 [N/8, K], None, None): the codes packed along N for the input-gradient kernel, built on first use
     (see gptq_prepared.PreparedWeight.twin; the block scales are fp32 already)."""
     if self._twin is None:
         if fmsa_hip.dx_twin_enabled() and self.group_size % 64 == 0:
-            self._twin = (fmsa_hip.gptq_transpose(self._keep[0]), None)
+            self._twin = (fmsa_hip.gptq_transpose(self._keep[0]), None, None)
         else:
-            self._twin = (None, None)
+            self._twin = (None, None, None)
     return self._twin
 
 

@@ -75,10 +75,18 @@ typedef struct fmsa_gptq_weight {
   int32_t group_size; /* > 0; G = ceil(K / group_size)                           */
   int32_t zero_offset;
   int32_t format;     /* enum fmsa_weight_format                                  */
-  int32_t reserved;   /* 0                                                        */
+  int32_t nibble_order; /* 0: the checkpoint's (nibble j = row 8*k8 + j).  1: interleaved, element 2p at nibble position
+                         * p and element 2p + 1 at position 4 + p (see fmsa_gptq_interleave): accepted by fmsa_gptq_lora_fwd
+                         * only, for the affine format with FMSA_F16 activations and group_size % 64 == 0 */
   const float* code;        /* CODEBOOK: 16 entries                               */
   const float* block_scale; /* CODEBOOK: [K / group_size, N]                      */
 } fmsa_gptq_weight;
+
+/* One-time re-ordering of the nibbles inside every word of qweight int32 [K/8, N] for the forward kernel's packed-half
+ * unpack (FMSA_F16 activations): out word [k8, n] holds q[8*k8 + e, n] with element 2p at nibble position p and element
+ * 2p + 1 at position 4 + p, so that (w >> 4p) & 0x000F000F is the pair (k, k+1) of MFMA fragment register p.  Hand the
+ * result to fmsa_gptq_lora_fwd as `qweight` with nibble_order = 1; everything else of the weight is unchanged. */
+int fmsa_gptq_interleave(const int32_t* qweight, int K, int N, int32_t* qweight_out, void* stream);
 
 /* Replaces dequant248 (UL/gptq/triton/kernels.py:125-153): materialises W[K, N] row-major in
  * `out_dtype` (FMSA_F16 = the reference's output type, FMSA_BF16, FMSA_F32) with one
@@ -272,9 +280,14 @@ typedef struct fmsa_bwd_proj {
    * scale_f32 [G, N].  When every projection of a call carries them (and every group_size % 64 == 0) the kernel
    * reads the twin: a lane's word is then its MFMA fragment, as in the forward kernel, instead of an 8 x 8 block of
    * nibbles that has to be transposed with byte shuffles.  Same values, same contraction order: bit-identical
-   * results.  NULL: the checkpoint layout in `w` is read. */
+   * results.  NULL: the checkpoint layout in `w` is read.
+   * negzp_f16 (affine format, FMSA_F16 activations only; optional): fp16 [G, N] = -(1024 + z + zero_offset), exact in
+   * fp16.  With it the twin is unpacked in packed half arithmetic, (1024 + q) - (1024 + z) exactly and one rounding in
+   * the product with the fp16 scale, i.e. RNE_fp16(scale * (q - z)) bit for bit at two thirds of the instructions;
+   * scale_f32 and nsz may then be NULL. */
   const int32_t* qweight_t;
   const float* scale_f32;
+  const void* negzp_f16;
 } fmsa_bwd_proj;
 
 enum fmsa_bwd_mode { FMSA_BWD_LINEAR = 0, FMSA_BWD_SWIGLU = 1 };
@@ -284,8 +297,10 @@ enum fmsa_bwd_mode { FMSA_BWD_LINEAR = 0, FMSA_BWD_SWIGLU = 1 };
  * caller builds it once per weight. */
 int fmsa_gptq_make_nsz(const fmsa_gptq_weight* w /*host*/, float* out, void* stream);
 
-/* The transposed twin of a packed weight for fmsa_bwd_proj.qweight_t: out int32 [N/8, K], nibble j of word
- * [n8, k] = q[k, 8*n8 + j], from qweight int32 [K/8, N] (pack() of qlinear_tritonv2.py:132-147 packs along K).
+/* The transposed twin of a packed weight for fmsa_bwd_proj.qweight_t: out int32 [N/8, K] from qweight int32 [K/8, N]
+ * (pack() of qlinear_tritonv2.py:132-147 packs along K).  Word [n8, k] holds q[k, 8*n8 + e] for e = 0..7 with the even
+ * elements in its low half and the odd ones in its high half: element 2p at nibble position p, element 2p + 1 at
+ * position 4 + p (a layout private to the kernel: (w >> 4p) & 0x000F000F is the pair of fragment register p).
  * For an act-order weight pass the row-repacked qweight (fmsa_gptq_permute_rows).  K % 8 == 0, N % 8 == 0. */
 int fmsa_gptq_transpose(const int32_t* qweight, int K, int N, int32_t* qweight_t_out, void* stream);
 

@@ -44,13 +44,13 @@ def test_probe_is_a_library_of_its_own():
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(fmsa_hip.GptqWeight) == 72
     assert ctypes.sizeof(fmsa_hip.FwdProj) == 128
-    assert ctypes.sizeof(fmsa_hip.BwdProj) == 160
+    assert ctypes.sizeof(fmsa_hip.BwdProj) == 168
     assert ctypes.sizeof(fmsa_hip.LoraGradJob) == 88
     assert ctypes.sizeof(fmsa_hip.LoraPackJob) == 64
 
 
-def _w(K=64, N=64, gs=64, q=0x1000, s=0x2000, z=0x3000, g=None, zo=0):
-    return fmsa_hip.GptqWeight(q, s, z, g, K, N, gs, zo, fmsa_hip.WEIGHT_AFFINE, 0, None, None)
+def _w(K=64, N=64, gs=64, q=0x1000, s=0x2000, z=0x3000, g=None, zo=0, order=0):
+    return fmsa_hip.GptqWeight(q, s, z, g, K, N, gs, zo, fmsa_hip.WEIGHT_AFFINE, order, None, None)
 
 
 def _cb(K=64, N=64, gs=64, q=0x1000, code=0x7000, bs=0x8000, g=None, fmt=None):
@@ -124,6 +124,17 @@ def test_fused_forward_validation():
     assert call(proj(ldy=32)) == -2
     assert call(proj(), n=1, mode=1) == -2                # SwiGLU needs exactly gate + up
     assert call(proj(), n=2, mode=1, H=None) == -1
+    # interleaved words (fmsa_gptq_interleave's output): fp16 activations, whole 64-row stages per group, nothing else
+    assert call(proj(w=_w(order=2))) == -2
+    assert call(proj(w=_w(order=1)), dt=1) == -5          # bf16 unpacks the checkpoint's order only
+    assert call(proj(w=_w(order=1, gs=32)), dt=0) == -5
+    assert lib.fmsa_gptq_dequant(ctypes.byref(_w(order=1)), 0, 0x1000, None) == -5   # the forward entry point only
+    il = lib.fmsa_gptq_interleave
+    assert il(None, 64, 64, 0x2000, None) == -1
+    assert il(0x1000, 64, 64, None, None) == -1
+    assert il(0x1000, 60, 64, 0x2000, None) == -2
+    assert il(0x1000, 64, 66, 0x2000, None) == -2
+    assert il(0x1004, 64, 64, 0x2000, None) == -3
 
     # the flavour that rotates Q / K in its epilogue: the same checks, plus those of the tables and of the head size
     fr = lib.fmsa_gptq_lora_fwd_rope
@@ -155,6 +166,7 @@ def test_fused_forward_validation():
     assert rcall(proj(), rope(), ldx=32) == -2             # the plain forward's checks still apply
     assert rcall(proj(w=_w(N=96), ldy=96), rope()) == -2   # N is not whole heads
     assert rcall(proj(w=_w(gs=32)), rope()) == -5          # group sizes below the 64-wide K stage
+    assert rcall(proj(w=_w(order=1)), rope(dtype=0), dt=0) == -5   # the rotating flavours read the checkpoint's nibble order
 
 
 def test_bwd_and_skinny_validation():

@@ -15,13 +15,18 @@ def dev(t):
     return t.cuda()
 
 
-def gweight(w, identity=True):
+def gweight(w, identity=True, interleaved=False):
     import fmsa_hip
 
     t = w.get("dev")  # the C struct holds raw pointers: one device copy per weight, kept alive by the dict
     if t is None:
         t = {k: dev(v) for k, v in w["t"].items()}
         w["dev"] = t
+    if interleaved:  # the forward kernel's packed-half unpack (fp16 activations) reads this copy
+        if "qweight_il" not in t:
+            t["qweight_il"] = fmsa_hip.gptq_interleave(t["qweight"])
+        return fmsa_hip.make_weight(t["qweight_il"], t["scales"], t["qzeros"], None, w["group_size"], w["zero_offset"],
+                                    nibble_order=1)
     return fmsa_hip.make_weight(t["qweight"], t["scales"], t["qzeros"], None if identity else t["g_idx"],
                                 w["group_size"], w["zero_offset"])
 
@@ -272,12 +277,16 @@ def test_fwd_linear(M, K, N, gs, r, bias, dtype):
     (y,) = fmsa_hip.gptq_lora_fwd(xd, [p])
     err = olora.max_rel_err(y.cpu(), ref)
     assert err < TOL, err
+    if dtype == torch.float16 and gs % 64 == 0:
+        # the packed-half unpack of the interleaved copy forms the same fp16 weights: identical products, bit for bit
+        (y_il,) = fmsa_hip.gptq_lora_fwd(xd, [{**p, "w": gweight(w, interleaved=True)}])
+        assert torch.equal(y_il, y)
 
 
-def _proj_fwd(w, x_dev, A, B, s, dtype):
+def _proj_fwd(w, x_dev, A, B, s, dtype, interleaved=False):
     import fmsa_hip
 
-    p = {"w": gweight(w), "r": A.shape[0], "s": s, "bias": None}
+    p = {"w": gweight(w, interleaved=interleaved), "r": A.shape[0], "s": s, "bias": None}
     p["U"] = fmsa_hip.lora_down(x_dev, dev(A.to(dtype)))
     p["B"] = dev(B.to(dtype))
     return p
@@ -299,6 +308,16 @@ def test_fwd_qkv_shared_input(dtype):
     for w, (A, B), y in zip(ws, ABs, outs):
         ref = olora.lora_linear(x.float(), w["dense"], A.to(dtype).float(), B.to(dtype).float(), s)
         assert olora.max_rel_err(y.cpu(), ref) < TOL
+    if dtype == torch.float16:
+        outs_il = fmsa_hip.gptq_lora_fwd(xd, [_proj_fwd(w, xd, A, B, s, dtype, True) for w, (A, B) in zip(ws, ABs)])
+        assert all(torch.equal(a, b) for a, b in zip(outs_il, outs))
+        # one nibble order per launch
+        mixed = [_proj_fwd(w, xd, A, B, s, dtype, i == 1) for i, (w, (A, B)) in enumerate(zip(ws, ABs))]
+        with pytest.raises(fmsa_hip.FmsaError):
+            fmsa_hip.gptq_lora_fwd(xd, mixed)
+    else:
+        with pytest.raises(fmsa_hip.FmsaError):  # the interleaved copy is for fp16 activations only
+            fmsa_hip.gptq_lora_fwd(xd, [_proj_fwd(w, xd, A, B, s, dtype, True) for w, (A, B) in zip(ws, ABs)])
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -321,6 +340,10 @@ def test_fwd_swiglu(M, H, I, dtype):
     h_ref = olora.swiglu_fwd(e.cpu(), g.cpu())
     assert olora.max_rel_err(h.cpu(), h_ref.float()) < 4e-3
     assert olora.max_rel_err(h.cpu(), torch.nn.functional.silu(e_ref) * g_ref) < TOL
+    if dtype == torch.float16:
+        il = fmsa_hip.gptq_lora_fwd(xd, [_proj_fwd(wg, xd, Ag, Bg, s, dtype, True), _proj_fwd(wu, xd, Au, Bu, s, dtype, True)],
+                                    fmsa_hip.FWD_SWIGLU)
+        assert all(torch.equal(a, b) for a, b in zip(il, (e, g, h)))
 
 
 def _twin(w):
@@ -329,8 +352,9 @@ def _twin(w):
     import fmsa_hip
 
     if w["group_size"] % 64 != 0:
-        return {"qweight_t": None, "scale_f32": None}
-    return {"qweight_t": fmsa_hip.gptq_transpose(w["dev"]["qweight"]), "scale_f32": w["dev"]["scales"].float().contiguous()}
+        return {"qweight_t": None, "scale_f32": None, "negzp_f16": None}
+    return {"qweight_t": fmsa_hip.gptq_transpose(w["dev"]["qweight"]), "scale_f32": w["dev"]["scales"].float().contiguous(),
+            "negzp_f16": fmsa_hip.gptq_negzp_f16(w["dev"]["qzeros"], w["N"], w["zero_offset"])}
 
 
 def _proj_bwd(w, dy_dev, A, B, s, dtype, mask_src=None, twin=False):
@@ -482,9 +506,26 @@ def test_bwd_swiglu(M, H, I, dtype, twin):
 
 
 @pytest.mark.parametrize("K,N", [(32, 32), (256, 96), (1056, 1024)])
+def test_gptq_interleave_bit_exact(K, N):
+    """Word [k8, n] of the interleaved copy holds q[8 k8 + e, n], element 2p at nibble position p and 2p + 1 at 4 + p."""
+    import numpy as np
+
+    import fmsa_hip
+
+    w = make_gptq(K, N, 32, seed=K + 5 * N)
+    q = ogptq.unpack_rows(w["np"]["qweight"]).astype(np.uint32)  # [K, N]
+    want = np.zeros((K // 8, N), dtype=np.uint32)
+    for j in range(8):
+        want |= q[j::8, :] << np.uint32(4 * (j // 2 + 4 * (j % 2)))
+    got = fmsa_hip.gptq_interleave(dev(w["t"]["qweight"])).cpu().numpy().view(np.uint32)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("K,N", [(32, 32), (256, 96), (1056, 1024)])
 def test_gptq_transpose_bit_exact(K, N):
-    """The twin's packing: nibble j of word [n8, k] = q[k, 8 n8 + j], against a plain numpy re-packing of the
-    unpacked 4-bit values (the unpack is the oracle's, which the layout tests pin bit by bit)."""
+    """The twin's packing: word [n8, k] holds q[k, 8 n8 + e], element 2p at nibble position p and 2p + 1 at 4 + p,
+    against a plain numpy re-packing of the unpacked 4-bit values (the unpack is the oracle's, which the layout tests
+    pin bit by bit)."""
     import numpy as np
 
     import fmsa_hip
@@ -492,7 +533,7 @@ def test_gptq_transpose_bit_exact(K, N):
     w = make_gptq(K, N, 32, seed=K + 3 * N)
     q = ogptq.unpack_rows(w["np"]["qweight"]).astype(np.uint32)  # [K, N]
     want = np.zeros((N // 8, K), dtype=np.uint32)
-    for j in range(8):
-        want |= q[:, j::8].T << np.uint32(4 * j)
+    for j in range(8):  # element j of a word: even elements fill the low half-word, odd ones the high half
+        want |= q[:, j::8].T << np.uint32(4 * (j // 2 + 4 * (j % 2)))
     got = fmsa_hip.gptq_transpose(dev(w["t"]["qweight"])).cpu().numpy().view(np.uint32)
     assert np.array_equal(got, want)
