@@ -346,6 +346,43 @@ def test_fwd_swiglu(M, H, I, dtype):
         assert all(torch.equal(a, b) for a, b in zip(il, (e, g, h)))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("scale_mul", [1.0, 2.0 ** -12, 2.0 ** 11])
+@pytest.mark.parametrize("v1", [False, True])
+def test_gemm_operands_are_the_dequantised_weight_bit_for_bit(dtype, scale_mul, v1):
+    """One-hot activations read the MFMA operand the kernels form straight back: with X = I the forward's output is
+    deq(W), with dY = I the input gradient is deq(W)^T, each entry one exact product, so both must equal the oracle's
+    dequantised weight (one rounding of the exact product to the activation type) bit for bit -- on the checkpoint
+    layout, on the transposed twin, and for fp16 through the packed-half routes (interleaved copy, negzp_f16 table).
+    Scales 2^-12 smaller put many products among fp16's subnormals, 2^11 larger near the top of its range."""
+    import numpy as np
+
+    import fmsa_hip
+
+    K, N, gs = 256, 512, 64
+    w = make_gptq(K, N, gs, seed=17, v1=v1)
+    w["np"]["scales"] = (w["np"]["scales"].astype(np.float32) * scale_mul).astype(np.float16)
+    assert np.isfinite(w["np"]["scales"]).all() and (w["np"]["scales"] != 0).all()
+    w["t"]["scales"] = torch.from_numpy(w["np"]["scales"].copy())
+    name = {torch.bfloat16: "bf16", torch.float16: "fp16"}[dtype]
+    want = ogptq.dequant(w["np"]["qweight"], w["np"]["scales"], w["np"]["qzeros"], w["np"]["g_idx"],
+                         zero_offset=w["zero_offset"], out=name)
+    if dtype == torch.float16 and scale_mul < 1:
+        assert (want.float().abs() < 2.0 ** -14).float().mean() > 0.2   # the case does reach the subnormals
+    eye_k, eye_n = dev(torch.eye(K, dtype=dtype)), dev(torch.eye(N, dtype=dtype))
+    base = {"r": 0, "s": 0.0, "bias": None}
+    routes = [False] + ([True] if dtype == torch.float16 else [])
+    for interleaved in routes:
+        (y,) = fmsa_hip.gptq_lora_fwd(eye_k, [{**base, "w": gweight(w, interleaved=interleaved)}])
+        assert torch.equal(y.cpu(), want), ("forward", interleaved)
+    gw = gweight(w)
+    pb = {"w": gw, "nsz": fmsa_hip.gptq_make_nsz(gw, eye_n.device), "r": 0, "s": 0.0, "dY": eye_n, "mask_src": None}
+    twin = _twin(w)
+    for extra in ({}, {**twin, "negzp_f16": None}, twin):
+        dx = fmsa_hip.gptq_lora_bwd_dx([{**pb, **extra}], N, K)
+        assert torch.equal(dx.cpu(), want.t()), ("input gradient", sorted(k for k, v in extra.items() if v is not None))
+
+
 def _twin(w):
     """The weight's transposed twin for the input-gradient kernel (packed along N, fp32 scales); None, None when a
     group does not hold whole 64-column tiles (the kernel then reads the checkpoint layout)."""

@@ -185,6 +185,33 @@ def test_nf4_prepare_bit_exact(N, K, blocksize, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("blocksize", [32, 64, 128])
+def test_gemm_operands_are_the_dequantised_weight_bit_for_bit(blocksize, dtype):
+    """One-hot activations read the MFMA operand straight back: with X = I the forward returns deq(W), with dY = I the
+    input gradient returns deq(W)^T, every entry one exact product, so each must equal the oracle's dequantised weight
+    rounded once to the activation type, bit for bit: the forward flavour that keeps rounded products as byte planes
+    (one block per 64-wide stage, one code book), the one that gathers code values and multiplies (two code-book
+    tensors in the launch, or smaller blocks), and the input gradient on both weight layouts."""
+    import fmsa_hip
+
+    K, N = 256, 512
+    w, keep, q = _prepared(N, K, 11 + blocksize, blocksize)
+    want = onf4.dequant(q, _NAME[dtype]).t().contiguous()  # [K, N]
+    eye_k, eye_n = torch.eye(K, dtype=dtype, device="cuda"), torch.eye(N, dtype=dtype, device="cuda")
+    proj = {"w": w, "U": None, "B": None, "bias": None, "r": 0, "s": 0.0}
+    (y,) = fmsa_hip.gptq_lora_fwd(eye_k, [proj])
+    assert torch.equal(y.cpu(), want)
+    code_twin = keep[2].clone()
+    y_a, y_b = fmsa_hip.gptq_lora_fwd(eye_k, [proj, dict(proj, w=fmsa_hip.make_codebook_weight(keep[0], code_twin, keep[1], blocksize))])
+    assert torch.equal(y_a.cpu(), want) and torch.equal(y_b.cpu(), want)
+    pb = {"w": w, "nsz": None, "dY": eye_n, "T": None, "At": None, "mask_src": None, "r": 0, "s": 0.0}
+    layouts = [{}] + ([{"qweight_t": fmsa_hip.gptq_transpose(keep[0])}] if blocksize % 64 == 0 else [])
+    for extra in layouts:
+        dx = fmsa_hip.gptq_lora_bwd_dx([{**pb, **extra}], N, K)
+        assert torch.equal(dx.cpu(), want.t()), sorted(extra)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,K,N,r,blocksize", [(200, 256, 96, 16, 64), (512, 1024, 512, 8, 64), (64, 1056, 288, 32, 32), (300, 512, 256, 16, 128),
                                                (1, 64, 32, 8, 64), (257, 1344, 608, 24, 64), (31, 96, 1184, 40, 32), (513, 640, 160, 8, 128),
                                                (100, 1152, 896, 16, 64), (7, 2048, 96, 64, 64)])
