@@ -84,6 +84,13 @@ def traffic_from_profile(label):
         print(f"bench.py: {os.path.basename(TRAFFIC_PROFILE)} was taken with other GEMM sources than the tree holds; "
               "roofline.traffic is left out until the counters are collected again", file=sys.stderr)
         return None, "counter summary is older than the kernel sources"
+    algorithmic = ALGORITHMIC_BYTES.get(label)
+    if algorithmic and not 0.5 * algorithmic <= value <= 32 * algorithmic:
+        # fewer bytes than the operands hold, or more than any re-read pattern of this tiling produces: the counters
+        # were scaled by the wrong calibration dispatch
+        print(f"bench.py: {os.path.basename(TRAFFIC_PROFILE)} reads {value:.3g} bytes for {label}, implausible against "
+              f"{algorithmic:.3g} algorithmic bytes; roofline.traffic is left out", file=sys.stderr)
+        return None, "counter summary is implausible (calibration)"
     return value, os.path.relpath(TRAFFIC_PROFILE, ROOT)
 
 

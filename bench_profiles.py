@@ -241,7 +241,9 @@ def summarize():
             n = r["Kernel_Name"]
             if is_gemm(n):
                 out[int(r["Dispatch_Id"])] = (short(n), wgs(r), float(r["Counter_Value"]))
-            elif "copyBuffer" in n:
+            elif "copyBuffer" in n and int(r["Grid_Size"]) > out.get("copy", ("", 0, 0.0))[1]:
+                # the 1 GiB calibration copy is the largest copy of the run (the step's own small copies, e.g. the
+                # one-time tables of a prepared weight, come after it)
                 out["copy"] = ("copyBuffer", int(r["Grid_Size"]), float(r["Counter_Value"]))
         return out
     fe, wr = load("fetch_layer", "FETCH_SIZE"), load("write_layer", "WRITE_SIZE")
