@@ -183,6 +183,23 @@ def test_config3_llama3_8b_qkvo():
     _check_split_sum(fo, [lin], x, [dO], g)
 
 
+@pytest.fixture
+def float16(monkeypatch):
+    """The reference's own arithmetic for this path (fp16 dequantisation output, fp16 benchmark runs): the same
+    cases with fp16 activations, which take the packed-half unpack kernels."""
+    import sys
+
+    monkeypatch.setattr(sys.modules[__name__], "DT", torch.float16)
+
+
+def test_config2_llama3_8b_mlp_float16(float16):
+    _mlp_case(_gptq_lora, 8192, 4096, 14336, 16, 16.0)
+
+
+def test_config3_llama3_8b_qkvo_float16(float16):
+    test_config3_llama3_8b_qkvo()
+
+
 def test_no_worse_than_materialised_decomposition():
     """The fused kernels' error against the fp32 oracle is no worse than that of the decomposition
     the reference runs (dense weight rounded to the activation dtype, library matmul, separate LoRA
