@@ -582,9 +582,10 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
   };
   // LoRA operands of the first 16 ranks of every projection: the A^T fragments of the lane's two columns are the same
   // for all token tiles (loaded once), the T fragments of the two token tiles of a pass are fetched one pass ahead.
-  u32x4 af0[3][NT], tf0[3][2];
-  bool lora_live[3];
-  static_for<0, 3>([&](auto p_c) {
+  constexpr int NP = swiglu ? 1 : 3;  // the SwiGLU-backward launch has one projection (the entry point checks)
+  u32x4 af0[NP][NT], tf0[NP][2];
+  bool lora_live[NP];
+  static_for<0, NP>([&](auto p_c) {
     constexpr int p = decltype(p_c)::value;
     const BwdTProjDev& P = a.p[p];
     lora_live[p] = p < a.n_proj && P.r > 0;
@@ -596,7 +597,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
     }
   });
   auto load_tf = [&](int q) {
-    static_for<0, 3>([&](auto p_c) {
+    static_for<0, NP>([&](auto p_c) {
       constexpr int p = decltype(p_c)::value;
       const BwdTProjDev& P = a.p[p];
 #pragma unroll
@@ -622,7 +623,7 @@ __global__ __launch_bounds__(256) void gptq_lora_bwd_dx_t_kernel(const BwdTArgs 
         for (int j = 0; j < NT; ++j)
 #pragma unroll
           for (int i = 0; i < 16; ++i) lora[j][i] = 0.f;
-        static_for<0, 3>([&](auto p_c) {
+        static_for<0, NP>([&](auto p_c) {
           constexpr int p = decltype(p_c)::value;
           if (lora_live[p]) {
             const BwdTProjDev& P = a.p[p];
