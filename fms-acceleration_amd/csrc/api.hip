@@ -125,7 +125,7 @@ const char* fmsa_strerror(int code) {
   }
 }
 
-int fmsa_abi_version(void) { return 8; }
+int fmsa_abi_version(void) { return 9; }
 
 int fmsa_gptq_dequant(const fmsa_gptq_weight* w, int out_dtype, void* out, void* stream) {
   if (!w || !out) return FMSA_ERR_NULL;

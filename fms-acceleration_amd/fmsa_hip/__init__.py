@@ -178,6 +178,9 @@ class BwdProj(Structure):
 _lib = None
 
 
+ABI_VERSION = 9  # include/fmsa.h as this binding mirrors it (fmsa_abi_version of the library must agree)
+
+
 def lib() -> ctypes.CDLL:
     """The loaded library; raises if it has not been built."""
     global _lib
@@ -192,6 +195,10 @@ def lib() -> ctypes.CDLL:
     L.fmsa_strerror.restype = ctypes.c_char_p
     L.fmsa_strerror.argtypes = [c_int]
     L.fmsa_abi_version.restype = c_int
+    if L.fmsa_abi_version() != ABI_VERSION:
+        # struct layouts and signatures below are those of ABI_VERSION: a library of another version would read them wrong
+        raise RuntimeError(f"{LIB_PATH} has ABI version {L.fmsa_abi_version()}, this binding is written for {ABI_VERSION}: "
+                           "rebuild it with `python fms-acceleration_amd/build_hip.py`")
     L.fmsa_gptq_dequant.argtypes = [POINTER(GptqWeight), c_int, c_void_p, c_void_p]
     L.fmsa_gptq_permute_rows.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]
     L.fmsa_permute_cols.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int64, c_void_p]

@@ -43,7 +43,8 @@ enum fmsa_dtype { FMSA_F16 = 0, FMSA_BF16 = 1, FMSA_F32 = 2 };
 /* Human-readable text for an error code (host pointer to a static string). */
 const char* fmsa_strerror(int code);
 
-/* ABI version; bumped on any signature change. */
+/* ABI version; bumped on any change of a signature or struct layout (9 here).  A binding should refuse a library whose
+ * version is not the one it was written for. */
 int fmsa_abi_version(void);
 
 /* ------------------------------------------------------------------------------------------

@@ -23,7 +23,7 @@ def test_header_and_library_agree():
     lib = fmsa_hip.lib()
     for n in names:
         assert getattr(lib, n) is not None
-    assert lib.fmsa_abi_version() >= 1
+    assert lib.fmsa_abi_version() == fmsa_hip.ABI_VERSION  # the binding refuses a library of another version
     assert lib.fmsa_strerror(0) == b"ok" and b"NULL" in lib.fmsa_strerror(-1)
 
 
