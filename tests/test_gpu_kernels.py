@@ -468,6 +468,9 @@ def test_fwd_and_bwd_random_shapes(M, K, N, gs, r, bias, dtype):
     (y,) = fmsa_hip.gptq_lora_fwd(xd, [p])
     ref = olora.lora_linear(x.float(), w["dense"], Aq, Bq, s, None if b is None else b.float())
     assert olora.max_rel_err(y.cpu(), ref) < TOL
+    if dtype == torch.float16 and gs % 64 == 0:  # the packed-half unpack of the interleaved copy: the same bits
+        (y_il,) = fmsa_hip.gptq_lora_fwd(xd, [{**p, "w": gweight(w, interleaved=True)}])
+        assert torch.equal(y_il, y)
     dy = randn((M, N), 3, dtype)
     dyd = dev(dy)
     if r:
